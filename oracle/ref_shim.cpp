@@ -1,0 +1,156 @@
+// TEST INFRASTRUCTURE ONLY. Flat C entry points over the reference's own x86 AVX-512-VNNI
+// objects, compiled where they lie under /root/reference by oracle/Makefile into
+// oracle/_ref/libboltref.so. Used (a) to write the golden vectors under tests/golden/ and
+// to pin oracle/oracle.c against the real reference, and (b) as the "reference" CPU
+// baseline in bench.py when the host CPU has avx512_vnni. Nothing in the product path may
+// load this file's output.
+//
+// Each wrapper builds the TensorDesc arguments exactly as the reference's own unit tests do
+// (compute/blas_enhance/tests/test_mmm.cpp:30-90, test_mvm.cpp:30-90) and forwards to the
+// public function; no arithmetic happens here.
+#include <cstdint>
+#include <cstring>
+#include "blas_enhance.h"
+#include "tensor_desc.h"
+#include "parameter_spec.h"
+#include "cpu/x86/int8/tensor_computing_int8.h"
+
+// internal (non-public) reference prototypes, compute/tensor/src/cpu/x86/tensor_computing_x86.h
+EE quantize_x86(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *qData, F32 *scale, int mode);
+EE dequantize_x86(TensorDesc qDesc, void *qData, const F32 *scale, TensorDesc bDesc, void *bData,
+    TensorDesc dDesc, void *dData);
+EE quantize_bias_offsetC(const void *bias, TensorDesc biasDesc, DataType qType, const void *filter,
+    TensorDesc filterDesc, const F32 *scale, void *offsetCBias);
+EE requantize_cpu(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDesc outputDesc,
+    INT8 *output, F32 outputScale, Arch arch);
+
+extern int OMP_NUM_THREADS;
+
+// bfmt: 0 = DF_NORMAL [K,N], 1 = DF_TRANSPOSE [N,K], 2 = packed DF_NKNxKx (logical [K,N])
+static TensorDesc rhs_desc(int bfmt, U32 K, U32 N)
+{
+    if (bfmt == 0) {
+        return tensor2df(DT_I8, DF_NORMAL, K, N);
+    }
+    if (bfmt == 1) {
+        return tensor2df(DT_I8, DF_TRANSPOSE, N, K);
+    }
+    return tensor2df(DT_I8, DF_NKNxKx, K, N);
+}
+
+// wfmt: 0 = DF_NORMAL [N,K], 1 = DF_TRANSPOSE [K,N], 2 = packed DF_NKN32K4 (logical [N,K])
+static TensorDesc mvm_desc(int wfmt, U32 N, U32 K, DataType dt)
+{
+    if (wfmt == 0) {
+        return tensor2df(dt, DF_NORMAL, N, K);
+    }
+    if (wfmt == 1) {
+        return tensor2df(dt, DF_TRANSPOSE, K, N);
+    }
+    return tensor2df(dt, matrix_vector_multiply_weight_format(dt), N, K);
+}
+
+extern "C" {
+
+void ref_set_threads(int n)
+{
+    OMP_NUM_THREADS = n;
+}
+
+int ref_mmm_transform_rhs_bytes(int bfmt, U32 K, U32 N, U32 *bytes, U32 *rhsBytes)
+{
+    return matrix_matrix_multiply_transform_rhs_bytes(rhs_desc(bfmt, K, N), bytes, rhsBytes, X86_AVX512);
+}
+
+// out_desc: {df, nDims, dims[0], dims[1]} of the transformed descriptor
+int ref_mmm_transform_rhs(int bfmt, U32 K, U32 N, const void *src, void *dst, U32 *out_desc)
+{
+    TensorDesc t;
+    memset(&t, 0xff, sizeof(t));
+    EE e = matrix_matrix_multiply_transform_rhs(rhs_desc(bfmt, K, N), src, &t, dst, X86_AVX512);
+    out_desc[0] = t.df;
+    out_desc[1] = t.nDims;
+    out_desc[2] = t.dims[0];
+    out_desc[3] = t.dims[1];
+    return e;
+}
+
+int ref_mmm_tmp_bytes(int transA, int bfmt, U32 M, U32 K, U32 N, U32 *bytes)
+{
+    TensorDesc a = transA ? tensor2df(DT_U8_Q, DF_TRANSPOSE, K, M) : tensor2df(DT_U8_Q, DF_NORMAL, M, K);
+    return matrix_matrix_multiply_tmp_bytes(a, rhs_desc(bfmt, K, N), bytes, X86_AVX512);
+}
+
+// cdt: DataType of C (DT_I32 / DT_F32 / DT_U8_Q)
+int ref_mmm(int transA, int bfmt, U32 M, U32 K, U32 N, const void *A, const void *B, U32 tmpBytes,
+    void *tmp, int cdt, void *C, const float *scale)
+{
+    TensorDesc a = transA ? tensor2df(DT_U8_Q, DF_TRANSPOSE, K, M) : tensor2df(DT_U8_Q, DF_NORMAL, M, K);
+    TensorDesc c = tensor2df((DataType)cdt, DF_NORMAL, M, N);
+    return matrix_matrix_multiply(a, A, rhs_desc(bfmt, K, N), B, tmpBytes, tmp, c, C, scale, X86_AVX512);
+}
+
+int ref_mvm_transform_weight_bytes(int wfmt, int wdt, U32 N, U32 K, U32 *bytes)
+{
+    return matrix_vector_multiply_transform_weight_bytes(mvm_desc(wfmt, N, K, (DataType)wdt), bytes, X86_AVX512);
+}
+
+int ref_mvm_transform_weight(int wfmt, U32 N, U32 K, const void *src, void *dst, U32 *out_desc)
+{
+    TensorDesc t;
+    memset(&t, 0xff, sizeof(t));
+    EE e = matrix_vector_multiply_transform_weight(mvm_desc(wfmt, N, K, DT_I8), src, &t, dst, X86_AVX512);
+    out_desc[0] = t.df;
+    out_desc[1] = t.nDims;
+    out_desc[2] = t.dims[0];
+    out_desc[3] = t.dims[1];
+    return e;
+}
+
+int ref_mvm_tmp_bytes(int wfmt, int wdt, U32 N, U32 K, U32 *bytes)
+{
+    DataType vdt = ((DataType)wdt == DT_I8) ? DT_U8_Q : DT_I8;
+    return matrix_vector_multiply_tmp_bytes(mvm_desc(wfmt, N, K, (DataType)wdt), tensor1d(vdt, K), bytes, X86_AVX512);
+}
+
+// wdt = DT_I8: s8 matrix x u8 vector; wdt = DT_U8_Q: u8 matrix (DF_NORMAL [N,K]) x s8 vector
+int ref_mvm(int wfmt, int wdt, U32 N, U32 K, const void *W, const void *x, U32 tmpBytes, void *tmp,
+    int rdt, void *y, const float *scale)
+{
+    DataType vdt = ((DataType)wdt == DT_I8) ? DT_U8_Q : DT_I8;
+    return matrix_vector_multiply(mvm_desc(wfmt, N, K, (DataType)wdt), W, tensor1d(vdt, K), x, tmpBytes,
+        tmp, tensor1d((DataType)rdt, N), y, scale, X86_AVX512);
+}
+
+int ref_quantize(int ddt, const void *data, U32 n, int qdt, void *q, float *scale, int mode)
+{
+    TensorDesc d = tensor1d((DataType)ddt, n);
+    TensorDesc qd = tensor1d((DataType)qdt, n);
+    return quantize_x86(d, data, &qd, q, scale, mode);
+}
+
+int ref_dequantize(int qdt, void *q, U32 n, const float *scale, float *out)
+{
+    TensorDesc qd = tensor1d((DataType)qdt, n);
+    TensorDesc dd = tensor1d(DT_F32, n);
+    TensorDesc bd = tensor1d(DT_F32, 0);
+    return dequantize_x86(qd, q, scale, bd, nullptr, dd, out);
+}
+
+// packed_filter = 1: `offsetC` holds the compensation vector of a packed weight blob and is
+// added; 0: native-format filter, the vector is not added (avx512/quantize.cpp:244,259-262).
+int ref_quantize_bias_offsetC(const float *bias, U32 N, const int32_t *offsetC, int packed_filter,
+    const float *scale, int32_t *out)
+{
+    TensorDesc bd = tensor1d(DT_F32, N);
+    TensorDesc fd = tensor2df(DT_I8, packed_filter ? DF_NKNxKx : DF_NORMAL, N, N);
+    return quantize_bias_offsetC(bias, bd, DT_I32, offsetC, fd, scale, out);
+}
+
+int ref_requantize(const int8_t *in, U32 n, float inScale, int8_t *out, float outScale)
+{
+    TensorDesc d = tensor1d(DT_I8, n);
+    return requantize_cpu(d, (INT8 *)in, inScale, d, out, outScale, X86_AVX512);
+}
+
+}  // extern "C"
