@@ -1,0 +1,119 @@
+"""ctypes binding of libbolt_gfx950.so, mirroring include/bolt_types.h and include/bolt_gfx950.h.
+
+The library is the product; this module only declares its C-ABI. There is no CPU fallback: if the
+shared library is missing, importing `lib()` raises.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libbolt_gfx950.so")
+
+# DataType (common/uni/include/data_type.h:67-85)
+DT_U8, DT_I8, DT_U32, DT_I32, DT_F16, DT_F16_8Q, DT_F32, DT_BIN01, DT_BIN11, DT_F32_8Q, DT_U8_Q = range(11)
+# DataFormat (common/uni/include/tensor_desc.h:33-78)
+DF_NCHW, DF_NCHWC8, DF_NCHWN16C8 = 0, 2, 9
+DF_TRANSPOSE, DF_NORMAL, DF_NK, DF_NKN32K4, DF_NKNxKx, DF_NCHWC16, DF_NCHWC2NxC4 = 13, 14, 17, 21, 39, 41, 42
+# EE (common/uni/include/error.h:159-170)
+SUCCESS, NULL_POINTER, NOT_MATCH, NOT_FOUND, ALLOC_FAILED = 0, 1, 2, 3, 4
+NOT_IMPLEMENTED, NOT_SUPPORTED, UNKNOWN = 50, 51, 99
+# Arch (common/uni/include/sys.h:44-55, two values appended)
+CPU_GENERAL, X86_AVX512, AMD_GFX950, AMD_GFX950_DEVICE = 1, 9, 11, 12
+
+DIM_LEN = 20
+
+
+class TensorDesc(C.Structure):
+    _pack_ = 8
+    _fields_ = [("dt", C.c_uint32), ("df", C.c_uint32), ("nDims", C.c_uint32), ("dims", C.c_uint32 * DIM_LEN)]
+
+    def __repr__(self):
+        return "TensorDesc(dt=%d, df=%d, dims=%s)" % (self.dt, self.df, list(self.dims[:self.nDims])[::-1])
+
+
+assert C.sizeof(TensorDesc) == 92
+
+
+def tensor4df(dt, df, n, c, h, w):
+    d = TensorDesc()
+    d.dt, d.df, d.nDims = dt, df, 4
+    d.dims[0], d.dims[1], d.dims[2], d.dims[3] = w, h, c, n
+    return d
+
+
+def tensor2df(dt, df, rows, cols):
+    d = tensor4df(dt, df, 1, 1, rows, cols)
+    d.nDims = 2
+    return d
+
+
+def tensor1d(dt, n):
+    d = tensor4df(dt, DF_NCHW, 1, 1, 1, n)
+    d.nDims = 1
+    return d
+
+
+_vp, _u32, _f32p, _u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
+_TDp = C.POINTER(TensorDesc)
+
+# name -> (restype, argtypes); every symbol include/bolt_gfx950.h declares
+SIGNATURES = {
+    "bolt_gfx950_init": (C.c_int, []),
+    "bolt_gfx950_set_stream": (C.c_int, [_vp]),
+    "bolt_gfx950_synchronize": (C.c_int, []),
+    "bolt_gfx950_last_error": (C.c_char_p, []),
+    "bolt_gfx950_malloc": (_vp, [C.c_size_t]),
+    "bolt_gfx950_free": (None, [_vp]),
+    "bolt_gfx950_memcpy_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "bolt_gfx950_memcpy_d2h": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "bolt_gfx950_timer_start": (C.c_int, []),
+    "bolt_gfx950_timer_stop": (C.c_int, [_f32p]),
+    "matrix_matrix_multiply_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, _u32p, C.c_int]),
+    "matrix_matrix_multiply_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, _vp,
+                                                C.c_int]),
+    "matrix_matrix_multiply_rhs_format_gfx950": (C.c_int, [C.c_int]),
+    "matrix_matrix_multiply_transform_rhs_bytes_gfx950": (C.c_int, [TensorDesc, _u32p, _u32p, C.c_int]),
+    "matrix_matrix_multiply_transform_rhs_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, _vp, C.c_int]),
+    "matrix_vector_multiply_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, _u32p, C.c_int]),
+    "matrix_vector_multiply_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, _vp,
+                                                C.c_int]),
+    "matrix_vector_multiply_weight_format_gfx950": (C.c_int, [C.c_int]),
+    "matrix_vector_multiply_transform_weight_bytes_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
+    "matrix_vector_multiply_transform_weight_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, _vp, C.c_int]),
+    "quantize_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, _vp, _vp, C.c_int, C.c_int]),
+    "dequantize_gfx950": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, TensorDesc, _vp, C.c_int]),
+    "quantize_bias_offsetC_gfx950": (C.c_int, [_vp, TensorDesc, C.c_int, _vp, TensorDesc, _vp, _vp, C.c_int]),
+    "requantize_gfx950": (C.c_int, [TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_float, C.c_int]),
+    "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
+    "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library with argtypes set. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+class BoltError(RuntimeError):
+    pass
+
+
+def check(code, what=""):
+    if code != SUCCESS:
+        msg = lib().bolt_gfx950_last_error()
+        raise BoltError("%s failed with EE=%d (%s)" % (what, code, (msg or b"").decode()))

@@ -1,0 +1,1083 @@
+// C-ABI entry points: argument validation, Bolt's tmp / offsetC / scale conventions, host <-> device
+// staging for the host-pointer mode, and dispatch to the kernels. No arithmetic on tensor data
+// happens on the CPU here except the load-time weight pack in host-pointer mode.
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/bolt_gfx950.h"
+#include "kernels.h"
+#include "layout.h"
+
+using namespace bg;
+
+namespace {
+
+struct Ctx {
+    std::mutex mu;
+    bool ready = false;
+    hipStream_t stream = nullptr;
+    uint32_t *ws = nullptr;  // device scratch words for the two-pass reductions
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+    struct Buf {
+        void *p;
+        size_t bytes;
+        bool busy;
+    };
+    std::vector<Buf> pool;
+};
+
+Ctx &ctx()
+{
+    static Ctx c;
+    return c;
+}
+
+EE fail(EE code, const char *what, hipError_t he = hipSuccess)
+{
+    Ctx &c = ctx();
+    c.err = what;
+    if (he != hipSuccess) {
+        c.err += ": ";
+        c.err += hipGetErrorString(he);
+    }
+    return code;
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e__ = (expr);                        \
+        if (e__ != hipSuccess) {                        \
+            return fail(UNKNOWN, #expr, e__);           \
+        }                                               \
+    } while (0)
+
+EE ensure_init()
+{
+    Ctx &c = ctx();
+    std::lock_guard<std::mutex> lk(c.mu);
+    if (c.ready) {
+        return SUCCESS;
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) {
+        return fail(NOT_SUPPORTED, "no HIP device available", e);
+    }
+    e = hipMalloc((void **)&c.ws, 256);
+    if (e != hipSuccess) {
+        return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
+    }
+    c.ready = true;
+    return SUCCESS;
+}
+
+// Grow-only device staging pool for the host-pointer mode.
+struct Stage {
+    std::vector<size_t> taken;
+    ~Stage()
+    {
+        Ctx &c = ctx();
+        std::lock_guard<std::mutex> lk(c.mu);
+        for (size_t i : taken) {
+            c.pool[i].busy = false;
+        }
+    }
+    void *get(size_t bytes)
+    {
+        bytes = std::max<size_t>(bytes, 256);
+        Ctx &c = ctx();
+        std::lock_guard<std::mutex> lk(c.mu);
+        for (size_t i = 0; i < c.pool.size(); ++i) {
+            if (!c.pool[i].busy && c.pool[i].bytes >= bytes) {
+                c.pool[i].busy = true;
+                taken.push_back(i);
+                return c.pool[i].p;
+            }
+        }
+        void *p = nullptr;
+        if (hipMalloc(&p, bytes) != hipSuccess) {
+            return nullptr;
+        }
+        c.pool.push_back({p, bytes, true});
+        taken.push_back(c.pool.size() - 1);
+        return p;
+    }
+};
+
+EE get2d(TensorDesc d, DataType *dt, DataFormat *df, U32 *rows, U32 *cols)
+{
+    if (d.nDims != 2) {
+        return NOT_MATCH;
+    }
+    *dt = d.dt;
+    *df = d.df;
+    *cols = d.dims[0];
+    *rows = d.dims[1];
+    return SUCCESS;
+}
+
+EE get1d(TensorDesc d, DataType *dt, U32 *len)
+{
+    if (d.nDims != 1) {
+        return NOT_MATCH;
+    }
+    *dt = d.dt;
+    *len = d.dims[0];
+    return SUCCESS;
+}
+
+bool aligned4(const void *p)
+{
+    return ((uintptr_t)p & 3) == 0;
+}
+
+Epilogue epi_from_scale(const F32 *scale)
+{
+    Epilogue e;
+    memset(&e, 0, sizeof(e));
+    if (scale == nullptr) {
+        e.mode = EPI_I32;
+    } else if (scale[0] < 0) {
+        e.mode = EPI_U8;
+        e.factor = scale[1];
+    } else {
+        e.mode = EPI_F32;
+        e.factor = 1 / scale[0];
+    }
+    return e;
+}
+
+// ---- host-side weight pack (host-pointer mode, load time) ----------------------------------------
+void pack_host(bool mmm, const INT8 *src, size_t sk, size_t sn, U32 K, U32 N, INT8 *dst, I32 *comp)
+{
+    const U32 Kp = align_up(K, 8), N16 = align_up(N, 16);
+    memset(dst, 0, (size_t)N16 * Kp);
+    for (U32 n = 0; n < N; ++n) {
+        I32 s = 0;
+        for (U32 k = 0; k < K; ++k) {
+            const INT8 v = src[k * sk + n * sn];
+            s += v;
+            dst[mmm ? mmm_packed_offset(n, k, Kp) : mvm_packed_offset(n, k, Kp)] = v;
+        }
+        comp[n] = s * (-128);
+    }
+}
+
+// bytes of the packed matrix part for an N x K weight
+U32 packed_matrix_bytes(U32 N, U32 K)
+{
+    return align_up(N, 16) * align_up(K, 8);
+}
+
+// ---- GEMM core (device pointers) -----------------------------------------------------------------
+EE mmm_device(U32 M, U32 N, U32 K, DataFormat adf, const void *A, DataFormat bdf, const void *B, void *tmp,
+    DataType cdt, void *C, const F32 *scale)
+{
+    Ctx &c = ctx();
+    const INT8 *Bp = (const INT8 *)B;
+    U8 *t = (U8 *)tmp;
+    const U32 rhs = packed_matrix_bytes(N, K);
+    if (bdf != DF_NKNxKx) {
+        // on-the-fly transform into tmp, then tmp advances past the packed matrix so that its
+        // first N int32 are the compensation vector the transform just wrote (mmm.cpp:207-219)
+        const bool tr = (bdf == DF_TRANSPOSE);
+        HIP_TRY(launch_pack_mmm((const int8_t *)B, tr ? 1 : N, tr ? K : 1, K, N, (int8_t *)t, (int32_t *)(t + rhs),
+            c.stream));
+        Bp = (const INT8 *)t;
+        t += rhs;
+    }
+    if (cdt == DT_I32) {
+        scale = nullptr;  // mmm.cpp:222-224
+    }
+    GemmArgs g;
+    g.A = (const uint8_t *)A;
+    g.transA = (adf == DF_TRANSPOSE);
+    g.lda = g.transA ? M : K;
+    g.Bp = (const int8_t *)Bp;
+    g.M = M;
+    g.N = N;
+    g.K = K;
+    g.ob = (const int32_t *)t;
+    g.comp = (const int32_t *)(Bp + rhs);
+    g.C = C;
+    g.epi = epi_from_scale(scale);
+    g.add_cin = (g.epi.mode != EPI_U8);
+    HIP_TRY(launch_gemm_u8s8(g, c.stream));
+    return SUCCESS;
+}
+
+EE mvm_device(U32 N, U32 K, DataType mdt, DataFormat mdf, const void *W, const void *x, void *tmp, void *y,
+    const F32 *scale)
+{
+    Ctx &c = ctx();
+    Epilogue epi = epi_from_scale(scale);
+    if (mdt == DT_U8_Q) {
+        // u8 matrix x s8 vector; N = rows of the matrix
+        const bool tr = (mdf == DF_TRANSPOSE);
+        HIP_TRY(launch_gemv_u8s8((const uint8_t *)W, tr ? 1 : K, tr ? N : 1, (const int8_t *)x, K, N, y, epi,
+            c.stream));
+        return SUCCESS;
+    }
+    GemvArgs g;
+    const U32 mat = packed_matrix_bytes(N, K);
+    if (mdf != DF_NKN32K4) {
+        // unpacked: tmp = [compensation N*4][packed matrix], as mvm.cpp:176-182 lays it out
+        U8 *t = (U8 *)tmp;
+        const bool tr = (mdf == DF_TRANSPOSE);
+        HIP_TRY(launch_pack_mvm((const int8_t *)W, tr ? N : 1, tr ? 1 : K, K, N, (int8_t *)(t + (size_t)N * 4),
+            (int32_t *)t, c.stream));
+        g.W = (const int8_t *)(t + (size_t)N * 4);
+        g.comp = (const int32_t *)t;
+    } else {
+        g.W = (const int8_t *)W;
+        g.comp = (const int32_t *)((const U8 *)W + mat);
+    }
+    g.ldw = align_up(K, 8);
+    g.x = (const uint8_t *)x;
+    g.K = K;
+    g.N = N;
+    g.ob = (const int32_t *)tmp;
+    g.y = y;
+    g.epi = epi;
+    g.add_yin = (epi.mode != EPI_U8);
+    HIP_TRY(launch_gemv_s8u8(g, c.stream));
+    return SUCCESS;
+}
+
+U32 out_elem_bytes(const F32 *scale)
+{
+    return (scale && scale[0] < 0) ? 1 : 4;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ---- runtime -------------------------------------------------------------------------------------
+EE bolt_gfx950_init(void)
+{
+    return ensure_init();
+}
+
+EE bolt_gfx950_set_stream(void *stream)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    ctx().stream = (hipStream_t)stream;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_synchronize(void)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipStreamSynchronize(ctx().stream));
+    return SUCCESS;
+}
+
+const char *bolt_gfx950_last_error(void)
+{
+    return ctx().err.c_str();
+}
+
+void *bolt_gfx950_malloc(size_t bytes)
+{
+    if (ensure_init() != SUCCESS) {
+        return nullptr;
+    }
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
+        return nullptr;
+    }
+    return p;
+}
+
+void bolt_gfx950_free(void *p)
+{
+    if (p) {
+        (void)hipFree(p);
+    }
+}
+
+EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+    HIP_TRY(hipStreamSynchronize(ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    HIP_TRY(hipStreamSynchronize(ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_timer_start(void)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    if (!c.ev0) {
+        HIP_TRY(hipEventCreate(&c.ev0));
+        HIP_TRY(hipEventCreate(&c.ev1));
+    }
+    HIP_TRY(hipEventRecord(c.ev0, c.stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_timer_stop(float *ms)
+{
+    Ctx &c = ctx();
+    if (!c.ev0 || !ms) {
+        return fail(NULL_POINTER, "timer_stop without timer_start");
+    }
+    HIP_TRY(hipEventRecord(c.ev1, c.stream));
+    HIP_TRY(hipEventSynchronize(c.ev1));
+    HIP_TRY(hipEventElapsedTime(ms, c.ev0, c.ev1));
+    return SUCCESS;
+}
+
+// ---- GEMM ----------------------------------------------------------------------------------------
+DataFormat matrix_matrix_multiply_rhs_format_gfx950(DataType dt)
+{
+    (void)dt;
+    return DF_NKNxKx;
+}
+
+// Sizes follow mmm_avx512_vnni.cpp:22-58 exactly so a caller sized for the x86 path fits.
+EE matrix_matrix_multiply_transform_rhs_bytes_gfx950(TensorDesc desc, U32 *bytes, U32 *rhsBytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    DataType dt;
+    DataFormat df;
+    U32 K, N;
+    EE e = get2d(desc, &dt, &df, &K, &N);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (dt != DT_I8 && dt != DT_U8_Q) {
+        return NOT_SUPPORTED;
+    }
+    if (df == DF_TRANSPOSE) {
+        std::swap(K, N);
+    }
+    U32 matrix = 0, total = 0;
+    if (df != DF_NKNxKx) {
+        matrix = packed_matrix_bytes(N, K);
+        total = N * 4 + matrix + 64;
+    }
+    if (rhsBytes) {
+        *rhsBytes = matrix;
+    }
+    if (bytes) {
+        *bytes = total;
+    }
+    return SUCCESS;
+}
+
+EE matrix_matrix_multiply_tmp_bytes_gfx950(TensorDesc matrixADesc, TensorDesc matrixBDesc, U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    DataType adt, bdt;
+    DataFormat adf, bdf;
+    U32 M, K, K2, N;
+    EE e = get2d(matrixADesc, &adt, &adf, &M, &K);
+    if (e != SUCCESS) {
+        return e;
+    }
+    e = get2d(matrixBDesc, &bdt, &bdf, &K2, &N);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (adf == DF_TRANSPOSE) {
+        std::swap(M, K);
+    }
+    if (bdf == DF_TRANSPOSE) {
+        std::swap(K2, N);
+    }
+    if (adt != DT_U8_Q && adt != DT_I8) {
+        return NOT_SUPPORTED;
+    }
+    e = matrix_matrix_multiply_transform_rhs_bytes_gfx950(matrixBDesc, bytes, nullptr, arch);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (adf == DF_NORMAL) {
+        *bytes += 32 * K;
+        if (K % 8 != 0) {
+            *bytes += align_up(M, 24) * 8;
+        }
+    } else if (adf == DF_TRANSPOSE) {
+        *bytes += align_up(M, 24) * std::min<U32>(4096, align_up(K, 8));
+    } else {
+        return NOT_SUPPORTED;
+    }
+    *bytes += N * 4;
+    *bytes += 64;
+    return SUCCESS;
+}
+
+EE matrix_matrix_multiply_transform_rhs_gfx950(TensorDesc desc, const void *src, TensorDesc *descTran, void *dst,
+    Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (desc.df == DF_NKNxKx) {
+        return SUCCESS;  // already packed: descTran and dst stay untouched (x86/mmm.cpp:135-137)
+    }
+    if (desc.dt != DT_I8 || (desc.df != DF_NORMAL && desc.df != DF_TRANSPOSE)) {
+        return NOT_SUPPORTED;
+    }
+    if (!src || !dst || !descTran) {
+        return NULL_POINTER;
+    }
+    DataType dt;
+    DataFormat df;
+    U32 rows, cols;
+    EE e = get2d(desc, &dt, &df, &rows, &cols);
+    if (e != SUCCESS) {
+        return e;
+    }
+    const bool tr = (df == DF_TRANSPOSE);
+    const U32 K = tr ? cols : rows, N = tr ? rows : cols;
+    const U32 mat = packed_matrix_bytes(N, K);
+    if (arch == AMD_GFX950) {
+        pack_host(true, (const INT8 *)src, tr ? 1 : N, tr ? K : 1, K, N, (INT8 *)dst, (I32 *)((U8 *)dst + mat));
+    } else {
+        e = ensure_init();
+        if (e != SUCCESS) {
+            return e;
+        }
+        if (!aligned4(dst)) {
+            return fail(NOT_SUPPORTED, "device dst must be 4-byte aligned");
+        }
+        HIP_TRY(launch_pack_mmm((const int8_t *)src, tr ? 1 : N, tr ? K : 1, K, N, (int8_t *)dst,
+            (int32_t *)((U8 *)dst + mat), ctx().stream));
+    }
+    *descTran = desc;
+    descTran->df = DF_NKNxKx;
+    if (tr) {
+        std::swap(descTran->dims[0], descTran->dims[1]);
+    }
+    return SUCCESS;
+}
+
+EE matrix_matrix_multiply_gfx950(TensorDesc matrixADesc, const void *matrixA, TensorDesc matrixBDesc,
+    const void *matrixB, U32 bytes, void *tmp, TensorDesc matrixCDesc, void *matrixC, const F32 *scale, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (bytes != 0 && tmp == nullptr) {
+        return NULL_POINTER;
+    }
+    if (!matrixA || !matrixB || !matrixC) {
+        return NULL_POINTER;
+    }
+    if (tensorNumElements(matrixCDesc) == 0) {
+        return SUCCESS;
+    }
+    DataType adt, bdt, cdt;
+    DataFormat adf, bdf, cdf;
+    U32 M, K, K2, N, CM, CN;
+    if (get2d(matrixADesc, &adt, &adf, &M, &K) != SUCCESS || get2d(matrixBDesc, &bdt, &bdf, &K2, &N) != SUCCESS ||
+        get2d(matrixCDesc, &cdt, &cdf, &CM, &CN) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (adt != bdt && !(adt == DT_U8_Q && bdt == DT_I8)) {
+        return NOT_MATCH;
+    }
+    if (adf == DF_TRANSPOSE) {
+        std::swap(M, K);
+    }
+    if (bdf == DF_TRANSPOSE) {
+        std::swap(K2, N);
+    }
+    if (M != CM || N != CN || K != K2) {
+        return NOT_MATCH;
+    }
+    if (bdt != DT_I8 || (adf != DF_NORMAL && adf != DF_TRANSPOSE) ||
+        (bdf != DF_NORMAL && bdf != DF_TRANSPOSE && bdf != DF_NKNxKx)) {
+        return NOT_SUPPORTED;
+    }
+    if (tmp == nullptr) {
+        return NULL_POINTER;  // the first N int32 of tmp carry offsetC (x86/mmm.cpp path)
+    }
+    U32 need = 0;
+    if (bdf != DF_NKNxKx) {
+        need = packed_matrix_bytes(N, K);
+        if (bytes < need + N * 4) {
+            return NOT_MATCH;
+        }
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    const F32 *sc = (cdt == DT_I32) ? nullptr : scale;
+    if (arch == AMD_GFX950_DEVICE) {
+        if (!aligned4(tmp) || !aligned4(matrixC) || !aligned4(matrixB)) {
+            return fail(NOT_SUPPORTED, "device tmp / B / C must be 4-byte aligned");
+        }
+        return mmm_device(M, N, K, adf, matrixA, bdf, matrixB, tmp, cdt, matrixC, sc);
+    }
+    // host-pointer mode
+    Ctx &c = ctx();
+    Stage st;
+    const size_t aBytes = (size_t)M * K;
+    const size_t bBytes = (bdf == DF_NKNxKx) ? (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4 : (size_t)K * N;
+    const size_t tBytes = (size_t)need + (size_t)N * 4;
+    const size_t cBytes = (size_t)M * N * out_elem_bytes(sc);
+    void *dA = st.get(aBytes), *dB = st.get(bBytes), *dT = st.get(tBytes), *dC = st.get(cBytes);
+    if (!dA || !dB || !dT || !dC) {
+        return fail(ALLOC_FAILED, "device staging");
+    }
+    HIP_TRY(hipMemcpyAsync(dA, matrixA, aBytes, hipMemcpyHostToDevice, c.stream));
+    HIP_TRY(hipMemcpyAsync(dB, matrixB, bBytes, hipMemcpyHostToDevice, c.stream));
+    if (bdf == DF_NKNxKx) {
+        HIP_TRY(hipMemcpyAsync(dT, tmp, (size_t)N * 4, hipMemcpyHostToDevice, c.stream));
+    }
+    if (out_elem_bytes(sc) == 4) {
+        HIP_TRY(hipMemcpyAsync(dC, matrixC, cBytes, hipMemcpyHostToDevice, c.stream));
+    }
+    e = mmm_device(M, N, K, adf, dA, bdf, dB, dT, cdt, dC, sc);
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(matrixC, dC, cBytes, hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return SUCCESS;
+}
+
+// ---- GEMV ----------------------------------------------------------------------------------------
+DataFormat matrix_vector_multiply_weight_format_gfx950(DataType dt)
+{
+    return (dt == DT_U8_Q) ? DF_NK : DF_NKN32K4;  // mvm.cpp:51-77
+}
+
+static EE mvm_bytes(TensorDesc matrixDesc, U32 *bytes)
+{
+    DataType dt;
+    DataFormat df;
+    U32 row, col;
+    EE e = get2d(matrixDesc, &dt, &df, &row, &col);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (df == DF_TRANSPOSE) {
+        std::swap(row, col);
+    }
+    if (dt != DT_I8 && dt != DT_U8_Q) {
+        return NOT_SUPPORTED;
+    }
+    // x86/mvm.cpp:23-42
+    *bytes = 0;
+    if (dt == DT_I8) {
+        *bytes += row * 4;
+    }
+    if (dt == DT_U8_Q && col % 32 != 0) {
+        *bytes += 32 * (row + 1);
+    }
+    if (df != matrix_vector_multiply_weight_format_gfx950(dt)) {
+        *bytes += align_up(row, 16) * align_up(col, 8);
+        *bytes += 32;
+    }
+    return SUCCESS;
+}
+
+EE matrix_vector_multiply_transform_weight_bytes_gfx950(TensorDesc desc, U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    return mvm_bytes(desc, bytes);
+}
+
+EE matrix_vector_multiply_tmp_bytes_gfx950(TensorDesc matrixDesc, TensorDesc vectorDesc, U32 *bytes, Arch arch)
+{
+    (void)vectorDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    return mvm_bytes(matrixDesc, bytes);  // x86/mvm.cpp:77-100: same formula
+}
+
+EE matrix_vector_multiply_transform_weight_gfx950(TensorDesc desc, const void *src, TensorDesc *descTran, void *dst,
+    Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (desc.df == matrix_vector_multiply_weight_format_gfx950(desc.dt)) {
+        return SUCCESS;  // x86/mvm.cpp:47-49
+    }
+    if (desc.dt != DT_I8 || (desc.df != DF_NORMAL && desc.df != DF_TRANSPOSE)) {
+        return NOT_SUPPORTED;
+    }
+    if (!src || !dst || !descTran) {
+        return NULL_POINTER;
+    }
+    DataType dt;
+    DataFormat df;
+    U32 rows, cols;
+    EE e = get2d(desc, &dt, &df, &rows, &cols);
+    if (e != SUCCESS) {
+        return e;
+    }
+    const bool tr = (df == DF_TRANSPOSE);
+    const U32 N = tr ? cols : rows, K = tr ? rows : cols;
+    const U32 mat = packed_matrix_bytes(N, K);
+    if (arch == AMD_GFX950) {
+        pack_host(false, (const INT8 *)src, tr ? N : 1, tr ? 1 : K, K, N, (INT8 *)dst, (I32 *)((U8 *)dst + mat));
+    } else {
+        e = ensure_init();
+        if (e != SUCCESS) {
+            return e;
+        }
+        if (!aligned4(dst)) {
+            return fail(NOT_SUPPORTED, "device dst must be 4-byte aligned");
+        }
+        HIP_TRY(launch_pack_mvm((const int8_t *)src, tr ? N : 1, tr ? 1 : K, K, N, (int8_t *)dst,
+            (int32_t *)((U8 *)dst + mat), ctx().stream));
+    }
+    *descTran = desc;
+    if (tr) {
+        std::swap(descTran->dims[0], descTran->dims[1]);
+    }
+    descTran->df = DF_NKN32K4;
+    return SUCCESS;
+}
+
+EE matrix_vector_multiply_gfx950(TensorDesc matrixDesc, const void *matrix, TensorDesc vectorDesc, const void *vector,
+    U32 bytes, void *tmp, TensorDesc resultDesc, void *result, const F32 *scale, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if ((bytes != 0 && tmp == nullptr) || !matrix || !vector || !result) {
+        return NULL_POINTER;
+    }
+    DataType mdt, vdt, rdt;
+    DataFormat mdf;
+    U32 row, col, vlen, rlen;
+    if (get2d(matrixDesc, &mdt, &mdf, &row, &col) != SUCCESS || get1d(vectorDesc, &vdt, &vlen) != SUCCESS ||
+        get1d(resultDesc, &rdt, &rlen) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (mdf == DF_TRANSPOSE) {
+        std::swap(row, col);
+    }
+    if (row != rlen || col != vlen) {
+        return NOT_MATCH;
+    }
+    if (mdt == DT_U8_Q && mdf == DF_NK) {
+        return NOT_SUPPORTED;  // mvm.cpp:172-175
+    }
+    if (mdt != DT_I8 && mdt != DT_U8_Q) {
+        return NOT_SUPPORTED;
+    }
+    if (mdt == DT_I8 && mdf != DF_NORMAL && mdf != DF_TRANSPOSE && mdf != DF_NKN32K4) {
+        return NOT_SUPPORTED;
+    }
+    if (mdt == DT_U8_Q && mdf != DF_NORMAL && mdf != DF_TRANSPOSE) {
+        return NOT_SUPPORTED;
+    }
+    if (row == 0) {
+        return SUCCESS;
+    }
+    const U32 N = row, K = col;
+    const bool unpacked = (mdt == DT_I8 && mdf != DF_NKN32K4);
+    if (mdt == DT_I8 && tmp == nullptr) {
+        return NULL_POINTER;  // CHECK_REQUIREMENT(offsetCBias != nullptr), x86/mvm.cpp:121
+    }
+    if (unpacked && bytes < N * 4 + packed_matrix_bytes(N, K)) {
+        return NOT_MATCH;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (arch == AMD_GFX950_DEVICE) {
+        if ((mdt == DT_I8 && !aligned4(tmp)) || !aligned4(result) || (mdt == DT_I8 && !aligned4(matrix))) {
+            return fail(NOT_SUPPORTED, "device tmp / matrix / result must be 4-byte aligned");
+        }
+        return mvm_device(N, K, mdt, mdf, matrix, vector, tmp, result, scale);
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const size_t wBytes = (mdt == DT_I8 && !unpacked) ? (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4 : (size_t)N * K;
+    const size_t tBytes = (size_t)N * 4 + (unpacked ? packed_matrix_bytes(N, K) : 0);
+    const size_t yBytes = (size_t)N * out_elem_bytes(scale);
+    void *dW = st.get(wBytes), *dX = st.get(K), *dT = st.get(tBytes), *dY = st.get(yBytes);
+    if (!dW || !dX || !dT || !dY) {
+        return fail(ALLOC_FAILED, "device staging");
+    }
+    HIP_TRY(hipMemcpyAsync(dW, matrix, wBytes, hipMemcpyHostToDevice, c.stream));
+    HIP_TRY(hipMemcpyAsync(dX, vector, K, hipMemcpyHostToDevice, c.stream));
+    if (mdt == DT_I8 && !unpacked) {
+        HIP_TRY(hipMemcpyAsync(dT, tmp, (size_t)N * 4, hipMemcpyHostToDevice, c.stream));
+    }
+    if (out_elem_bytes(scale) == 4) {
+        HIP_TRY(hipMemcpyAsync(dY, result, yBytes, hipMemcpyHostToDevice, c.stream));
+    }
+    e = mvm_device(N, K, mdt, mdf, dW, dX, dT, dY, scale);
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(result, dY, yBytes, hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return SUCCESS;
+}
+
+// ---- quantize family -----------------------------------------------------------------------------
+EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *qData, F32 *scale, int mode, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!qDesc) {
+        return NULL_POINTER;
+    }
+    const DataType ddt = dDesc.dt, qdt = qDesc->dt;
+    const bool f32in = (ddt == DT_F32 || ddt == DT_F32_8Q);
+    const bool ok = (f32in && (qdt == DT_I8 || qdt == DT_U8_Q)) || (ddt == DT_U8_Q && qdt == DT_I8) ||
+        (ddt == DT_I32 && (qdt == DT_I8 || qdt == DT_U8_Q));
+    if (!ok) {
+        return NOT_SUPPORTED;
+    }
+    const bool needs_scale = !(ddt == DT_U8_Q);
+    if (needs_scale && scale == nullptr) {
+        return NOT_MATCH;  // avx512/quantize.cpp:123-125
+    }
+    const U32 n = tensorNumElements(dDesc);
+    if (n != 0 && (!data || !qData)) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const void *dIn = data;
+    void *dOut = qData;
+    const size_t inBytes = (size_t)n * bytesOf(ddt);
+    if (arch == AMD_GFX950) {
+        void *a = st.get(inBytes), *b = st.get(n);
+        if (!a || !b) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, data, inBytes, hipMemcpyHostToDevice, c.stream));
+        dIn = a;
+        dOut = b;
+    } else if (!aligned4(data) && ddt != DT_U8_Q) {
+        return fail(NOT_SUPPORTED, "device data must be 4-byte aligned");
+    }
+    float *dscale = (float *)(c.ws + 8);
+    bool read_back = false;
+    if (f32in) {
+        const bool dynamic = (!mode || *scale <= 0);
+        if (dynamic) {
+            HIP_TRY(launch_absmax_f32((const float *)dIn, n, c.ws, c.stream));
+        }
+        HIP_TRY(launch_quantize_f32((const float *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, *scale, nullptr, mode, dscale,
+            c.stream));
+        read_back = dynamic;
+    } else if (ddt == DT_U8_Q) {
+        HIP_TRY(launch_u8_to_i8((const uint8_t *)dIn, n, (int8_t *)dOut, c.stream));
+    } else {
+        const bool dynamic = (scale[0] < 0 && scale[1] > 0);
+        if (dynamic) {
+            HIP_TRY(launch_absmax_i32((const int32_t *)dIn, n, c.ws, c.stream));
+        }
+        HIP_TRY(launch_requant_i32((const int32_t *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, scale[0], scale[1], dscale,
+            c.stream));
+        read_back = dynamic;
+    }
+    if (arch == AMD_GFX950 && n) {
+        HIP_TRY(hipMemcpyAsync(qData, dOut, n, hipMemcpyDeviceToHost, c.stream));
+    }
+    if (read_back) {
+        // the scale is a host value in this interface: the call completes before returning it
+        HIP_TRY(hipMemcpyAsync(scale, dscale, 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    } else if (arch == AMD_GFX950) {
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
+EE dequantize_gfx950(TensorDesc qDesc, void *qData, const F32 *scale, TensorDesc bDesc, void *bData, TensorDesc dDesc,
+    void *dData, Arch arch)
+{
+    (void)bDesc;
+    (void)bData;  // the x86 path ignores the bias argument (cpu/x86/dequantize.cpp:19-48)
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (dDesc.dt != DT_F32 || (qDesc.dt != DT_I32 && qDesc.dt != DT_U8_Q)) {
+        return NOT_SUPPORTED;
+    }
+    if (!scale) {
+        return NULL_POINTER;
+    }
+    const U32 n = tensorNumElements(dDesc);
+    if (n == 0) {
+        return SUCCESS;
+    }
+    if (!qData || !dData) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const void *dIn = qData;
+    void *dOut = dData;
+    const size_t inBytes = (size_t)n * bytesOf(qDesc.dt);
+    if (arch == AMD_GFX950) {
+        void *a = st.get(inBytes), *b = st.get((size_t)n * 4);
+        if (!a || !b) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, qData, inBytes, hipMemcpyHostToDevice, c.stream));
+        dIn = a;
+        dOut = b;
+    }
+    if (qDesc.dt == DT_I32) {
+        HIP_TRY(launch_dequant_i32((const int32_t *)dIn, n, nullptr, *scale, (float *)dOut, c.stream));
+    } else {
+        HIP_TRY(launch_dequant_u8((const uint8_t *)dIn, n, nullptr, *scale, (float *)dOut, c.stream));
+    }
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(dData, dOut, (size_t)n * 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
+static bool native_filter_format(DataFormat df)
+{
+    return df == DF_NCHW || df == DF_NHWC || df == DF_MTK || df == DF_NORMAL || df == DF_TRANSPOSE;
+}
+
+EE quantize_bias_offsetC_gfx950(const void *bias, TensorDesc biasDesc, DataType qType, const void *filter,
+    TensorDesc filterDesc, const F32 *scale, void *offsetCBias, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (qType != DT_I32 || (bias && biasDesc.dt != DT_F32 && biasDesc.dt != DT_I32)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bias && !filter) {
+        return SUCCESS;  // avx512/quantize.cpp:246-248
+    }
+    if (!offsetCBias) {
+        return NULL_POINTER;
+    }
+    U32 N = bias ? tensorNumElements(biasDesc) : 0;
+    const bool no_bias = (!bias || N == 0);
+    if (no_bias) {
+        N = std::max(filterDesc.dims[0], filterDesc.dims[1]);
+    }
+    // `filter` points at the compensation vector of a packed blob; native formats carry none
+    const bool add_off = filter && !native_filter_format(filterDesc.df);
+    if (!no_bias && biasDesc.dt == DT_F32 && !scale) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const void *dBias = no_bias ? nullptr : bias;
+    const void *dOff = add_off ? filter : nullptr;
+    void *dOut = offsetCBias;
+    if (arch == AMD_GFX950) {
+        dOut = st.get((size_t)N * 4);
+        if (dBias) {
+            void *b = st.get((size_t)N * 4);
+            HIP_TRY(hipMemcpyAsync(b, bias, (size_t)N * 4, hipMemcpyHostToDevice, c.stream));
+            dBias = b;
+        }
+        if (dOff) {
+            void *o = st.get((size_t)N * 4);
+            HIP_TRY(hipMemcpyAsync(o, filter, (size_t)N * 4, hipMemcpyHostToDevice, c.stream));
+            dOff = o;
+        }
+    }
+    if (!no_bias && biasDesc.dt == DT_I32) {
+        // integer bias (cpu/x86/quantize.cpp:100-110) has no caller on the int8 FullyConnected /
+        // Convolution path
+        return fail(NOT_SUPPORTED, "DT_I32 bias is not supported");
+    }
+    HIP_TRY(launch_bias_offsetC((const float *)dBias, N, (const int32_t *)dOff, nullptr, scale ? scale[0] : 1.0f,
+        (int32_t *)dOut, c.stream));
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(offsetCBias, dOut, (size_t)N * 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
+EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDesc outputDesc, INT8 *output,
+    F32 outputScale, Arch arch)
+{
+    (void)inputDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    const U32 n = tensorNumElements(outputDesc);
+    if (n == 0) {
+        return SUCCESS;
+    }
+    if (!input || !output) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    if (arch == AMD_GFX950) {
+        if (outputScale == inputScale) {
+            memcpy(output, input, n);
+            return SUCCESS;
+        }
+        Stage st;
+        void *a = st.get(n), *b = st.get(n);
+        if (!a || !b) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, input, n, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(launch_requantize_i8((const int8_t *)a, n, outputScale / inputScale, (int8_t *)b, c.stream));
+        HIP_TRY(hipMemcpyAsync(output, b, n, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        return SUCCESS;
+    }
+    if (outputScale == inputScale) {
+        HIP_TRY(hipMemcpyAsync(output, input, n, hipMemcpyDeviceToDevice, c.stream));
+        return SUCCESS;
+    }
+    HIP_TRY(launch_requantize_i8(input, n, outputScale / inputScale, output, c.stream));
+    return SUCCESS;
+}
+
+// ---- device-resident-scale forms ------------------------------------------------------------------
+EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode)
+{
+    if (qdt != DT_I8 && qdt != DT_U8_Q) {
+        return NOT_SUPPORTED;
+    }
+    if (!data || !q || !dscale) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    // the caller's scale lives on the device, so whether it asks for a dynamic scale is only known
+    // there: the |max| pass always runs.
+    HIP_TRY(launch_absmax_f32(data, n, c.ws, c.stream));
+    HIP_TRY(launch_quantize_f32(data, n, q, qdt == DT_U8_Q, c.ws, 0.0f, dscale, mode, dscale, c.stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
+    float *C, const float *dscaleI, const float *scaleW, const float *bias)
+{
+    if (!A || !packedB || !offsetC || !C || !dscaleI || !scaleW) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = (const uint8_t *)A;
+    g.lda = K;
+    g.Bp = (const int8_t *)packedB;
+    g.M = M;
+    g.N = N;
+    g.K = K;
+    g.ob = offsetC;
+    g.comp = (const int32_t *)((const U8 *)packedB + packed_matrix_bytes(N, K));
+    g.C = C;
+    g.epi.mode = EPI_F32_CH;
+    g.epi.scaleI = dscaleI;
+    g.epi.scaleW = scaleW;
+    g.epi.bias = bias;
+    HIP_TRY(launch_gemm_u8s8(g, ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void *x, const I32 *offsetC, float *y,
+    const float *dscaleI, const float *scaleW, const float *bias)
+{
+    if (!packedW || !x || !offsetC || !y || !dscaleI || !scaleW) {
+        return NULL_POINTER;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.W = (const int8_t *)packedW;
+    g.ldw = align_up(K, 8);
+    g.x = (const uint8_t *)x;
+    g.K = K;
+    g.N = N;
+    g.ob = offsetC;
+    g.comp = (const int32_t *)((const U8 *)packedW + packed_matrix_bytes(N, K));
+    g.y = y;
+    g.epi.mode = EPI_F32_CH;
+    g.epi.scaleI = dscaleI;
+    g.epi.scaleW = scaleW;
+    g.epi.bias = bias;
+    HIP_TRY(launch_gemv_s8u8(g, ctx().stream));
+    return SUCCESS;
+}
+
+}  // extern "C"

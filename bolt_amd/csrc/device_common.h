@@ -1,0 +1,117 @@
+// Device-side helpers shared by the gfx950 kernels: the exact rounding / saturation steps of
+// the x86 AVX-512 epilogues the results must match bit-for-bit, and wave64 reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bg {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// vcvtps2dq: round to nearest even; NaN and out-of-range give 0x80000000.
+__device__ __forceinline__ int rne_i32(float v)
+{
+    if (!(v >= -2147483648.0f && v < 2147483648.0f)) {
+        return (int)0x80000000;
+    }
+    return (int)__builtin_rintf(v);
+}
+
+// vpmovusdb: the dword is saturated as an UNSIGNED number, so every negative becomes 255.
+__device__ __forceinline__ unsigned usat8_u(int v)
+{
+    return ((unsigned)v > 255u) ? 255u : (unsigned)v;
+}
+
+// vpmovsdb: signed saturation to [-128, 127].
+__device__ __forceinline__ int ssat8(int v)
+{
+    return v < -128 ? -128 : (v > 127 ? 127 : v);
+}
+
+// Output selector of the GEMM / GEMV / conv epilogue.
+enum EpiMode : int {
+    EPI_I32 = 0,       // raw accumulator
+    EPI_F32 = 1,       // cvt(acc) * factor                      (factor = 1.0f / scale[0])
+    EPI_U8 = 2,        // usat8_u(rne(cvt(acc) * factor) + 128)  (factor = scale[1])
+    EPI_F32_CH = 3,    // cvt(acc) * (1.0f / (sI * sW[n])) + bias[n]   per-output-channel extension
+    EPI_U8_TRUNC = 4   // (int)(cvt(acc) * factor + 128.0f), > 255 -> 255, else low byte
+};
+
+struct Epilogue {
+    int mode;
+    float factor;            // EPI_F32 / EPI_U8 when dfactor == nullptr
+    const float *dfactor;    // optional device scalar: EPI_F32 uses 1.0f / *dfactor, EPI_U8 uses *dfactor
+    const float *scaleI;     // EPI_F32_CH: device scalar input scale
+    const float *scaleW;     // EPI_F32_CH: device per-channel weight scales [N]
+    const float *bias;       // EPI_F32_CH: optional device fp32 bias [N]
+};
+
+__device__ __forceinline__ float epi_factor(const Epilogue &e)
+{
+    if (e.dfactor) {
+        float s = *e.dfactor;
+        return (e.mode == EPI_F32) ? 1.0f / s : s;
+    }
+    return e.factor;
+}
+
+__device__ __forceinline__ unsigned epi_u8(int acc, float factor)
+{
+    float f = (float)acc * factor;
+    return usat8_u((int)((unsigned)rne_i32(f) + 128u));
+}
+
+__device__ __forceinline__ unsigned epi_u8_trunc(int acc, float factor)
+{
+    float f = (float)acc * factor;
+    float g = f + 128.0f;
+    int t = (!(g >= -2147483648.0f && g < 2147483648.0f)) ? (int)0x80000000 : (int)g;
+    return (t > 255) ? 255u : ((unsigned)t & 0xffu);
+}
+
+__device__ __forceinline__ float epi_f32_ch(int acc, float sI, float sW, const float *bias, int n)
+{
+    float s = sI * sW;
+    float f = 1.0f / s;
+    float v = (float)acc * f;
+    if (bias) {
+        v = v + bias[n];
+    }
+    return v;
+}
+
+__device__ __forceinline__ int wave_reduce_add(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
+__device__ __forceinline__ float wave_reduce_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, off, 64));
+    }
+    return v;
+}
+
+__device__ __forceinline__ int wave_reduce_max_i(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        int o = __shfl_xor(v, off, 64);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+}  // namespace bg

@@ -1,0 +1,72 @@
+// Launchers of the gfx950 kernels. Every pointer is a device pointer; launches are asynchronous on
+// the given stream. The C-ABI layer (api.hip) validates shapes before calling any of these.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "device_common.h"
+
+namespace bg {
+
+// ---- GEMV ---------------------------------------------------------------------------------------
+struct GemvArgs {
+    const int8_t *W;     // packed weight: row-major [ALIGN(N,16)][ldw], rows zero-padded
+    uint32_t ldw;        // ALIGN(K, 8)
+    const uint8_t *x;    // [K]
+    uint32_t K, N;
+    const int32_t *ob;   // caller's offsetC (+ folded bias) [N]
+    const int32_t *comp; // -128 * sum_k W[n][k], stored behind the packed matrix [N]
+    void *y;
+    int add_yin;         // accumulate into the int32 bits already in y
+    Epilogue epi;
+};
+hipError_t launch_gemv_s8u8(const GemvArgs &a, hipStream_t st);
+hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const int8_t *x, uint32_t K, uint32_t M,
+    void *y, const Epilogue &epi, hipStream_t st);
+
+// ---- GEMM ---------------------------------------------------------------------------------------
+struct GemmArgs {
+    const uint8_t *A;    // u8 activations
+    uint32_t lda;        // bytes between consecutive m (transA = 0) or consecutive k (transA = 1)
+    int transA;          // 1: A stored [K][M]
+    const int8_t *Bp;    // packed right-hand side (fragment layout, see pack.hip)
+    uint32_t M, N, K;
+    const int32_t *ob;   // caller's offsetC (+ folded bias) [N]
+    const int32_t *comp; // blob's own compensation vector [N]
+    void *C;             // [M][N] row-major
+    int add_cin;         // accumulate into the int32 bits already in C
+    Epilogue epi;
+};
+hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
+
+// ---- weight pack --------------------------------------------------------------------------------
+// src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].
+hipError_t launch_pack_mmm(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t K, uint32_t N, int8_t *dst,
+    int32_t *comp, hipStream_t st);
+hipError_t launch_pack_mvm(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t K, uint32_t N, int8_t *dst,
+    int32_t *comp, hipStream_t st);
+
+// ---- quantize family ----------------------------------------------------------------------------
+// Device scratch word layout used by the two-pass kernels: ws[0] = max bits / max int.
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st);
+// Caller's scale = *ds_in (device) if given, else s_in. Dynamic when !mode or that scale <= 0:
+// the scale used is max(caller's, 127 / max|x|) with max|x| taken from ws[0]. The scale used is
+// written to *ds_out (device) when non-null.
+hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
+    const float *ds_in, int mode, float *ds_out, hipStream_t st);
+hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st);
+// s0 = output scale (< 0: dynamic from ws[0]), s1 = scale of the int32 data; the resulting output
+// scale is written to *ds_out (device) when non-null.
+hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s0,
+    float s1, float *ds_out, hipStream_t st);
+hipError_t launch_u8_to_i8(const uint8_t *x, uint32_t n, int8_t *q, hipStream_t st);
+hipError_t launch_dequant_i32(const int32_t *q, uint32_t n, const float *dscale, float scale, float *out,
+    hipStream_t st);
+hipError_t launch_dequant_u8(const uint8_t *q, uint32_t n, const float *dscale, float scale, float *out,
+    hipStream_t st);
+// out[n] = (int)round(bias[n] * s) + offsetC[n]; bias / offsetC may be null; s = scale or *dscaleA * scaleB
+hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *offsetC, const float *dscaleA,
+    float scaleB, int32_t *out, hipStream_t st);
+hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float rescale, int8_t *out, hipStream_t st);
+hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
+
+}  // namespace bg

@@ -1,0 +1,361 @@
+// HBM-bound element-wise kernels of the quantized path: per-tensor symmetric quantize
+// (fp32 -> u8 / s8), int32 -> u8 / s8 requantize, dequantize, bias fold, s8 rescale.
+// Numerics follow Bolt's AVX-512 kernels step by step
+// (compute/tensor/src/cpu/x86/int8/avx512/quantize.cpp, dequantize.cpp): every fp32 multiply and
+// add rounds separately (the translation unit is built with -ffp-contract=off), conversions are
+// round-to-nearest-even, narrowing saturates the way vpmovusdb / vpmovsdb do.
+//
+// Dynamic scales need the tensor-wide |max| before the map pass, so quantize is two launches:
+// a grid-stride reduction that folds into one device word with atomicMax (non-negative fp32
+// order like their bit patterns), then the map pass, in which every thread derives the scale
+// from that word. 16 elements per thread: 4 x 128-bit loads, one 128-bit store.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace bg {
+
+static inline uint32_t grid_for(uint32_t n, uint32_t per_thread, uint32_t block, uint32_t cap)
+{
+    uint64_t threads = ((uint64_t)n + per_thread - 1) / per_thread;
+    uint64_t blocks = (threads + block - 1) / block;
+    if (blocks < 1) {
+        blocks = 1;
+    }
+    if (blocks > cap) {
+        blocks = cap;
+    }
+    return (uint32_t)blocks;
+}
+
+__global__ void fill_u32_kernel(uint32_t *p, uint32_t n, uint32_t v)
+{
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st)
+{
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, n, v);
+    return hipGetLastError();
+}
+
+// ---- |max| reductions ---------------------------------------------------------------------------
+// avx512/quantize.cpp:21-68: sign bit cleared, vmaxps (a NaN never replaces the running max).
+template <int VEC>
+__global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict__ x, uint32_t n, uint32_t *ws)
+{
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    float m = 0.0f;
+    if (VEC) {
+        const uint32_t n4 = n / 4;
+        const v4f *x4 = (const v4f *)x;
+        for (uint32_t i = tid; i < n4; i += stride) {
+            v4f v = x4[i];
+            float a = fabsf(v.x), b = fabsf(v.y), c = fabsf(v.z), d = fabsf(v.w);
+            m = (a > m) ? a : m;
+            m = (b > m) ? b : m;
+            m = (c > m) ? c : m;
+            m = (d > m) ? d : m;
+        }
+        for (uint32_t i = n4 * 4 + tid; i < n; i += stride) {
+            float a = fabsf(x[i]);
+            m = (a > m) ? a : m;
+        }
+    } else {
+        for (uint32_t i = tid; i < n; i += stride) {
+            float a = fabsf(x[i]);
+            m = (a > m) ? a : m;
+        }
+    }
+    uint32_t bits = __float_as_uint(m);
+    bits = (uint32_t)wave_reduce_max_i((int)bits);  // non-negative floats: integer order == float order
+    if ((threadIdx.x & 63) == 0 && bits != 0) {
+        atomicMax(ws, bits);
+    }
+}
+
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st)
+{
+    hipError_t e = launch_fill_u32(ws, 1, 0, st);
+    if (e != hipSuccess || n == 0) {
+        return e;
+    }
+    const uint32_t blocks = grid_for(n, 16, 256, 2048);
+    if (((uintptr_t)x & 15) == 0) {
+        hipLaunchKernelGGL((absmax_f32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, ws);
+    } else {
+        hipLaunchKernelGGL((absmax_f32_kernel<0>), dim3(blocks), dim3(256), 0, st, x, n, ws);
+    }
+    return hipGetLastError();
+}
+
+// avx512/quantize.cpp:70-119: vpabsd + vpmaxsd, so |INT32_MIN| stays negative and never wins.
+__global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t *__restrict__ x, uint32_t n, uint32_t *ws)
+{
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    int m = 0;
+    for (uint32_t i = tid; i < n; i += stride) {
+        int v = x[i];
+        int a = (v == (int)0x80000000) ? v : (v < 0 ? -v : v);
+        m = (a > m) ? a : m;
+    }
+    m = wave_reduce_max_i(m);
+    if ((threadIdx.x & 63) == 0 && m != 0) {
+        atomicMax((int *)ws, m);
+    }
+}
+
+hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st)
+{
+    hipError_t e = launch_fill_u32(ws, 1, 0, st);
+    if (e != hipSuccess || n == 0) {
+        return e;
+    }
+    hipLaunchKernelGGL(absmax_i32_kernel, dim3(grid_for(n, 8, 256, 2048)), dim3(256), 0, st, x, n, ws);
+    return hipGetLastError();
+}
+
+// ---- fp32 -> u8 / s8 ----------------------------------------------------------------------------
+__device__ __forceinline__ unsigned q_u8(float x, float s)
+{
+    // avx512/quantize.cpp:150-155: vmulps, vaddps 128.0f, vcvtps2dq {rn}, clamp [1, 255]
+    float t = x * s;
+    float u = t + 128.0f;
+    int v = rne_i32(u);
+    v = v < 1 ? 1 : v;
+    v = v > 255 ? 255 : v;
+    return (unsigned)v;
+}
+
+__device__ __forceinline__ unsigned q_i8(float x, float s)
+{
+    // avx512/quantize.cpp:208-212: vmulps, vcvtps2dq, clamp [-127, 127]
+    int v = rne_i32(x * s);
+    v = v < -127 ? -127 : v;
+    v = v > 127 ? 127 : v;
+    return (unsigned)v & 0xffu;
+}
+
+template <int TO_U8>
+__device__ __forceinline__ unsigned q4(v4f v, float s)
+{
+    if (TO_U8) {
+        return q_u8(v.x, s) | (q_u8(v.y, s) << 8) | (q_u8(v.z, s) << 16) | (q_u8(v.w, s) << 24);
+    }
+    return q_i8(v.x, s) | (q_i8(v.y, s) << 8) | (q_i8(v.z, s) << 16) | (q_i8(v.w, s) << 24);
+}
+
+// avx512/quantize.cpp:129-133 / :189-193: dynamic when !mode or the caller's scale is <= 0;
+// the result is max(caller's scale, 127 / max|x|), with 127 / 0 replaced by 1.
+__device__ __forceinline__ float resolve_scale(float s_in, int mode, const uint32_t *ws)
+{
+    if (!mode || s_in <= 0) {
+        float m = __uint_as_float(ws[0]);
+        float dyn = (m == 0.0f) ? 1.0f : 127.0f / m;
+        return (s_in > dyn) ? s_in : dyn;
+    }
+    return s_in;
+}
+
+template <int TO_U8, int VEC>
+__global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restrict__ x, uint32_t n,
+    uint8_t *__restrict__ q, const uint32_t *__restrict__ ws, float s_in, const float *ds_in, int mode,
+    float *ds_out)  // ds_in may alias ds_out: the resolved scale is a fixed point of resolve_scale
+{
+    const float s = resolve_scale(ds_in ? *ds_in : s_in, mode, ws);
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid == 0 && ds_out) {
+        *ds_out = s;
+    }
+    const uint32_t stride = gridDim.x * blockDim.x;
+    if (VEC) {
+        const uint32_t n16 = n / 16;
+        const v4f *x4 = (const v4f *)x;
+        v4i *q16 = (v4i *)q;
+        for (uint32_t i = tid; i < n16; i += stride) {
+            v4f a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+            v4i o = {(int)q4<TO_U8>(a, s), (int)q4<TO_U8>(b, s), (int)q4<TO_U8>(c, s), (int)q4<TO_U8>(d, s)};
+            q16[i] = o;
+        }
+        for (uint32_t i = n16 * 16 + tid; i < n; i += stride) {
+            q[i] = (uint8_t)(TO_U8 ? q_u8(x[i], s) : q_i8(x[i], s));
+        }
+    } else {
+        for (uint32_t i = tid; i < n; i += stride) {
+            q[i] = (uint8_t)(TO_U8 ? q_u8(x[i], s) : q_i8(x[i], s));
+        }
+    }
+}
+
+hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
+    const float *ds_in, int mode, float *ds_out, hipStream_t st)
+{
+    const bool vec = (((uintptr_t)x | (uintptr_t)q) & 15) == 0;
+    const uint32_t blocks = grid_for(n, vec ? 16 : 1, 256, 8192);
+#define BG_LAUNCH_Q(U, V)                                                                                        \
+    hipLaunchKernelGGL((quantize_f32_kernel<U, V>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s_in, \
+        ds_in, mode, ds_out)
+    if (to_u8) {
+        if (vec) {
+            BG_LAUNCH_Q(1, 1);
+        } else {
+            BG_LAUNCH_Q(1, 0);
+        }
+    } else {
+        if (vec) {
+            BG_LAUNCH_Q(0, 1);
+        } else {
+            BG_LAUNCH_Q(0, 0);
+        }
+    }
+#undef BG_LAUNCH_Q
+    return hipGetLastError();
+}
+
+// ---- int32 -> u8 / s8 ---------------------------------------------------------------------------
+// avx512/quantize.cpp:315-361 (s8: ssat8(rne(cvt(x) * r))) and :364-416
+// (u8: usat8_u(rne(cvt(x) * r + 128.0f)), fp32 add before rounding).
+template <int TO_U8>
+__global__ __launch_bounds__(256) void requant_i32_kernel(const int32_t *__restrict__ x, uint32_t n,
+    uint8_t *__restrict__ q, const uint32_t *__restrict__ ws, float s0, float s1, float *__restrict__ ds_out)
+{
+    float r = 0.0f;
+    float out0 = s0;
+    if (s0 < 0 && s1 > 0) {
+        int m = (int)ws[0];
+        r = (m == 0) ? 1.0f : 127.0f / (float)m;
+        out0 = s1 * r;
+    } else if (s0 > 0 && s1 > 0) {
+        r = s0 / s1;
+    }
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid == 0 && ds_out) {
+        *ds_out = out0;
+    }
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = tid; i < n; i += stride) {
+        float t = (float)x[i] * r;
+        if (TO_U8) {
+            float u = t + 128.0f;
+            q[i] = (uint8_t)usat8_u(rne_i32(u));
+        } else {
+            q[i] = (uint8_t)ssat8(rne_i32(t));
+        }
+    }
+}
+
+hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s0,
+    float s1, float *ds_out, hipStream_t st)
+{
+    const uint32_t blocks = grid_for(n, 4, 256, 8192);
+    if (to_u8) {
+        hipLaunchKernelGGL((requant_i32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s0, s1,
+            ds_out);
+    } else {
+        hipLaunchKernelGGL((requant_i32_kernel<0>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s0, s1,
+            ds_out);
+    }
+    return hipGetLastError();
+}
+
+// avx512/quantize.cpp:271-313
+__global__ void u8_to_i8_kernel(const uint8_t *__restrict__ x, uint32_t n, int8_t *__restrict__ q)
+{
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        q[i] = (int8_t)(uint8_t)(x[i] + 0x80);
+    }
+}
+
+hipError_t launch_u8_to_i8(const uint8_t *x, uint32_t n, int8_t *q, hipStream_t st)
+{
+    hipLaunchKernelGGL(u8_to_i8_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, x, n, q);
+    return hipGetLastError();
+}
+
+// ---- dequantize: avx512/dequantize.cpp:18-101, f = cvt(q) * (1 / s) -----------------------------
+__global__ void dequant_i32_kernel(const int32_t *__restrict__ q, uint32_t n, const float *__restrict__ ds, float s,
+    float *__restrict__ out)
+{
+    const float f = 1 / (ds ? *ds : s);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        out[i] = (float)q[i] * f;
+    }
+}
+
+__global__ void dequant_u8_kernel(const uint8_t *__restrict__ q, uint32_t n, const float *__restrict__ ds, float s,
+    float *__restrict__ out)
+{
+    const float f = 1 / (ds ? *ds : s);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        out[i] = (float)((int)q[i] - 128) * f;
+    }
+}
+
+hipError_t launch_dequant_i32(const int32_t *q, uint32_t n, const float *ds, float s, float *out, hipStream_t st)
+{
+    hipLaunchKernelGGL(dequant_i32_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, q, n, ds, s, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_u8(const uint8_t *q, uint32_t n, const float *ds, float s, float *out, hipStream_t st)
+{
+    hipLaunchKernelGGL(dequant_u8_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, q, n, ds, s, out);
+    return hipGetLastError();
+}
+
+// ---- bias fold: avx512/quantize.cpp:236-269 -----------------------------------------------------
+// out[n] = (I32)(round(bias[n] * s) + offsetC[n]); round() is half away from zero.
+__global__ void bias_offsetC_kernel(const float *__restrict__ bias, uint32_t N, const int32_t *__restrict__ offsetC,
+    const float *__restrict__ dsA, float sB, int32_t *__restrict__ out)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N) {
+        return;
+    }
+    if (!bias) {
+        out[i] = offsetC ? offsetC[i] : 0;
+        return;
+    }
+    const float s = dsA ? (*dsA * sB) : sB;
+    float p = bias[i] * s;
+    double r = round((double)p);
+    if (offsetC) {
+        r += (double)offsetC[i];
+    }
+    out[i] = (int32_t)r;
+}
+
+hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *offsetC, const float *dsA, float sB,
+    int32_t *out, hipStream_t st)
+{
+    if (N == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(bias_offsetC_kernel, dim3((N + 255) / 256), dim3(256), 0, st, bias, N, offsetC, dsA, sB, out);
+    return hipGetLastError();
+}
+
+// ---- s8 rescale: compute/tensor/src/cpu/requantize.cpp:20-50 ------------------------------------
+__global__ void requantize_i8_kernel(const int8_t *__restrict__ in, uint32_t n, float r, int8_t *__restrict__ out)
+{
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float v = r * (float)in[i] + 0.0f;
+        out[i] = (int8_t)(int)v;
+    }
+}
+
+hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float r, int8_t *out, hipStream_t st)
+{
+    hipLaunchKernelGGL(requantize_i8_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, in, n, r, out);
+    return hipGetLastError();
+}
+
+}  // namespace bg

@@ -1,0 +1,104 @@
+/*
+ * C-ABI of libbolt_gfx950.so -- the MI355X (gfx950) implementation of Bolt's quantized
+ * matrix-product path. Plain pointers, sizes and Bolt's own POD records only.
+ *
+ * Every function that replaces a Bolt function keeps that function's argument list and
+ * meaning, with the `_gfx950` suffix Bolt's per-architecture back ends use (`_x86`, `_arm`);
+ * the comment above each declaration names the interface it replaces. `arch` selects the
+ * pointer convention:
+ *   AMD_GFX950         all data pointers are HOST pointers; the call stages operands to the
+ *                      GPU, runs, copies results back and returns when they are in place.
+ *   AMD_GFX950_DEVICE  all data pointers (matrices, vectors, tmp, results) are DEVICE pointers,
+ *                      4-byte aligned; work is enqueued on the library stream and the call
+ *                      returns without waiting. TensorDesc and `scale` arguments stay on the host.
+ * Errors come back as Bolt's EE codes; nothing here calls exit().
+ */
+#ifndef BOLT_GFX950_H
+#define BOLT_GFX950_H
+
+#include "bolt_types.h"
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- runtime ------------------------------------------------------------------------- */
+/* No counterpart in the reference (a CPU library needs no device context). */
+EE bolt_gfx950_init(void);
+/* stream: a hipStream_t (NULL = the default stream). The library never creates streams. */
+EE bolt_gfx950_set_stream(void *stream);
+EE bolt_gfx950_synchronize(void);
+const char *bolt_gfx950_last_error(void);
+void *bolt_gfx950_malloc(size_t bytes);
+void bolt_gfx950_free(void *dptr);
+EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes);
+EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes);
+/* Event pair on the library stream; stop returns the elapsed milliseconds after waiting. */
+EE bolt_gfx950_timer_start(void);
+EE bolt_gfx950_timer_stop(float *ms);
+
+/* ---- blas_enhance: int8 GEMM --------------------------------------------------------- */
+/* compute/blas_enhance/include/blas_enhance.h:36-37  matrix_matrix_multiply_tmp_bytes */
+EE matrix_matrix_multiply_tmp_bytes_gfx950(TensorDesc matrixADesc, TensorDesc matrixBDesc, U32 *bytes, Arch arch);
+/* blas_enhance.h:39-48  matrix_matrix_multiply
+ * C = C_in + offsetC + A(u8) x B(s8); the first N int32 of `tmp` are offsetC (+ folded bias);
+ * scale: NULL -> int32, scale[0] > 0 -> fp32 * (1/scale[0]), scale[0] < 0 -> u8 with scale[1]. */
+EE matrix_matrix_multiply_gfx950(TensorDesc matrixADesc, const void *matrixA, TensorDesc matrixBDesc,
+    const void *matrixB, U32 bytes, void *tmp, TensorDesc matrixCDesc, void *matrixC, const F32 *scale, Arch arch);
+/* blas_enhance.h:67  matrix_matrix_multiply_rhs_format */
+DataFormat matrix_matrix_multiply_rhs_format_gfx950(DataType dt);
+/* blas_enhance.h:70  matrix_matrix_multiply_transform_rhs_bytes */
+EE matrix_matrix_multiply_transform_rhs_bytes_gfx950(TensorDesc desc, U32 *bytes, U32 *rhsBytes, Arch arch);
+/* blas_enhance.h:73-74  matrix_matrix_multiply_transform_rhs */
+EE matrix_matrix_multiply_transform_rhs_gfx950(TensorDesc desc, const void *src, TensorDesc *descTran, void *dst,
+    Arch arch);
+
+/* ---- blas_enhance: int8 GEMV --------------------------------------------------------- */
+/* blas_enhance.h:55  matrix_vector_multiply_tmp_bytes */
+EE matrix_vector_multiply_tmp_bytes_gfx950(TensorDesc matrixDesc, TensorDesc vectorDesc, U32 *bytes, Arch arch);
+/* blas_enhance.h:57-66  matrix_vector_multiply */
+EE matrix_vector_multiply_gfx950(TensorDesc matrixDesc, const void *matrix, TensorDesc vectorDesc, const void *vector,
+    U32 bytes, void *tmp, TensorDesc resultDesc, void *result, const F32 *scale, Arch arch);
+/* blas_enhance.h:77  matrix_vector_multiply_weight_format */
+DataFormat matrix_vector_multiply_weight_format_gfx950(DataType dt);
+/* blas_enhance.h:79  matrix_vector_multiply_transform_weight_bytes */
+EE matrix_vector_multiply_transform_weight_bytes_gfx950(TensorDesc desc, U32 *bytes, Arch arch);
+/* blas_enhance.h:82-83  matrix_vector_multiply_transform_weight */
+EE matrix_vector_multiply_transform_weight_gfx950(TensorDesc desc, const void *src, TensorDesc *descTran, void *dst,
+    Arch arch);
+
+/* ---- tensor_computing: quantize / dequantize / requantize ---------------------------- */
+/* compute/tensor/src/cpu/x86/quantize.cpp:19  quantize_x86 (reached from quantize(),
+ * compute/tensor/src/quantize.cpp:19-34). F32 -> {I8, U8_Q}, U8_Q -> I8, I32 -> {I8, U8_Q}.
+ * `scale` is a host pointer, read and written as the reference does. */
+EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *qData, F32 *scale, int mode,
+    Arch arch);
+/* compute/tensor/src/cpu/x86/dequantize.cpp:19  dequantize_x86 (bias ignored, as on x86). */
+EE dequantize_gfx950(TensorDesc qDesc, void *qData, const F32 *scale, TensorDesc bDesc, void *bData,
+    TensorDesc dDesc, void *dData, Arch arch);
+/* compute/tensor/src/cpu/x86/quantize.cpp:64  quantize_bias_offsetC */
+EE quantize_bias_offsetC_gfx950(const void *bias, TensorDesc biasDesc, DataType qType, const void *filter,
+    TensorDesc filterDesc, const F32 *scale, void *offsetCBias, Arch arch);
+/* compute/tensor/src/cpu/requantize.cpp:20  requantize_cpu */
+EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDesc outputDesc, INT8 *output,
+    F32 outputScale, Arch arch);
+
+/* ---- asynchronous forms with device-resident scales (AMD_GFX950_DEVICE only) -------- */
+/* No counterpart in the reference: Bolt keeps a tensor's scale in host memory
+ * (common/memory/include/tensor.hpp:83-96). These keep it on the GPU so that
+ * quantize -> GEMM -> dequantize chains never wait for the host.
+ *   quantize: *dscale (device, in/out) plays the role of `scale` in quantize_gfx950.
+ *   GEMM/GEMV: fp32 out[m][n] = cvt(acc) * (1.0f / (*dscaleI * scaleW[n])) + bias[n], with
+ *   per-output-channel weight scales scaleW[N] and optional fp32 bias[N] (both device);
+ *   reduces to the per-tensor reference epilogue when every scaleW[n] is equal and bias is NULL. */
+EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode);
+EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
+    float *C, const float *dscaleI, const float *scaleW, const float *bias);
+EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void *x, const I32 *offsetC, float *y,
+    const float *dscaleI, const float *scaleW, const float *bias);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

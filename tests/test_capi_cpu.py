@@ -1,0 +1,150 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every declared symbol, the
+size queries reproduce the reference's formulas, the host-pointer weight transform produces the
+observable contract (blob size, offsetC position and value, transformed descriptor), and argument
+validation returns the reference's EE codes."""
+import ctypes as C
+import itertools
+import os
+import re
+
+import numpy as np
+import pytest
+
+from bolt_amd import capi, host
+from bolt_amd.capi import (AMD_GFX950, DF_NKN32K4, DF_NKNxKx, DF_NORMAL, DF_TRANSPOSE, DT_F32, DT_I8, DT_I32, DT_U8_Q,
+                           tensor1d, tensor2df)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = capi.lib()
+    header = open(os.path.join(ROOT, "include", "bolt_gfx950.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*_gfx950|bolt_gfx950_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(L, name), name
+    assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
+
+
+def test_tensor_desc_layout():
+    d = tensor2df(DT_I8, DF_TRANSPOSE, 3, 5)
+    assert C.sizeof(d) == 92 and d.nDims == 2 and d.dims[0] == 5 and d.dims[1] == 3
+    raw = bytes(d)
+    assert raw[:12] == np.array([1, 13, 2], np.uint32).tobytes()
+
+
+def test_size_queries_match_oracle(oracle):
+    for N, K in itertools.product([1, 7, 16, 17, 48, 100, 1024, 3072], [1, 7, 8, 9, 77, 768, 4097]):
+        for df in (DF_NORMAL, DF_TRANSPOSE):
+            assert host.mmm_transform_rhs_bytes(host.rhs_desc(df, K, N)) == oracle.mmm_transform_rhs_bytes(N, K)
+            assert host.mvm_transform_weight_bytes(host.mvm_desc(df, N, K)) == oracle.mvm_transform_weight_bytes(N, K)
+        assert host.mmm_transform_rhs_bytes(host.rhs_desc(DF_NKNxKx, K, N)) == (0, 0)
+        assert host.mvm_transform_weight_bytes(host.mvm_desc(DF_NKN32K4, N, K)) == N * 4
+        assert host.mvm_tmp_bytes(host.mvm_desc(DF_NKN32K4, N, K), tensor1d(DT_U8_Q, K)) == N * 4
+        assert host.mvm_transform_weight_bytes(host.mvm_desc(DF_NORMAL, N, K, DT_U8_Q)) == \
+            oracle.mvm_transform_weight_bytes(N, K, DT_U8_Q)
+        for M, tA, pk in itertools.product([1, 5, 24, 25, 64, 385], [False, True], [False, True]):
+            ad = tensor2df(DT_U8_Q, DF_TRANSPOSE, K, M) if tA else tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+            bd = host.rhs_desc(DF_NKNxKx if pk else DF_TRANSPOSE, K, N)
+            assert host.mmm_tmp_bytes(ad, bd) == oracle.mmm_tmp_bytes(N, M, K, tA, pk)
+    assert host.mmm_transform_rhs_bytes(host.rhs_desc(DF_TRANSPOSE, 1024, 1024)) == (1052736, 1048576)
+    assert host.mvm_transform_weight_bytes(host.mvm_desc(DF_NORMAL, 4096, 4096)) == 16793632
+
+
+def mmm_unpack(blob, N, K):
+    """Independent restatement of the fragment layout: 16-column blocks of 16*Kp bytes, each holding
+    Kp//16 fragments [n16][k16] and, when Kp % 16 == 8, one [n16][k8] fragment."""
+    Kp, N16 = (K + 7) // 8 * 8, (N + 15) // 16 * 16
+    out = np.zeros((N16, Kp), np.int8)
+    b = blob[:N16 * Kp].view(np.int8).reshape(N16 // 16, 16 * Kp)
+    full = Kp // 16
+    for nb in range(N16 // 16):
+        if full:
+            frag = b[nb, :full * 256].reshape(full, 16, 16)          # [kb][n][k]
+            out[nb * 16:(nb + 1) * 16, :full * 16] = frag.transpose(1, 0, 2).reshape(16, full * 16)
+        if Kp % 16:
+            out[nb * 16:(nb + 1) * 16, full * 16:] = b[nb, full * 256:].reshape(16, 8)
+    return out
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (16, 16), (17, 9), (48, 64), (100, 77), (33, 24), (64, 4104)])
+def test_host_weight_transform_contract(oracle, N, K):
+    rng = np.random.default_rng(N * 131 + K)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    want_off = oracle.offsetC(W, True)
+    Kp, N16 = (K + 7) // 8 * 8, (N + 15) // 16 * 16
+    for df, src in ((DF_TRANSPOSE, W), (DF_NORMAL, np.ascontiguousarray(W.T))):
+        blob, dt, rhs = host.mmm_transform_rhs(src, df, K, N)
+        assert rhs == N16 * Kp and blob.size == rhs + 4 * N + 64
+        assert (dt.dt, dt.df, dt.nDims, dt.dims[0], dt.dims[1]) == (DT_I8, DF_NKNxKx, 2, N, K)
+        assert np.array_equal(blob[rhs:rhs + 4 * N].view(np.int32), want_off)
+        full = mmm_unpack(blob, N, K)
+        assert np.array_equal(full[:N, :K], W) and not full[N:].any() and not full[:, K:].any()
+    for df, src in ((DF_NORMAL, W), (DF_TRANSPOSE, np.ascontiguousarray(W.T))):
+        blob, dt = host.mvm_transform_weight(src, df, N, K)
+        assert blob.size == 4 * N + N16 * Kp + 32
+        assert (dt.dt, dt.df, dt.nDims, dt.dims[0], dt.dims[1]) == (DT_I8, DF_NKN32K4, 2, K, N)
+        assert np.array_equal(blob[N16 * Kp:N16 * Kp + 4 * N].view(np.int32), want_off)
+        full = blob[:N16 * Kp].view(np.int8).reshape(N16, Kp)
+        assert np.array_equal(full[:N, :K], W) and not full[N:].any() and not full[:, K:].any()
+
+
+def test_transform_of_packed_input_is_a_no_op():
+    L = capi.lib()
+    dt = capi.TensorDesc()
+    dt.df = 1234
+    dst = np.full(8, 7, np.uint8)
+    src = np.zeros(8, np.int8)
+    assert L.matrix_matrix_multiply_transform_rhs_gfx950(host.rhs_desc(DF_NKNxKx, 2, 2), host.ptr(src), C.byref(dt),
+                                                        host.ptr(dst), AMD_GFX950) == capi.SUCCESS
+    assert L.matrix_vector_multiply_transform_weight_gfx950(host.mvm_desc(DF_NKN32K4, 2, 2), host.ptr(src), C.byref(dt),
+                                                           host.ptr(dst), AMD_GFX950) == capi.SUCCESS
+    assert dt.df == 1234 and (dst == 7).all()
+
+
+def test_error_codes_follow_the_reference():
+    L = capi.lib()
+    a = np.zeros((4, 8), np.uint8)
+    b = np.zeros(16 * 8 + 64 + 4 * 4, np.int8)
+    c = np.zeros((4, 4), np.int32)
+    tmp = np.zeros(1024, np.uint8)
+    ad, bd, cd = tensor2df(DT_U8_Q, DF_NORMAL, 4, 8), host.rhs_desc(DF_NKNxKx, 8, 4), tensor2df(DT_I32, DF_NORMAL, 4, 4)
+    mm = L.matrix_matrix_multiply_gfx950
+    # unknown arch -> NOT_SUPPORTED without touching anything (mmm.cpp:199,237)
+    assert mm(ad, host.ptr(a), bd, host.ptr(b), 1024, host.ptr(tmp), cd, host.ptr(c), None, capi.X86_AVX512) == \
+        capi.NOT_SUPPORTED
+    # null operands / tmp missing while bytes != 0 -> NULL_POINTER (mmm.cpp:161-166)
+    assert mm(ad, None, bd, host.ptr(b), 1024, host.ptr(tmp), cd, host.ptr(c), None, AMD_GFX950) == capi.NULL_POINTER
+    assert mm(ad, host.ptr(a), bd, host.ptr(b), 1024, None, cd, host.ptr(c), None, AMD_GFX950) == capi.NULL_POINTER
+    # empty C -> SUCCESS early (mmm.cpp:167-169)
+    assert mm(ad, host.ptr(a), bd, host.ptr(b), 1024, host.ptr(tmp), tensor2df(DT_I32, DF_NORMAL, 0, 4), host.ptr(c),
+              None, AMD_GFX950) == capi.SUCCESS
+    # shape / dtype mismatch -> NOT_MATCH (mmm.cpp:181-197)
+    assert mm(ad, host.ptr(a), bd, host.ptr(b), 1024, host.ptr(tmp), tensor2df(DT_I32, DF_NORMAL, 4, 5), host.ptr(c),
+              None, AMD_GFX950) == capi.NOT_MATCH
+    assert mm(tensor2df(DT_F32, DF_NORMAL, 4, 8), host.ptr(a), bd, host.ptr(b), 1024, host.ptr(tmp), cd, host.ptr(c),
+              None, AMD_GFX950) == capi.NOT_MATCH
+    assert mm(tensor1d(DT_U8_Q, 8), host.ptr(a), bd, host.ptr(b), 1024, host.ptr(tmp), cd, host.ptr(c), None,
+              AMD_GFX950) == capi.NOT_MATCH
+    mv = L.matrix_vector_multiply_gfx950
+    x = np.zeros(8, np.uint8)
+    y = np.zeros(4, np.int32)
+    md = host.mvm_desc(DF_NKN32K4, 4, 8)
+    assert mv(md, host.ptr(b), tensor1d(DT_U8_Q, 8), None, 1024, host.ptr(tmp), tensor1d(DT_I32, 4), host.ptr(y), None,
+              AMD_GFX950) == capi.NULL_POINTER
+    assert mv(md, host.ptr(b), tensor1d(DT_U8_Q, 9), host.ptr(x), 1024, host.ptr(tmp), tensor1d(DT_I32, 4), host.ptr(y),
+              None, AMD_GFX950) == capi.NOT_MATCH
+    # u8 matrix tagged DF_NK is refused (mvm.cpp:172-175)
+    assert mv(tensor2df(DT_U8_Q, capi.DF_NK, 4, 8), host.ptr(b), tensor1d(DT_I8, 8), host.ptr(x), 1024, host.ptr(tmp),
+              tensor1d(DT_I32, 4), host.ptr(y), None, AMD_GFX950) == capi.NOT_SUPPORTED
+    # quantize without a scale pointer -> NOT_MATCH (avx512/quantize.cpp:123-125)
+    qd = tensor1d(DT_U8_Q, 8)
+    f = np.zeros(8, np.float32)
+    assert L.quantize_gfx950(tensor1d(DT_F32, 8), host.ptr(f), C.byref(qd), host.ptr(x), None, 0, AMD_GFX950) == \
+        capi.NOT_MATCH
+    qd2 = tensor1d(DT_I32, 8)
+    s = (C.c_float * 2)(1, 1)
+    assert L.quantize_gfx950(tensor1d(DT_F32, 8), host.ptr(f), C.byref(qd2), host.ptr(x), C.cast(s, C.c_void_p), 0,
+                             AMD_GFX950) == capi.NOT_SUPPORTED

@@ -1,0 +1,274 @@
+"""GPU parity tests for the int8 GEMM / GEMV C-ABI against the CPU oracle: bit-exact int32, u8 and
+fp32 outputs (fp32 is a single multiply of an exact int32 conversion, so it is compared bit for bit,
+stricter than the 1e-6 relative the path asks for). Both pointer conventions are exercised:
+numpy buffers (host pointers, AMD_GFX950) and torch CUDA tensors (device pointers,
+AMD_GFX950_DEVICE)."""
+import itertools
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from bolt_amd import capi, host  # noqa: E402
+from bolt_amd.capi import (DF_NKN32K4, DF_NKNxKx, DF_NORMAL, DF_TRANSPOSE, DT_F32, DT_I8, DT_I32, DT_U8_Q, tensor1d,
+                           tensor2df)  # noqa: E402
+
+EDGE = [1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65]
+NP_OF = {DT_I32: np.int32, DT_F32: np.float32, DT_U8_Q: np.uint8}
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def torch_mod():
+    import torch
+    assert torch.cuda.is_available()
+    capi.check(capi.lib().bolt_gfx950_init(), "init")
+    return torch
+
+
+def dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run_mmm(torch, device_mode, A, adf, B, bdf, M, K, N, offsetC, Cin, cdt, scale):
+    """Reference call order: tmp bytes -> offsetC at the head of tmp -> multiply."""
+    ad = tensor2df(DT_U8_Q, DF_TRANSPOSE, K, M) if adf == DF_TRANSPOSE else tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+    bd = host.rhs_desc(bdf, K, N)
+    tmpBytes = host.mmm_tmp_bytes(ad, bd) + M * N * 4
+    tmp = np.zeros(tmpBytes, np.uint8)
+    if offsetC is not None:
+        tmp[:4 * N] = np.ascontiguousarray(offsetC, dtype=np.int32).view(np.uint8)
+    Cbuf = np.array(Cin, dtype=NP_OF[cdt]).reshape(M, N).copy()
+    cd = tensor2df(cdt, DF_NORMAL, M, N)
+    if device_mode:
+        dA, dB, dT, dC = dev(torch, A), B if hasattr(B, "data_ptr") else dev(torch, B), dev(torch, tmp), dev(torch, Cbuf)
+        e = host.matrix_matrix_multiply(dA, ad, dB, bd, dT, dC, cd, scale)
+        capi.check(e, "mmm")
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        return dC.cpu().numpy()
+    Bh = B.cpu().numpy() if hasattr(B, "data_ptr") else B
+    e = host.matrix_matrix_multiply(np.ascontiguousarray(A), ad, np.ascontiguousarray(Bh), bd, tmp, Cbuf, cd, scale)
+    capi.check(e, "mmm")
+    return Cbuf
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+@pytest.mark.parametrize("bfmt", ["packed", "normal", "transpose"])
+@pytest.mark.parametrize("transA", [False, True])
+def test_mmm_i32_edges(torch_mod, oracle, device_mode, bfmt, transA):
+    rng = np.random.default_rng(17 + device_mode + 2 * transA)
+    shapes = list(itertools.product(EDGE, [1, 7, 8, 9, 16, 33, 64, 65, 130], EDGE))
+    step = 23 if not device_mode else 7
+    say("mmm i32 edges", device_mode, bfmt, transA, len(shapes[::step]))
+    for M, K, N in shapes[::step]:
+        A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+        W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+        Cin = rng.integers(-1000, 1000, size=(M, N), dtype=np.int32)
+        off = oracle.offsetC(W, True)
+        Aarg = np.ascontiguousarray(A.T) if transA else A
+        adf = DF_TRANSPOSE if transA else DF_NORMAL
+        if bfmt == "packed":
+            blob, dt, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            offb = off + rng.integers(-9999, 9999, size=N, dtype=np.int32)   # caller-folded bias
+            got = run_mmm(torch_mod, device_mode, Aarg, adf, blob, DF_NKNxKx, M, K, N, offb, Cin, DT_I32, None)
+            want = oracle.mmm(Aarg, W, offb, Cin, DT_I32, transA=transA)
+        elif bfmt == "transpose":
+            got = run_mmm(torch_mod, device_mode, Aarg, adf, W, DF_TRANSPOSE, M, K, N, None, Cin, DT_I32, None)
+            want = oracle.mmm(Aarg, W, off, Cin, DT_I32, transA=transA)
+        else:
+            got = run_mmm(torch_mod, device_mode, Aarg, adf, np.ascontiguousarray(W.T), DF_NORMAL, M, K, N, None, Cin,
+                          DT_I32, None)
+            want = oracle.mmm(Aarg, W, off, Cin, DT_I32, transA=transA)
+        assert np.array_equal(got, want), (M, K, N)
+
+
+@pytest.mark.parametrize("M,K,N", [(3, 4095, 48), (5, 4097, 50), (2, 8200, 17), (385, 9, 49), (64, 1024, 1024),
+                                   (128, 768, 768), (200, 136, 264)])
+def test_mmm_all_outputs_device(torch_mod, oracle, M, K, N):
+    say("mmm outputs", M, K, N)
+    rng = np.random.default_rng(M * 7 + K)
+    A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    off = oracle.offsetC(W, True) + rng.integers(-5000, 5000, size=N, dtype=np.int32)
+    blob, dt, rhs = host.mmm_transform_rhs(dev(torch_mod, W), DF_TRANSPOSE, K, N)   # device-side pack kernel
+    hblob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)                     # host-side pack
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    assert np.array_equal(blob.cpu().numpy()[:rhs + 4 * N], hblob[:rhs + 4 * N])
+    Cin = rng.integers(-99, 99, size=(M, N), dtype=np.int32)
+    got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, Cin, DT_I32, None)
+    assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
+    s = np.float32(37.25)
+    z = np.zeros((M, N), np.float32)
+    got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, z, DT_F32, [s])
+    want = oracle.mmm(A, W, off, z, DT_F32, scale=[s])
+    assert np.array_equal(got.view(np.int32), want.view(np.int32))
+    acc = oracle.mmm(A, W, off, np.zeros((M, N), np.int32), DT_I32)
+    r = np.float32(127.0 / max(1, np.abs(acc).max()))
+    zu = np.zeros((M, N), np.uint8)
+    got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, zu, DT_U8_Q, [-1, r])
+    assert np.array_equal(got, oracle.mmm(A, W, off, zu, DT_U8_Q, scale=[-1, r]))
+    # DT_I32 output ignores a scale pointer (mmm.cpp:222-224)
+    got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, Cin, DT_I32, [s])
+    assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
+
+
+def test_mmm_u8_epilogue_ties_and_saturation(torch_mod, oracle):
+    M, K, N = 16, 8, 16
+    A = np.full((M, K), 128, np.uint8)
+    W = np.zeros((N, K), np.int8)
+    blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+    accs = np.array([524289, 524288, 1572864, -524288, 1, -1, 0, 300 << 20, -(140 << 20), -(129 << 20),
+                     -(128 << 20) - (1 << 19), 127 << 20, (127 << 20) + (1 << 19), 255 << 20, -(1 << 31),
+                     (1 << 31) - 1], np.int64).astype(np.int32)
+    r = np.float32(2.0 ** -20)
+    zu = np.zeros((M, N), np.uint8)
+    for mode in (False, True):
+        got = run_mmm(torch_mod, mode, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, accs, zu, DT_U8_Q, [-1, r])
+        assert np.array_equal(got, oracle.mmm(A, W, accs, zu, DT_U8_Q, scale=[-1, r]))
+        assert got[0, 0] == 129 and got[0, 8] == 255 and got[0, 7] == 255
+
+
+def run_mvm(torch, device_mode, W, mdesc, x, N, K, offsetC, yin, scale, vdt=DT_U8_Q, ydt=DT_I32):
+    tmpBytes = host.mvm_tmp_bytes(mdesc, tensor1d(vdt, K)) + 2 * N * 4 + N * K + 64
+    tmp = np.zeros(tmpBytes, np.uint8)
+    if offsetC is not None:
+        tmp[:4 * N] = np.ascontiguousarray(offsetC, dtype=np.int32).view(np.uint8)
+    y = np.array(yin, dtype=NP_OF[ydt]).reshape(N).copy()
+    vd, rd = tensor1d(vdt, K), tensor1d(ydt, N)
+    if device_mode:
+        dW = W if hasattr(W, "data_ptr") else dev(torch, W)
+        dx, dT, dy = dev(torch, x), dev(torch, tmp), dev(torch, y)
+        capi.check(host.matrix_vector_multiply(dW, mdesc, dx, vd, dT, dy, rd, scale), "mvm")
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        return dy.cpu().numpy()
+    Wh = W.cpu().numpy() if hasattr(W, "data_ptr") else np.ascontiguousarray(W)
+    capi.check(host.matrix_vector_multiply(Wh, mdesc, np.ascontiguousarray(x), vd, tmp, y, rd, scale), "mvm")
+    return y
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+@pytest.mark.parametrize("wfmt", ["packed", "normal", "transpose"])
+def test_mvm_edges(torch_mod, oracle, device_mode, wfmt):
+    rng = np.random.default_rng(7 + device_mode)
+    Ns = [1, 2, 3, 7, 8, 9, 15, 16, 17, 31, 33, 63, 64, 65, 100, 200]
+    Ks = [1, 2, 3, 4, 7, 8, 9, 15, 16, 17, 77, 1023, 1024, 1025, 2049, 4100]
+    combos = list(itertools.product(Ns, Ks))[::(1 if device_mode else 3)]
+    say("mvm edges", device_mode, wfmt, len(combos))
+    for N, K in combos:
+        W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+        x = rng.integers(0, 256, size=K, dtype=np.uint8)
+        yin = rng.integers(-500, 500, size=N, dtype=np.int32)
+        if wfmt == "packed":
+            blob, dt = host.mvm_transform_weight(W, DF_NORMAL, N, K)
+            off = oracle.offsetC(W, True) + rng.integers(-3000, 3000, size=N, dtype=np.int32)
+            args = (blob, host.mvm_desc(DF_NKN32K4, N, K), x, N, K, off)
+        elif wfmt == "normal":
+            off = oracle.offsetC(W, True)
+            args = (W, host.mvm_desc(DF_NORMAL, N, K), x, N, K, None)
+        else:
+            off = oracle.offsetC(W, True)
+            args = (np.ascontiguousarray(W.T), host.mvm_desc(DF_TRANSPOSE, N, K), x, N, K, None)
+        got = run_mvm(torch_mod, device_mode, *args, yin, None)
+        assert np.array_equal(got, oracle.mvm(W, x, off, yin, DT_I32)), (N, K)
+        s = np.float32(11.5)
+        z = np.zeros(N, np.float32)
+        got = run_mvm(torch_mod, device_mode, *args, z, [s], ydt=DT_F32)
+        assert np.array_equal(got.view(np.int32), oracle.mvm(W, x, off, z, DT_F32, scale=[s]).view(np.int32)), (N, K)
+        if wfmt == "packed":   # u8 output is defined on the pre-packed route only (see test_oracle_vs_ref)
+            r = np.float32(0.004)
+            zu = np.zeros(N, np.uint8)
+            got = run_mvm(torch_mod, device_mode, *args, zu, [-1, r], ydt=DT_U8_Q)
+            assert np.array_equal(got, oracle.mvm(W, x, off, zu, DT_U8_Q, scale=[-1, r])), (N, K)
+
+
+def test_mvm_decode_shape_and_device_pack(torch_mod, oracle):
+    rng = np.random.default_rng(4096)
+    N = K = 4096
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    blob, dt = host.mvm_transform_weight(dev(torch_mod, W), DF_NORMAL, N, K)
+    off = oracle.offsetC(W, True)
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    assert np.array_equal(blob.cpu().numpy()[N * K:N * K + 4 * N].view(np.int32), off)
+    for seed in range(4):
+        x = np.random.default_rng(seed).integers(0, 256, size=K, dtype=np.uint8)
+        z = np.zeros(N, np.int32)
+        got = run_mvm(torch_mod, True, blob, host.mvm_desc(DF_NKN32K4, N, K), x, N, K, off, z, None)
+        assert np.array_equal(got, oracle.mvm(W, x, off, z, DT_I32))
+        # misaligned activation vector (byte-granular path)
+        xx = dev(torch_mod, np.concatenate([[0], x]).astype(np.uint8))[1:]
+        tmp = dev(torch_mod, off)
+        y = torch_mod.zeros(N, dtype=torch_mod.int32, device="cuda")
+        capi.check(host.matrix_vector_multiply(blob, host.mvm_desc(DF_NKN32K4, N, K), xx, tensor1d(DT_U8_Q, K),
+                                               tmp.view(torch_mod.uint8), y, tensor1d(DT_I32, N), None), "mvm")
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        assert np.array_equal(y.cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_mvm_u8_matrix_s8_vector(torch_mod, oracle, device_mode):
+    rng = np.random.default_rng(9)
+    for M, K in itertools.product([1, 3, 4, 5, 8, 9, 17, 40], [1, 15, 16, 17, 63, 64, 65, 300]):
+        A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+        x = rng.integers(-127, 128, size=K, dtype=np.int8)
+        yin = rng.integers(-500, 500, size=M, dtype=np.int32)
+        got = run_mvm(torch_mod, device_mode, A, host.mvm_desc(DF_NORMAL, M, K, DT_U8_Q), x, M, K, None, yin, None,
+                      vdt=DT_I8)
+        assert np.array_equal(got, oracle.mvm_u8mat(A, x, yin, DT_I32)), (M, K)
+        At = np.ascontiguousarray(A.T)
+        got = run_mvm(torch_mod, device_mode, At, host.mvm_desc(DF_TRANSPOSE, M, K, DT_U8_Q), x, M, K, None, yin, None,
+                      vdt=DT_I8)
+        assert np.array_equal(got, oracle.mvm_u8mat(At, x, yin, DT_I32, a_is_KM=True)), (M, K)
+        s = np.float32(3.0)
+        z = np.zeros(M, np.float32)
+        got = run_mvm(torch_mod, device_mode, A, host.mvm_desc(DF_NORMAL, M, K, DT_U8_Q), x, M, K, None, z, [s],
+                      vdt=DT_I8, ydt=DT_F32)
+        assert np.array_equal(got.view(np.int32), oracle.mvm_u8mat(A, x, z, DT_F32, scale=[s]).view(np.int32))
+
+
+def test_per_channel_epilogue(torch_mod, oracle):
+    """Per-output-channel weight scales + fp32 bias (not in the reference): closed form, and reduction
+    to the reference's per-tensor result when all channel scales are equal."""
+    torch = torch_mod
+    rng = np.random.default_rng(5)
+    L = capi.lib()
+    for M, K, N in [(1, 256, 96), (7, 100, 33), (64, 1024, 1024)]:
+        A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+        W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+        off = oracle.offsetC(W, True)
+        acc = oracle.mmm(A, W, off, np.zeros((M, N), np.int32), DT_I32)
+        sI = np.float32(31.75)
+        sW = (1.0 / rng.uniform(0.005, 0.02, size=N)).astype(np.float32)
+        bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+        want = oracle.dequant_per_channel(acc, sI, sW, bias)
+        blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+        dA, dB, dOff = dev(torch, A), dev(torch, blob), dev(torch, off)
+        dsI, dsW, dbias = dev(torch, np.array([sI])), dev(torch, sW), dev(torch, bias)
+        out = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        capi.check(L.bolt_gfx950_mmm_int8_perchannel(M, N, K, dA.data_ptr(), dB.data_ptr(), dOff.data_ptr(),
+                                                     out.data_ptr(), dsI.data_ptr(), dsW.data_ptr(), dbias.data_ptr()),
+                   "mmm_perchannel")
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+        assert np.array_equal(out.cpu().numpy().view(np.int32), want.view(np.int32))
+        # all channels equal, no bias == reference per-tensor fp32 epilogue with scale = sI * sW
+        sW1 = np.full(N, np.float32(100.0), np.float32)
+        dsW1 = dev(torch, sW1)
+        capi.check(L.bolt_gfx950_mmm_int8_perchannel(M, N, K, dA.data_ptr(), dB.data_ptr(), dOff.data_ptr(),
+                                                     out.data_ptr(), dsI.data_ptr(), dsW1.data_ptr(), None), "mmm_pc")
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+        ref = oracle.mmm(A, W, off, np.zeros((M, N), np.float32), DT_F32, scale=[sI * np.float32(100.0)])
+        assert np.array_equal(out.cpu().numpy().view(np.int32), ref.view(np.int32))
+        if M == 1:
+            vblob, _ = host.mvm_transform_weight(W, DF_NORMAL, N, K)
+            dV = dev(torch, vblob)
+            y = torch.zeros(N, dtype=torch.float32, device="cuda")
+            capi.check(L.bolt_gfx950_mvm_int8_perchannel(N, K, dV.data_ptr(), dA.data_ptr(), dOff.data_ptr(),
+                                                         y.data_ptr(), dsI.data_ptr(), dsW.data_ptr(), dbias.data_ptr()),
+                       "mvm_perchannel")
+            capi.check(L.bolt_gfx950_synchronize(), "sync")
+            assert np.array_equal(y.cpu().numpy().view(np.int32), want[0].view(np.int32))

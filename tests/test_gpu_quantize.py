@@ -1,0 +1,159 @@
+"""GPU parity tests for quantize / dequantize / requantize / bias fold against the CPU oracle.
+u8 / s8 / int32 outputs and the returned scales are compared bit for bit; so are the fp32 outputs
+(one reciprocal and one multiply, same order as the reference)."""
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from bolt_amd import capi, host  # noqa: E402
+from bolt_amd.capi import DT_F32, DT_I8, DT_I32, DT_U8_Q  # noqa: E402
+from test_oracle_vs_ref import tie_table  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def torch_mod():
+    import torch
+    assert torch.cuda.is_available()
+    capi.check(capi.lib().bolt_gfx950_init(), "init")
+    return torch
+
+
+def both_modes(torch, x):
+    yield "host", np.ascontiguousarray(x), (lambda t: np.asarray(t))
+    yield "device", torch.from_numpy(np.ascontiguousarray(x)).cuda(), (lambda t: t.cpu().numpy())
+
+
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 1000, 65536, 4096 * 768 + 5])
+@pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
+def test_quantize_f32(torch_mod, oracle, n, qdt):
+    print("quantize_f32", n, qdt, flush=True)
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    for scale, mode in [(-1.0, 0), (20.0, 0), (1000.0, 0), (20.0, 1), (-1.0, 1), (0.0, 1)]:
+        want, ws = oracle.quantize_f32(x, qdt, scale, mode)
+        for name, buf, back in both_modes(torch_mod, x):
+            s = [scale]
+            got = back(host.quantize(buf, DT_F32, qdt, s, mode))
+            assert s[0] == ws and np.array_equal(got, want), (name, scale, mode)
+
+
+@pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
+def test_quantize_f32_special_inputs(torch_mod, oracle, qdt):
+    cases = [np.zeros(33, np.float32),
+             np.concatenate([np.full(40, 1e-3, np.float32), [1e6]]).astype(np.float32),
+             tie_table(1.0), tie_table(0.5), np.array([-3.0, 3.0, -0.0, 1e-30, -1e30], np.float32)]
+    for x in cases:
+        for scale, mode in [(-1.0, 0), (1.0, 1), (0.5, 1), (2.0, 0)]:
+            want, ws = oracle.quantize_f32(x, qdt, scale, mode)
+            for name, buf, back in both_modes(torch_mod, x):
+                s = [scale]
+                got = back(host.quantize(buf, DT_F32, qdt, s, mode))
+                assert s[0] == ws and np.array_equal(got, want), (name, scale, mode)
+
+
+def test_quantize_f32_async_device_scale(torch_mod, oracle):
+    torch = torch_mod
+    L = capi.lib()
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(4096 * 64).astype(np.float32)
+    dx = torch.from_numpy(x).cuda()
+    for qdt, tdt in ((DT_U8_Q, torch.uint8), (DT_I8, torch.int8)):
+        for scale, mode in [(-1.0, 0), (1000.0, 0), (20.0, 1)]:
+            ds = torch.tensor([scale], dtype=torch.float32, device="cuda")
+            q = torch.empty(x.size, dtype=tdt, device="cuda")
+            capi.check(L.bolt_gfx950_quantize_f32_async(dx.data_ptr(), x.size, qdt, q.data_ptr(), ds.data_ptr(), mode),
+                       "quantize_async")
+            capi.check(L.bolt_gfx950_synchronize(), "sync")
+            want, ws = oracle.quantize_f32(x, qdt, scale, mode)
+            assert np.float32(ds.item()) == ws and np.array_equal(q.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
+def test_quantize_i32(torch_mod, oracle, qdt):
+    rng = np.random.default_rng(5)
+    cases = [rng.integers(-200000, 200000, size=n, dtype=np.int32) for n in (1, 15, 16, 17, 4099, 32 * 64 * 56 * 56)]
+    cases.append(np.zeros(20, np.int32))
+    cases.append(np.array([524289, 524288, -(140 << 20), 300 << 20, -(128 << 20) - (1 << 19), -(1 << 31), (1 << 31) - 1,
+                           (1 << 19), 3 << 19, -(1 << 19), -(3 << 19)], np.int64).astype(np.int32))
+    for x in cases:
+        for sc in ([-1.0, 0.37], [0.05, 0.37], [400.0, 0.37], [-1.0, -1.0], [2.0 ** -20, 1.0]):
+            want, ws = oracle.quantize_i32(x, qdt, sc)
+            for name, buf, back in both_modes(torch_mod, x):
+                s = [np.float32(sc[0]), np.float32(sc[1])]
+                got = back(host.quantize(buf, DT_I32, qdt, s))
+                assert np.array_equal(np.array(s, np.float32), ws), (name, sc, s, ws)
+                assert np.array_equal(got, want), (name, sc, x.size)
+
+
+def test_u8_to_i8(torch_mod, oracle):
+    for n in [1, 63, 64, 65, 1000]:
+        x = (np.arange(n) * 37 % 256).astype(np.uint8)
+        for name, buf, back in both_modes(torch_mod, x):
+            assert np.array_equal(back(host.quantize(buf, DT_U8_Q, DT_I8, [1.0])), oracle.u8_to_i8(x))
+
+
+def test_bias_fold(torch_mod, oracle):
+    s = np.float32(8.0)
+    bias = np.concatenate([(np.arange(-20, 21) + 0.5) / 8.0, [0.3, -0.3, 1e3, -1e3, 0.0]]).astype(np.float32)
+    off = (np.arange(bias.size, dtype=np.int32) - 7) * 1000
+    N = bias.size
+    for name, b, back in both_modes(torch_mod, bias):
+        o = off if name == "host" else torch_mod.from_numpy(off).cuda()
+        assert np.array_equal(back(host.quantize_bias_offsetC(b, o, s, N)), oracle.bias_offsetC(bias, off, s))
+        assert np.array_equal(back(host.quantize_bias_offsetC(b, o, s, N, packed_filter=False)),
+                              oracle.bias_offsetC(bias, None, s))
+        assert np.array_equal(back(host.quantize_bias_offsetC(None, o, s, N)), off)
+    rng = np.random.default_rng(3)
+    b = rng.standard_normal(1024).astype(np.float32) * 0.1
+    sc = np.float32(41.7) * np.float32(100.0)
+    o = rng.integers(-10 ** 6, 10 ** 6, size=1024, dtype=np.int32)
+    assert np.array_equal(host.quantize_bias_offsetC(b, o, sc, 1024), oracle.bias_offsetC(b, o, sc))
+
+
+def test_dequantize(torch_mod, oracle):
+    rng = np.random.default_rng(11)
+    for n in [1, 16, 17, 100, 4096, 4096 * 768]:
+        q = rng.integers(-2 ** 31, 2 ** 31 - 1, size=n, dtype=np.int64).astype(np.int32)
+        for s in [0.37, 3.0, 4170.0, 1e-3]:
+            want = oracle.dequantize(q, DT_I32, s)
+            for name, buf, back in both_modes(torch_mod, q):
+                assert np.array_equal(back(host.dequantize(buf, DT_I32, s)).view(np.int32), want.view(np.int32))
+    for n in [1, 16, 17, 300]:
+        q = rng.integers(0, 256, size=n, dtype=np.uint8)
+        for s in [0.37, 3.0, 63.5]:
+            want = oracle.dequantize(q, DT_U8_Q, s)
+            for name, buf, back in both_modes(torch_mod, q):
+                assert np.array_equal(back(host.dequantize(buf, DT_U8_Q, s)).view(np.int32), want.view(np.int32))
+
+
+def test_requantize(torch_mod, oracle):
+    x = np.arange(-128, 128, dtype=np.int8)
+    for si, so in [(1.0, 1.0), (2.0, 1.0), (1.0, 0.9), (3.0, 2.0), (7.0, 6.99)]:
+        for name, buf, back in both_modes(torch_mod, x):
+            assert np.array_equal(back(host.requantize(buf, si, so)), oracle.requantize(x, si, so)), (si, so)
+
+
+def test_roundtrip_properties_at_full_size(torch_mod):
+    """Size-independent properties at the BERT FFN activation size (4096 x 3072): the extreme value
+    maps to 1 / 255, zero maps to 128, quantize is monotone, and dequantize(quantize(x)) is within
+    half a quantisation step."""
+    torch = torch_mod
+    n = 4096 * 3072
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(n, device="cuda", generator=g)
+    x[123] = 0.0
+    s = [-1.0]
+    q = host.quantize(x, DT_F32, DT_U8_Q, s)
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    amax = x.abs().max().item()
+    assert s[0] == np.float32(127.0) / np.float32(amax)
+    i = int(x.abs().argmax().item())
+    assert int(q[i].item()) in (1, 255) and int(q[123].item()) == 128
+    order = torch.argsort(x)
+    assert bool((q[order][1:].to(torch.int16) >= q[order][:-1].to(torch.int16)).all())
+    back = host.dequantize(q, DT_U8_Q, s[0])
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    assert float((back - x).abs().max().item()) <= 0.5 / float(s[0]) * 1.0001
