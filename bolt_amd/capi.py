@@ -87,6 +87,8 @@ SIGNATURES = {
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "bolt_gfx950_mvm_int8_strided_batch": (C.c_int, [_u32, _u32, _u32, _vp, C.c_size_t, _u32, _vp, _vp, _vp, _vp,
+                                                     _vp]),
 }
 
 _lib = None

@@ -225,6 +225,7 @@ EE mvm_device(U32 N, U32 K, DataType mdt, DataFormat mdf, const void *W, const v
         return SUCCESS;
     }
     GemvArgs g;
+    memset(&g, 0, sizeof(g));
     const U32 mat = packed_matrix_bytes(N, K);
     if (mdf != DF_NKN32K4) {
         // unpacked: tmp = [compensation N*4][packed matrix], as mvm.cpp:176-182 lays it out
@@ -1076,6 +1077,47 @@ EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void
     g.epi.scaleI = dscaleI;
     g.epi.scaleW = scaleW;
     g.epi.bias = bias;
+    HIP_TRY(launch_gemv_s8u8(g, ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_mvm_int8_strided_batch(U32 batch, U32 N, U32 K, const void *packedW, size_t weightStride,
+    U32 weightCopies, const void *x, float *y, const float *dscaleI, const float *scaleW, const float *bias)
+{
+    if (!packedW || !x || !y || !dscaleI || !scaleW) {
+        return NULL_POINTER;
+    }
+    if (batch == 0 || N == 0) {
+        return SUCCESS;
+    }
+    const size_t blob = (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4;
+    if (weightCopies == 0 || batch > 65535 || (weightCopies > 1 && (weightStride < blob || (weightStride & 3)))) {
+        return NOT_MATCH;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.W = (const int8_t *)packedW;
+    g.ldw = align_up(K, 8);
+    g.x = (const uint8_t *)x;
+    g.K = K;
+    g.N = N;
+    g.comp = (const int32_t *)((const U8 *)packedW + packed_matrix_bytes(N, K));
+    g.ob = g.comp;  // no folded bias: offsetC is each blob's own compensation vector
+    g.y = y;
+    g.epi.mode = EPI_F32_CH;
+    g.epi.scaleI = dscaleI;
+    g.epi.scaleW = scaleW;
+    g.epi.bias = bias;
+    g.batch.count = batch;
+    g.batch.wcopies = weightCopies;
+    g.batch.wstride = weightStride;
+    g.batch.xstride = K;
+    g.batch.ystride = N * 4;
+    g.batch.ob_in_blob = 1;
     HIP_TRY(launch_gemv_s8u8(g, ctx().stream));
     return SUCCESS;
 }

@@ -25,8 +25,23 @@ typedef int v2i_a4 __attribute__((ext_vector_type(2), aligned(4)));
 template <int ROWS, int XV>
 __global__ __launch_bounds__(256) void gemv_s8u8_kernel(const int8_t *__restrict__ W, uint32_t ldw,
     const uint8_t *__restrict__ x, uint32_t K, uint32_t N, const int32_t *__restrict__ ob,
-    const int32_t *__restrict__ comp, void *__restrict__ y, uint32_t tail0, int add_yin, Epilogue epi)
+    const int32_t *__restrict__ comp, void *__restrict__ y, uint32_t tail0, int add_yin, Epilogue epi,
+    GemvBatch bt)
 {
+    // strided batch of independent products: slice b uses weight blob b % wcopies, its own
+    // activation vector, result vector and (per-channel epilogue) input scale
+    if (gridDim.y > 1 || bt.wcopies) {
+        const uint32_t b = blockIdx.y;
+        const size_t wo = (size_t)(bt.wcopies ? b % bt.wcopies : 0) * bt.wstride;
+        W += wo;
+        comp = (const int32_t *)((const char *)comp + wo);
+        ob = (const int32_t *)((const char *)ob + (bt.ob_in_blob ? wo : 0));
+        x += (size_t)b * bt.xstride;
+        y = (char *)y + (size_t)b * bt.ystride;
+        if (epi.scaleI) {
+            epi.scaleI += b;
+        }
+    }
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const uint32_t n0 = wave * ROWS;
@@ -172,12 +187,14 @@ static hipError_t launch_s8u8(const GemvArgs &a, hipStream_t st)
     const uint32_t waves = (a.N + ROWS - 1) / ROWS;
     const uint32_t blocks = (waves + 3) / 4;
     const uint32_t tail0 = a.N - a.N % 8;
-    if (((uintptr_t)a.x & 3) == 0) {
-        hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 1>), dim3(blocks), dim3(256), 0, st, a.W, a.ldw, a.x, a.K,
-            a.N, a.ob, a.comp, a.y, tail0, a.add_yin, a.epi);
+    const dim3 grid(blocks, a.batch.count ? a.batch.count : 1);
+    const bool xv = (((uintptr_t)a.x | (uintptr_t)a.batch.xstride) & 3) == 0;
+    if (xv) {
+        hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 1>), grid, dim3(256), 0, st, a.W, a.ldw, a.x, a.K, a.N, a.ob,
+            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch);
     } else {
-        hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 0>), dim3(blocks), dim3(256), 0, st, a.W, a.ldw, a.x, a.K,
-            a.N, a.ob, a.comp, a.y, tail0, a.add_yin, a.epi);
+        hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 0>), grid, dim3(256), 0, st, a.W, a.ldw, a.x, a.K, a.N, a.ob,
+            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch);
     }
     return hipGetLastError();
 }

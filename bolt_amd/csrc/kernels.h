@@ -8,6 +8,15 @@
 namespace bg {
 
 // ---- GEMV ---------------------------------------------------------------------------------------
+struct GemvBatch {
+    uint32_t count;      // number of independent products in the launch (0 / 1: a single one)
+    uint32_t wcopies;    // slice b reads the weight blob b % wcopies (0: one blob)
+    size_t wstride;      // bytes between consecutive weight blobs
+    uint32_t xstride;    // bytes between activation vectors
+    uint32_t ystride;    // bytes between result vectors
+    int ob_in_blob;      // ob points into the blob and moves with it
+};
+
 struct GemvArgs {
     const int8_t *W;     // packed weight: row-major [ALIGN(N,16)][ldw], rows zero-padded
     uint32_t ldw;        // ALIGN(K, 8)
@@ -18,6 +27,7 @@ struct GemvArgs {
     void *y;
     int add_yin;         // accumulate into the int32 bits already in y
     Epilogue epi;
+    GemvBatch batch;
 };
 hipError_t launch_gemv_s8u8(const GemvArgs &a, hipStream_t st);
 hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const int8_t *x, uint32_t K, uint32_t M,

@@ -97,6 +97,15 @@ EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const voi
     float *C, const float *dscaleI, const float *scaleW, const float *bias);
 EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void *x, const I32 *offsetC, float *y,
     const float *dscaleI, const float *scaleW, const float *bias);
+/* `batch` independent matrix_vector_multiply products in ONE launch (decode serving: many
+ * requests, one step each): product b multiplies weight blob number b % weightCopies (blobs are
+ * weightStride bytes apart, each a complete transform_weight output) with activation vector
+ * x + b*K, writes y + b*N, and uses dscaleI[b] as its input scale. offsetC is each blob's own
+ * compensation vector (no folded bias); bias, if given, is the fp32 bias of the per-channel
+ * epilogue. No counterpart in the reference, whose GEMV is one call per vector
+ * (mvm_avx512_vnni.cpp:703-759). */
+EE bolt_gfx950_mvm_int8_strided_batch(U32 batch, U32 N, U32 K, const void *packedW, size_t weightStride,
+    U32 weightCopies, const void *x, float *y, const float *dscaleI, const float *scaleW, const float *bias);
 
 #ifdef __cplusplus
 }
