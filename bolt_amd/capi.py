@@ -62,6 +62,7 @@ SIGNATURES = {
     "bolt_gfx950_set_stream": (C.c_int, [_vp]),
     "bolt_gfx950_synchronize": (C.c_int, []),
     "bolt_gfx950_last_error": (C.c_char_p, []),
+    "bolt_gfx950_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "bolt_gfx950_malloc": (_vp, [C.c_size_t]),
     "bolt_gfx950_free": (None, [_vp]),
     "bolt_gfx950_memcpy_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),

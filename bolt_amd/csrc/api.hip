@@ -291,6 +291,18 @@ const char *bolt_gfx950_last_error(void)
     return ctx().err.c_str();
 }
 
+EE bolt_gfx950_set_option(const char *name, int value)
+{
+    if (!name) {
+        return NULL_POINTER;
+    }
+    if (strcmp(name, "gemm_tile") == 0) {
+        gemm_force_tile(value);
+        return SUCCESS;
+    }
+    return NOT_FOUND;
+}
+
 void *bolt_gfx950_malloc(size_t bytes)
 {
     if (ensure_init() != SUCCESS) {

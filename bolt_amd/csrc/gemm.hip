@@ -125,10 +125,527 @@ __global__ __launch_bounds__(256) void gemm_u8s8_general_kernel(GemmArgs a)
     }
 }
 
+// Tiled kernel for K % 16 == 0, row-major A with 16-byte aligned rows.
+//
+// Block = 4 waves (WM x WN), block tile (WM*TM*16) x (WN*TN*16), K step 128 (two 64-wide MFMA
+// K tiles). Both operands are staged in LDS in MFMA-fragment order: one fragment = the 1 KiB that
+// the 64 lanes of a 16x16x64 MFMA consume, lane l at byte 16*l, so every fragment read is one
+// conflict-free ds_read_b128 per lane. B fragments are a straight copy of the packed global
+// layout; A fragments are gathered with the same lane pattern (lane (i, g) reads 16 bytes of row
+// i at K offset 16*g) and re-biased (^ 0x80) on the way through registers. Two LDS stages: the
+// global loads of K step t+1 are issued before the MFMAs of step t and parked in registers.
+template <int WM, int WN, int TM, int TN>
+struct GemmTile {
+    static constexpr int kBM = WM * TM * 16;
+    static constexpr int kBN = WN * TN * 16;
+    static constexpr int kBK = 128;
+    static constexpr int kAFrags = (kBM / 16) * 2;   // per stage
+    static constexpr int kBFrags = (kBN / 16) * 2;
+    static constexpr int kWaves = WM * WN;
+    static constexpr int kALoads = kAFrags / kWaves;  // fragments loaded per wave
+    static constexpr int kBLoads = kBFrags / kWaves;
+    static constexpr int kStageBytes = (kAFrags + kBFrags) * 1024;
+    static constexpr int kLdsBytes = 2 * kStageBytes;
+};
+
+// Epilogue through LDS. Each wave parks 2 row-blocks (32 rows) of its tile at a time in its own LDS
+// region as a row-major int32 panel, then walks it so that every lane owns 4 consecutive columns
+// and every global access (C_in load, result store) of a wave is a contiguous run of TN*16
+// elements per row. The per-column terms (offsetC - compensation, channel scale, bias) are loaded
+// once per lane; the C_in loads of a panel are all issued before the first store so their latency
+// overlaps. Call after the last K-loop barrier.
+template <int MODE, int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
+{
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    constexpr int kCols = TN * 16;
+    constexpr int kPitch = kCols + 4;  // words; +4 keeps the 4 row groups of a tile on different banks
+    constexpr int kXPer = (TM < 2) ? TM : 2;
+    constexpr int kLanesPerRow = kCols / 4;
+    constexpr int kRowsPerIter = 64 / kLanesPerRow;
+    constexpr int kIters = kXPer * 16 / kRowsPerIter;
+    int32_t *panel = (int32_t *)smem + wave * 32 * kPitch;
+    const uint32_t cl = (lane % kLanesPerRow) * 4;
+    const uint32_t r0 = lane / kLanesPerRow;
+    const uint32_t n = n0 + wn * kCols + cl;
+    const bool vec = (n + 4 <= a.N) && ((a.N & 3) == 0);
+    const bool use_cin = a.add_cin && MODE != EPI_U8;
+
+    uint32_t base[4];
+    float sw[4], bs[4];
+    float factor = 0.0f, sI = 0.0f;
+    if (MODE == EPI_F32 || MODE == EPI_U8) {
+        factor = epi_factor(a.epi);
+    } else if (MODE == EPI_F32_CH) {
+        sI = *a.epi.scaleI;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const bool ok = n + c < a.N;
+        base[c] = ok ? (uint32_t)a.ob[n + c] - (uint32_t)a.comp[n + c] : 0u;
+        sw[c] = (MODE == EPI_F32_CH && ok) ? a.epi.scaleW[n + c] : 1.0f;
+        bs[c] = (MODE == EPI_F32_CH && ok && a.epi.bias) ? a.epi.bias[n + c] : 0.0f;
+    }
+
+#pragma unroll
+    for (int xh = 0; xh < TM; xh += kXPer) {
+#pragma unroll
+        for (int x = 0; x < kXPer; ++x) {
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    panel[(x * 16 + 4 * g + r) * kPitch + y * 16 + i] = acc[xh + x][y][r];
+                }
+            }
+        }
+        v4i cin[kIters];
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const uint32_t m = m0 + (wm * TM + xh) * 16 + r0 + it * kRowsPerIter;
+            cin[it] = (v4i){0, 0, 0, 0};
+            if (use_cin && m < a.M && n < a.N) {
+                const int32_t *p = (const int32_t *)a.C + (size_t)m * a.N + n;
+                if (vec) {
+                    cin[it] = *(const v4i *)p;
+                } else {
+                    for (int c = 0; c < 4 && n + c < a.N; ++c) {
+                        cin[it][c] = p[c];
+                    }
+                }
+            }
+        }
+        // the same wave wrote the panel and reads it back: LDS operations of one wave complete in order
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const uint32_t rr = r0 + it * kRowsPerIter;
+            const uint32_t m = m0 + (wm * TM + xh) * 16 + rr;
+            if (m >= a.M || n >= a.N) {
+                continue;
+            }
+            const v4i v = *(const v4i *)(panel + rr * kPitch + cl);
+            int t[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                t[c] = (int)((uint32_t)v[c] + base[c] + (uint32_t)cin[it][c]);  // int32 wrap
+            }
+            const size_t idx = (size_t)m * a.N + n;
+            if (MODE == EPI_I32) {
+                if (vec) {
+                    *(v4i *)((int32_t *)a.C + idx) = (v4i){t[0], t[1], t[2], t[3]};
+                } else {
+                    for (int c = 0; c < 4 && n + c < a.N; ++c) {
+                        ((int32_t *)a.C)[idx + c] = t[c];
+                    }
+                }
+            } else if (MODE == EPI_U8) {
+                unsigned b[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    b[c] = epi_u8(t[c], factor);
+                }
+                if (vec) {
+                    *(uint32_t *)((uint8_t *)a.C + idx) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                } else {
+                    for (int c = 0; c < 4 && n + c < a.N; ++c) {
+                        ((uint8_t *)a.C)[idx + c] = (uint8_t)b[c];
+                    }
+                }
+            } else {
+                float f[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (MODE == EPI_F32) {
+                        f[c] = (float)t[c] * factor;
+                    } else {
+                        const float s = sI * sw[c];
+                        const float q = 1.0f / s;
+                        f[c] = (float)t[c] * q;
+                        if (a.epi.bias) {
+                            f[c] = f[c] + bs[c];
+                        }
+                    }
+                }
+                if (vec) {
+                    *(v4f *)((float *)a.C + idx) = (v4f){f[0], f[1], f[2], f[3]};
+                } else {
+                    for (int c = 0; c < 4 && n + c < a.N; ++c) {
+                        ((float *)a.C)[idx + c] = f[c];
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // panel reads done before the next pair of row-blocks overwrites it
+    }
+}
+
+template <int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes)
+{
+    (void)lds_bytes;
+    switch (a.epi.mode) {
+        case EPI_I32:
+            epilogue_rows<EPI_I32, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            break;
+        case EPI_F32:
+            epilogue_rows<EPI_F32, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            break;
+        case EPI_U8:
+            epilogue_rows<EPI_U8, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            break;
+        default:
+            epilogue_rows<EPI_F32_CH, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            break;
+    }
+}
+
+template <int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_tiled_kernel(GemmArgs a)
+{
+    using T = GemmTile<WM, WN, TM, TN>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t m0 = blockIdx.y * T::kBM, n0 = blockIdx.x * T::kBN;
+    const uint32_t K = a.K;  // == Kp, multiple of 16
+    const uint32_t nblocks = align_up(a.N, 16) >> 4;
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+    v4i acc[TM][TN];
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            acc[x][y] = (v4i){0, 0, 0, 0};
+        }
+    }
+    v4i ra[T::kALoads], rb[T::kBLoads];
+
+    // per-lane global addresses of this wave's fragments at k0 = 0
+    const uint8_t *pa[T::kALoads];
+    const int8_t *pb[T::kBLoads];
+    bool va[T::kALoads], vb[T::kBLoads];
+#pragma unroll
+    for (int q = 0; q < T::kALoads; ++q) {
+        const uint32_t f = wave * T::kALoads + q;
+        const uint32_t row = m0 + (f >> 1) * 16 + i;
+        va[q] = row < a.M;
+        pa[q] = a.A + (size_t)(va[q] ? row : 0) * a.lda + (f & 1) * 64 + g * 16;
+    }
+#pragma unroll
+    for (int q = 0; q < T::kBLoads; ++q) {
+        const uint32_t f = wave * T::kBLoads + q;
+        const uint32_t nb = (n0 >> 4) + (f >> 1);
+        vb[q] = nb < nblocks;
+        pb[q] = a.Bp + (size_t)(vb[q] ? nb : 0) * 16 * K + (size_t)((f & 1) * 4 + g) * 256 + i * 16;
+    }
+
+#define BG_LOAD_GLOBAL(k0)                                                                  \
+    {                                                                                       \
+        _Pragma("unroll") for (int q = 0; q < T::kALoads; ++q)                              \
+        {                                                                                   \
+            const uint32_t f = wave * T::kALoads + q;                                       \
+            const uint32_t k = (k0) + (f & 1) * 64 + g * 16;                                \
+            const bool ok = va[q] && k < K;                                                 \
+            /* branch-free: out-of-range lanes read a valid dummy address and are zeroed */ \
+            const v4i v = *(const v4i *)(ok ? pa[q] + (k0) : a.A);                          \
+            ra[q] = ok ? (v ^ flip) : (v4i){0, 0, 0, 0};                                    \
+        }                                                                                   \
+        _Pragma("unroll") for (int q = 0; q < T::kBLoads; ++q)                              \
+        {                                                                                   \
+            const uint32_t f = wave * T::kBLoads + q;                                       \
+            const uint32_t k = (k0) + (f & 1) * 64 + g * 16;                                \
+            const bool ok = vb[q] && k < K;                                                 \
+            const v4i v = *(const v4i *)(ok ? pb[q] + (size_t)(k0) * 16 : a.Bp);            \
+            rb[q] = ok ? v : (v4i){0, 0, 0, 0};                                             \
+        }                                                                                   \
+    }
+#define BG_STORE_LDS(stage)                                                                 \
+    {                                                                                       \
+        uint8_t *sA_ = smem + (stage) * T::kStageBytes;                                     \
+        uint8_t *sB_ = sA_ + T::kAFrags * 1024;                                             \
+        _Pragma("unroll") for (int q = 0; q < T::kALoads; ++q)                              \
+        {                                                                                   \
+            *(v4i *)(sA_ + (wave * T::kALoads + q) * 1024 + lane * 16) = ra[q];             \
+        }                                                                                   \
+        _Pragma("unroll") for (int q = 0; q < T::kBLoads; ++q)                              \
+        {                                                                                   \
+            *(v4i *)(sB_ + (wave * T::kBLoads + q) * 1024 + lane * 16) = rb[q];             \
+        }                                                                                   \
+    }
+
+    const uint32_t ksteps = (K + T::kBK - 1) / T::kBK;
+    BG_LOAD_GLOBAL(0u);
+    BG_STORE_LDS(0);
+    __syncthreads();
+    for (uint32_t t = 0; t < ksteps; ++t) {
+        const int cur = t & 1;
+        if (t + 1 < ksteps) {
+            BG_LOAD_GLOBAL((t + 1) * T::kBK);
+        }
+        const uint8_t *sA = smem + cur * T::kStageBytes;
+        const uint8_t *sB = sA + T::kAFrags * 1024;
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
+            v4i fa[TM], fb[TN];
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+                fa[x] = *(const v4i *)(sA + (((wm * TM + x) << 1) + kh) * 1024 + lane * 16);
+            }
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                fb[y] = *(const v4i *)(sB + (((wn * TN + y) << 1) + kh) * 1024 + lane * 16);
+            }
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+#pragma unroll
+                for (int y = 0; y < TN; ++y) {
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[x], fb[y], acc[x][y], 0, 0, 0);
+                }
+            }
+        }
+        if (t + 1 < ksteps) {
+            BG_STORE_LDS(cur ^ 1);
+        }
+        __syncthreads();
+    }
+#undef BG_LOAD_GLOBAL
+#undef BG_STORE_LDS
+
+    epilogue_panel<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+}
+
+// Pipelined kernel for K % 64 == 0 (the shapes that matter for throughput).
+//
+// Same fragment-order LDS staging as above, but the tiles travel global -> LDS directly
+// (global_load_lds_dwordx4: every lane supplies its own global address, the 64 x 16 bytes land at
+// consecutive LDS addresses = exactly one MFMA fragment), with STAGES K tiles of 64 in flight so
+// that HBM / L2 latency is covered by several tiles' worth of MFMAs instead of one. No staging
+// registers; A is re-biased (^ 0x80) after the fragment read. One s_barrier per K tile:
+//   wait until this wave's share of tile t has landed -> barrier (everyone's share has landed and
+//   everyone is done reading tile t-1) -> refill the buffer of tile t-1 with tile t+STAGES-1 ->
+//   MFMAs on tile t.
+// Rows / column blocks past the matrix edge load a clamped (valid) address; what they produce is
+// never stored. Workgroup ids are re-mapped so that each XCD (ids are dealt round-robin over the 8
+// XCDs) works on one contiguous band of output tiles and re-uses its A rows / B columns in its L2.
+template <int WM, int WN, int TM, int TN, int STAGES>
+struct GemmDma {
+    static constexpr int kBM = WM * TM * 16;
+    static constexpr int kBN = WN * TN * 16;
+    static constexpr int kWaves = WM * WN;
+    static constexpr int kAFrags = kBM / 16;
+    static constexpr int kBFrags = kBN / 16;
+    static constexpr int kLoads = (kAFrags + kBFrags) / kWaves;  // fragments each wave fetches per K tile
+    static constexpr int kStageBytes = (kAFrags + kBFrags) * 1024;
+    static constexpr int kLdsBytes = STAGES * kStageBytes;
+    static_assert((kAFrags + kBFrags) % kWaves == 0, "fragments must divide evenly over the waves");
+};
+
+__device__ __forceinline__ constexpr int vmcnt_imm(int n)
+{
+    return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8);  // expcnt / lgkmcnt: no wait
+}
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+template <int WM, int WN, int TM, int TN, int STAGES>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
+{
+    using T = GemmDma<WM, WN, TM, TN, STAGES>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+
+    // XCD-aware tile order: hardware deals linear workgroup ids round-robin to the 8 XCDs; give XCD x
+    // the x-th contiguous eighth of the tile sequence, and walk that sequence in bands of 8 M-tiles.
+    const uint32_t tiles_m = (a.M + T::kBM - 1) / T::kBM, tiles_n = (a.N + T::kBN - 1) / T::kBN;
+    const uint32_t total = tiles_m * tiles_n;
+    uint32_t pid = blockIdx.x;
+    if (total % 8 == 0) {
+        pid = (pid % 8) * (total / 8) + pid / 8;
+    }
+    const uint32_t band = 8 * tiles_n;
+    const uint32_t band_id = pid / band;
+    const uint32_t band_rows = (tiles_m - band_id * 8 < 8) ? tiles_m - band_id * 8 : 8;
+    const uint32_t tm = band_id * 8 + (pid % band) % band_rows;
+    const uint32_t tn = (pid % band) / band_rows;
+    const uint32_t m0 = tm * T::kBM, n0 = tn * T::kBN;
+
+    const uint32_t K = a.K;
+    const uint32_t nblocks = align_up(a.N, 16) >> 4;
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+    v4i acc[TM][TN];
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            acc[x][y] = (v4i){0, 0, 0, 0};
+        }
+    }
+
+    // this wave's fragments: f = wave + q * kWaves; f < kAFrags is an A fragment (16 rows x 64 K-bytes)
+    const uint8_t *src[T::kLoads];
+    uint32_t step_bytes[T::kLoads];
+#pragma unroll
+    for (int q = 0; q < T::kLoads; ++q) {
+        const uint32_t f = wave + q * T::kWaves;
+        if (f < (uint32_t)T::kAFrags) {
+            uint32_t row = m0 + f * 16 + i;
+            row = row < a.M ? row : a.M - 1;
+            src[q] = a.A + (size_t)row * a.lda + g * 16;
+            step_bytes[q] = 64;
+        } else {
+            uint32_t nb = (n0 >> 4) + (f - T::kAFrags);
+            nb = nb < nblocks ? nb : nblocks - 1;
+            src[q] = (const uint8_t *)a.Bp + (size_t)nb * 16 * K + lane * 16;
+            step_bytes[q] = 1024;
+        }
+    }
+    const uint32_t ksteps = K / 64;
+
+#define BG_ISSUE(tile)                                                                                   \
+    {                                                                                                    \
+        uint8_t *st_ = smem + ((tile) % STAGES) * T::kStageBytes;                                        \
+        _Pragma("unroll") for (int q = 0; q < T::kLoads; ++q)                                            \
+        {                                                                                                \
+            __builtin_amdgcn_global_load_lds((gptr_t)(src[q] + (size_t)(tile)*step_bytes[q]),            \
+                (lptr_t)(st_ + (wave + q * T::kWaves) * 1024), 16, 0, 0);                                \
+        }                                                                                                \
+    }
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        if ((uint32_t)s < ksteps) {
+            BG_ISSUE((uint32_t)s);
+        }
+    }
+    for (uint32_t t = 0; t < ksteps; ++t) {
+        // tile t is the oldest batch in flight; up to STAGES-2 younger ones may stay outstanding
+        if (t + (STAGES - 2) < ksteps) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
+        } else {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (t + (STAGES - 1) < ksteps) {
+            BG_ISSUE(t + (STAGES - 1));
+        }
+        const uint8_t *sA = smem + (t % STAGES) * T::kStageBytes;
+        const uint8_t *sB = sA + T::kAFrags * 1024;
+        v4i fb[TN];
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            fb[y] = *(const v4i *)(sB + (wn * TN + y) * 1024 + lane * 16);
+        }
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            const v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16) ^ flip;
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[y], acc[x][y], 0, 0, 0);
+            }
+        }
+    }
+#undef BG_ISSUE
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // every wave is done with the K-loop buffers before they become the panel
+    asm volatile("" ::: "memory");
+    epilogue_panel<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+}
+
+template <int WM, int WN, int TM, int TN, int STAGES>
+static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
+{
+    using T = GemmDma<WM, WN, TM, TN, STAGES>;
+    static_assert(WM * WN * 32 * (TN * 16 + 4) * 4 <= T::kLdsBytes, "epilogue panel must fit the K-loop LDS");
+    static bool attr_set = false;
+    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
+        if (e != hipSuccess) {
+            return e;
+        }
+        attr_set = true;
+    }
+    const uint32_t tiles = ((a.N + T::kBN - 1) / T::kBN) * ((a.M + T::kBM - 1) / T::kBM);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), T::kLdsBytes, st, a);
+    return hipGetLastError();
+}
+
+template <int WM, int WN, int TM, int TN>
+static hipError_t launch_tiled(const GemmArgs &a, hipStream_t st)
+{
+    using T = GemmTile<WM, WN, TM, TN>;
+    static bool attr_set = false;
+    auto kern = gemm_u8s8_tiled_kernel<WM, WN, TM, TN>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
+        if (e != hipSuccess) {
+            return e;
+        }
+        attr_set = true;
+    }
+    dim3 grid((a.N + T::kBN - 1) / T::kBN, (a.M + T::kBM - 1) / T::kBM);
+    hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), T::kLdsBytes, st, a);
+    return hipGetLastError();
+}
+
+static int g_force_tile = -1;  // test hook: -1 = heuristic
+
+void gemm_force_tile(int t)
+{
+    g_force_tile = t;
+}
+
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
 {
     if (a.M == 0 || a.N == 0) {
         return hipSuccess;
+    }
+    const bool tiled_ok = !a.transA && (a.K % 16 == 0) && (a.lda % 16 == 0) && (((uintptr_t)a.A & 15) == 0) &&
+        (((uintptr_t)a.Bp & 15) == 0) && a.K >= 64;
+    int tile = 0;
+    if (tiled_ok) {
+        const uint64_t b256 = (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+        const uint64_t b128 = (uint64_t)((a.M + 127) / 128) * ((a.N + 127) / 128);
+        if (b256 >= 192) {
+            tile = 1;
+        } else if (b128 >= 64 || (a.M >= 128 && a.N >= 128)) {
+            tile = 2;
+        }
+    }
+    if (g_force_tile >= 0 && (tiled_ok || g_force_tile == 0)) {
+        tile = g_force_tile;
+    }
+    const bool dma_ok = tiled_ok && (a.K % 64 == 0);
+    if (tile >= 3 && !dma_ok) {
+        tile = tiled_ok ? 2 : 0;
+    }
+    switch (tile) {
+        case 1:
+            return launch_tiled<2, 2, 8, 8>(a, st);  // 256 x 256
+        case 2:
+            return launch_tiled<2, 2, 4, 4>(a, st);  // 128 x 128
+        case 3:
+            return launch_dma<2, 2, 8, 4, 3>(a, st);  // 256 x 128, 3 stages, 2 blocks / CU
+        case 4:
+            return launch_dma<2, 2, 4, 4, 4>(a, st);  // 128 x 128, 4 stages
+        case 5:
+            return launch_dma<2, 4, 8, 4, 4>(a, st);  // 256 x 256, 8 waves, 4 stages
+        case 6:
+            return launch_dma<2, 2, 8, 4, 4>(a, st);  // 256 x 128, 4 stages
+        default:
+            break;
     }
     dim3 grid((a.N + 63) / 64, (a.M + 63) / 64);
     hipLaunchKernelGGL(gemm_u8s8_general_kernel, grid, dim3(256), 0, st, a);

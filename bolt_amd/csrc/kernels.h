@@ -47,6 +47,8 @@ struct GemmArgs {
     Epilogue epi;
 };
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
+// tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
+void gemm_force_tile(int tile);
 
 // ---- weight pack --------------------------------------------------------------------------------
 // src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].

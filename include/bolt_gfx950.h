@@ -30,6 +30,9 @@ EE bolt_gfx950_init(void);
 EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
+/* Tuning knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1 = 256x256 block
+ * tiles, 2 = 128x128 block tiles (tiled kernels need K % 16 == 0; otherwise the general one runs). */
+EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);
 EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes);
