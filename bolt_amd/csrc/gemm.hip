@@ -454,12 +454,13 @@ __device__ __forceinline__ constexpr int vmcnt_imm(int n)
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-template <int WM, int WN, int TM, int TN, int STAGES>
+template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it scalar
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
 
@@ -491,85 +492,153 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         }
     }
 
-    // this wave's fragments: f = wave + q * kWaves; f < kAFrags is an A fragment (16 rows x 64 K-bytes)
-    const uint8_t *src[T::kLoads];
-    uint32_t step_bytes[T::kLoads];
+    // This wave's fragments per K tile: kQA A fragments (16 rows x 64 K-bytes), then B fragments.
+    // Addresses are split into a wave-uniform 64-bit base that advances with the tile (scalar
+    // registers, scalar ALU) and a 32-bit per-lane offset that never changes, so the loop issues
+    // its loads without any per-lane 64-bit arithmetic.
+    constexpr int kQA = T::kAFrags / T::kWaves;
+    static_assert(T::kAFrags % T::kWaves == 0, "A fragments must divide evenly over the waves");
+    uint32_t off[T::kLoads];
 #pragma unroll
     for (int q = 0; q < T::kLoads; ++q) {
-        const uint32_t f = wave + q * T::kWaves;
-        if (f < (uint32_t)T::kAFrags) {
-            uint32_t row = m0 + f * 16 + i;
+        if (q < kQA) {
+            uint32_t row = m0 + (wave + q * T::kWaves) * 16 + i;
             row = row < a.M ? row : a.M - 1;
-            src[q] = a.A + (size_t)row * a.lda + g * 16;
-            step_bytes[q] = 64;
+            off[q] = row * a.lda + g * 16;
         } else {
-            uint32_t nb = (n0 >> 4) + (f - T::kAFrags);
+            uint32_t nb = (n0 >> 4) + (wave + (q - kQA) * T::kWaves);
             nb = nb < nblocks ? nb : nblocks - 1;
-            src[q] = (const uint8_t *)a.Bp + (size_t)nb * 16 * K + lane * 16;
-            step_bytes[q] = 1024;
+            off[q] = nb * 16 * K + lane * 16;
         }
     }
     const uint32_t ksteps = K / 64;
 
-#define BG_ISSUE(tile)                                                                                   \
+// slot: which LDS buffer (slot % STAGES); tile: which K tile to fetch. Past the end of K the
+// schedule keeps issuing (slot advances, tile is clamped to the last one) so that the number of
+// loads in flight, and with it every vmcnt wait, is the same in every step; the refetched tile
+// lands in a buffer nobody reads any more.
+#define BG_ISSUE(slot, tile)                                                                             \
     {                                                                                                    \
-        uint8_t *st_ = smem + ((tile) % STAGES) * T::kStageBytes;                                        \
+        uint8_t *st_ = smem + ((slot) % STAGES) * T::kStageBytes;                                        \
         _Pragma("unroll") for (int q = 0; q < T::kLoads; ++q)                                            \
         {                                                                                                \
-            __builtin_amdgcn_global_load_lds((gptr_t)(src[q] + (size_t)(tile)*step_bytes[q]),            \
-                (lptr_t)(st_ + (wave + q * T::kWaves) * 1024), 16, 0, 0);                                \
+            const uint8_t *base_ = (q < kQA) ? a.A + (size_t)(tile)*64 : (const uint8_t *)a.Bp + (size_t)(tile)*1024; \
+            const int f_ = (q < kQA) ? (wave + q * T::kWaves) : (T::kAFrags + wave + (q - kQA) * T::kWaves);       \
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_ + off[q]), (lptr_t)(st_ + f_ * 1024), 16, 0, 0);         \
         }                                                                                                \
     }
+#define BG_CLAMP(tile) ((tile) < ksteps ? (tile) : ksteps - 1)
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
-        if ((uint32_t)s < ksteps) {
-            BG_ISSUE((uint32_t)s);
-        }
+        BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s));
     }
-    for (uint32_t t = 0; t < ksteps; ++t) {
-        // tile t is the oldest batch in flight; up to STAGES-2 younger ones may stay outstanding
-        if (t + (STAGES - 2) < ksteps) {
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
-        } else {
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    if constexpr (!PIPE) {
+        for (uint32_t t = 0; t < ksteps; ++t) {
+            // tile t is the oldest batch in flight; up to STAGES-2 younger ones may stay outstanding
+            if (t + (STAGES - 2) < ksteps) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
+            } else {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (t + (STAGES - 1) < ksteps) {
+                BG_ISSUE(t + (STAGES - 1), t + (STAGES - 1));
+            }
+            const uint8_t *sA = smem + (t % STAGES) * T::kStageBytes;
+            const uint8_t *sB = sA + T::kAFrags * 1024;
+            v4i fb[TN];
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                fb[y] = *(const v4i *)(sB + (wn * TN + y) * 1024 + lane * 16);
+            }
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+                const v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16) ^ flip;
+#pragma unroll
+                for (int y = 0; y < TN; ++y) {
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[y], acc[x][y], 0, 0, 0);
+                }
+            }
         }
+    } else {
+        // Fragment-prefetch schedule: the fragments of tile t+1 are read from LDS into a second
+        // register set while the MFMAs of tile t run, so no MFMA ever waits for an LDS read. That
+        // needs tile t+1 landed before step t starts: one tile more "landed ahead" than above.
+        static_assert(STAGES >= 3, "fragment prefetch needs at least 3 stages");
+        v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+#define BG_READ_FRAGS(tile, FA, FB)                                                          \
+    {                                                                                        \
+        const uint8_t *sA_ = smem + ((tile) % STAGES) * T::kStageBytes;                      \
+        const uint8_t *sB_ = sA_ + T::kAFrags * 1024;                                        \
+        _Pragma("unroll") for (int y = 0; y < TN; ++y)                                       \
+        {                                                                                    \
+            FB[y] = *(const v4i *)(sB_ + (wn * TN + y) * 1024 + lane * 16);                  \
+        }                                                                                    \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                       \
+        {                                                                                    \
+            FA[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + lane * 16); /* raw u8 */      \
+        }                                                                                    \
+    }
+#define BG_STEP(tt, FA, FB, NA, NB)                                                          \
+    {                                                                                        \
+        /* this wave's share of tile tt+1 has landed (younger tiles may stay in flight), and */ \
+        /* the fragment reads issued one step ago (FA / FB) are complete                     */ \
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * T::kLoads) & 0xf0ff);            \
+        asm volatile("" ::: "memory");                                                       \
+        __builtin_amdgcn_s_barrier();                                                        \
+        asm volatile("" ::: "memory");                                                       \
+        BG_ISSUE((tt) + (STAGES - 1), BG_CLAMP((tt) + (STAGES - 1)));                        \
+        BG_READ_FRAGS(BG_CLAMP((tt) + 1), NA, NB);                                           \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                       \
+        {                                                                                    \
+            const v4i fx_ = FA[x] ^ flip; /* re-bias at use: the read itself stays in flight */ \
+            _Pragma("unroll") for (int y = 0; y < TN; ++y)                                   \
+            {                                                                                \
+                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx_, FB[y], acc[x][y], 0, 0, 0); \
+            }                                                                                \
+        }                                                                                    \
+        /* issue order for the scheduler: the tile fetches first, then one LDS fragment read */ \
+        /* slipped in after every second MFMA, so the reads ride under the matrix pipeline   */ \
+        __builtin_amdgcn_sched_group_barrier(0x020, T::kLoads, 0);                           \
+        _Pragma("unroll") for (int r_ = 0; r_ < TM + TN; ++r_)                               \
+        {                                                                                    \
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                               \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                               \
+        }                                                                                    \
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 2 * (TM + TN), 0);             \
+    }
+        // tile 0 landed everywhere
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (t + (STAGES - 1) < ksteps) {
-            BG_ISSUE(t + (STAGES - 1));
+        BG_READ_FRAGS(0u, fa0, fb0);
+        for (uint32_t t = 0; t < ksteps; t += 2) {  // ksteps is even here (K % 128 == 0)
+            BG_STEP(t, fa0, fb0, fa1, fb1);
+            BG_STEP(t + 1, fa1, fb1, fa0, fb0);
         }
-        const uint8_t *sA = smem + (t % STAGES) * T::kStageBytes;
-        const uint8_t *sB = sA + T::kAFrags * 1024;
-        v4i fb[TN];
-#pragma unroll
-        for (int y = 0; y < TN; ++y) {
-            fb[y] = *(const v4i *)(sB + (wn * TN + y) * 1024 + lane * 16);
-        }
-#pragma unroll
-        for (int x = 0; x < TM; ++x) {
-            const v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16) ^ flip;
-#pragma unroll
-            for (int y = 0; y < TN; ++y) {
-                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[y], acc[x][y], 0, 0, 0);
-            }
-        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches before the buffers are reused
+#undef BG_STEP
+#undef BG_READ_FRAGS
     }
 #undef BG_ISSUE
+#undef BG_CLAMP
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();  // every wave is done with the K-loop buffers before they become the panel
     asm volatile("" ::: "memory");
     epilogue_panel<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES>
+template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     static_assert(WM * WN * 32 * (TN * 16 + 4) * 4 <= T::kLdsBytes, "epilogue panel must fit the K-loop LDS");
     static bool attr_set = false;
-    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES>;
+    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
         if (e != hipSuccess) {
@@ -618,10 +687,13 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     if (tiled_ok) {
         const uint64_t b256 = (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
         const uint64_t b128 = (uint64_t)((a.M + 127) / 128) * ((a.N + 127) / 128);
-        if (b256 >= 192) {
-            tile = 1;
-        } else if (b128 >= 64 || (a.M >= 128 && a.N >= 128)) {
-            tile = 2;
+        // measured on MI355X: 256 x 256 / 8 waves wins once it fills most of the 256 CUs; below
+        // that 128 x 128 tiles keep more CUs busy; tiny problems go to the general kernel
+        const bool k64 = (a.K % 64 == 0);
+        if (b256 >= 128 && k64) {
+            tile = 7;
+        } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
+            tile = k64 ? 10 : 2;
         }
     }
     if (g_force_tile >= 0 && (tiled_ok || g_force_tile == 0)) {
@@ -630,6 +702,9 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     const bool dma_ok = tiled_ok && (a.K % 64 == 0);
     if (tile >= 3 && !dma_ok) {
         tile = tiled_ok ? 2 : 0;
+    }
+    if (tile >= 7 && a.K % 128 != 0) {
+        tile = 4;  // the fragment-prefetch schedule walks K in pairs of 64-wide tiles
     }
     switch (tile) {
         case 1:
@@ -644,6 +719,14 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 4, 8, 4, 4>(a, st);  // 256 x 256, 8 waves, 4 stages
         case 6:
             return launch_dma<2, 2, 8, 4, 4>(a, st);  // 256 x 128, 4 stages
+        case 7:
+            return launch_dma<2, 4, 8, 4, 4, true>(a, st);  // 256 x 256, 8 waves, fragment prefetch
+        case 8:
+            return launch_dma<2, 2, 8, 8, 4, true>(a, st);  // 256 x 256, 4 waves of 128 x 128
+        case 9:
+            return launch_dma<2, 2, 8, 4, 4, true>(a, st);  // 256 x 128, fragment prefetch
+        case 10:
+            return launch_dma<2, 2, 4, 4, 4, true>(a, st);  // 128 x 128, fragment prefetch
         default:
             break;
     }

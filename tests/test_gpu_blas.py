@@ -118,6 +118,65 @@ def test_mmm_all_outputs_device(torch_mod, oracle, M, K, N):
     assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
+def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
+    """Each GEMM kernel (general, register-staged tiles, LDS-DMA pipelines) is forced in turn on
+    shapes with ragged M / N edges, one and many K tiles, and all four epilogues."""
+    L = capi.lib()
+    rng = np.random.default_rng(tile)
+    try:
+        capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
+        for M, K, N in [(1, 64, 16), (130, 128, 70), (256, 64, 256), (300, 256, 200), (257, 192, 513),
+                        (512, 1024, 384), (100, 1040, 48)]:
+            say("variant", tile, M, K, N)
+            A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+            W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+            off = oracle.offsetC(W, True) + rng.integers(-5000, 5000, size=N, dtype=np.int32)
+            blob, dt, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            Cin = rng.integers(-99, 99, size=(M, N), dtype=np.int32)
+            got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, Cin, DT_I32, None)
+            assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32)), (M, K, N)
+            s = np.float32(3.5)
+            z = np.zeros((M, N), np.float32)
+            got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, z, DT_F32, [s])
+            assert np.array_equal(got.view(np.int32), oracle.mmm(A, W, off, z, DT_F32, scale=[s]).view(np.int32))
+            acc = oracle.mmm(A, W, off, np.zeros((M, N), np.int32), DT_I32)
+            r = np.float32(127.0 / max(1, np.abs(acc).max()))
+            zu = np.zeros((M, N), np.uint8)
+            got = run_mmm(torch_mod, True, A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, off, zu, DT_U8_Q, [-1, r])
+            assert np.array_equal(got, oracle.mmm(A, W, off, zu, DT_U8_Q, scale=[-1, r])), (M, K, N)
+    finally:
+        L.bolt_gfx950_set_option(b"gemm_tile", -1)
+
+
+def test_mmm_full_size_properties(torch_mod, oracle):
+    """At the square-sweep size (4096^3) the oracle would take minutes, so the result is pinned by
+    size-independent properties: linearity in A (A1 + A2 in the signed domain), rows reproduced by
+    the GEMV kernel, and exact agreement on a random sample of outputs."""
+    torch = torch_mod
+    M = K = N = 4096
+    g = torch.Generator(device="cuda").manual_seed(7)
+    A1 = torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+    A2 = torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+    W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+    off = blob[rhs:rhs + 4 * N].clone()
+    ad, cd = tensor2df(DT_U8_Q, DF_NORMAL, M, K), tensor2df(DT_I32, DF_NORMAL, M, N)
+
+    def mm(A):
+        C = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+        capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, C, cd, None), "mmm")
+        return C
+    C1, C2, C12 = mm(A1), mm(A2), mm(A1 + A2)
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    # sum (a-128) w is affine in a: C(A1+A2) = C(A1) + C(A2) + 128 * colsum(W) = C1 + C2 - offsetC
+    assert torch.equal(C12, C1 + C2 - off.view(torch.int32)[None, :])
+    Wh, offh = W.cpu().numpy(), off.cpu().numpy().view(np.int32)
+    rows = [0, 1, 255, 256, 2047, 4095]
+    want = oracle.mmm(A1[rows].cpu().numpy(), Wh, offh, np.zeros((len(rows), N), np.int32), DT_I32)
+    assert np.array_equal(C1[rows].cpu().numpy(), want)
+
+
 def test_mmm_u8_epilogue_ties_and_saturation(torch_mod, oracle):
     M, K, N = 16, 8, 16
     A = np.full((M, K), 128, np.uint8)
