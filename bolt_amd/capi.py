@@ -85,6 +85,9 @@ SIGNATURES = {
     "dequantize_gfx950": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, TensorDesc, _vp, C.c_int]),
     "quantize_bias_offsetC_gfx950": (C.c_int, [_vp, TensorDesc, C.c_int, _vp, TensorDesc, _vp, _vp, C.c_int]),
     "requantize_gfx950": (C.c_int, [TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_float, C.c_int]),
+    "fully_connected_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, _u32p, C.c_int]),
+    "fully_connected_gfx950": (C.c_int, [TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_float, TensorDesc, _vp, _u32,
+                                         _vp, TensorDesc, _vp, _f32p, C.c_int]),
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

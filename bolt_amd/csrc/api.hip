@@ -1015,6 +1015,203 @@ EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDe
     return SUCCESS;
 }
 
+// ---- int8 FullyConnected (x86 branch of compute/tensor/src/fully_connected.cpp:372-495) ------------
+static void fc_dims(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, U32 *M, U32 *K, U32 *N)
+{
+    *N = outputDesc.dims[0];                                     // fw, fully_connected.cpp:370
+    *K = (*N) ? tensorNumElements(filterDesc) / (*N) : 0;        // fh
+    *M = (*K) ? tensorNumElements(inputDesc) / (*K) : 0;
+}
+
+EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    if (filterDesc.nDims != 2) {
+        return NOT_MATCH;
+    }
+    U32 M, K, N;
+    fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N);
+    EE e;
+    if (M != 1) {
+        e = matrix_matrix_multiply_tmp_bytes_gfx950(tensor2df(inputDesc.dt, DF_NORMAL, M, K), filterDesc, bytes, arch);
+    } else {
+        e = matrix_vector_multiply_tmp_bytes_gfx950(filterDesc, tensor1d(inputDesc.dt, K), bytes, arch);
+    }
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (filterDesc.dt == DT_I8) {  // fully_connected.cpp:149-156
+        if (inputDesc.dt != DT_I8) {
+            *bytes += tensorNumBytes(inputDesc);
+        }
+        *bytes += N * 4;
+        *bytes += tensorNumElements(outputDesc) * 4;
+    }
+    return SUCCESS;
+}
+
+// all pointers are device pointers here
+static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataFormat fdf, const void *filter, F32 scaleW,
+    const void *bias, void *tmp, DataType odt, void *output, F32 *outputScale)
+{
+    Ctx &c = ctx();
+    F32 scaleO = scaleI * scaleW;  // :396
+    F32 sarr[2] = {-1, -1};
+    const F32 *scale = nullptr;
+    DataType cdt = odt;
+    if (odt == DT_F32) {
+        scale = &scaleO;  // :381-382
+    } else if (odt == DT_U8_Q) {
+        if (*outputScale > 0) {
+            sarr[1] = *outputScale / scaleO;  // :383-387, :408-410
+            scale = sarr;
+        } else {
+            cdt = DT_I32;  // :388
+        }
+    }
+    U8 *t = (U8 *)tmp;
+    void *dst = output;
+    if (cdt != odt) {
+        dst = t;  // int32 result parked at the head of tmp, offsetC behind it (:400-403, :432-436)
+        t += (size_t)M * N * 4;
+    }
+    const U32 mat = packed_matrix_bytes(N, K);
+    const bool packed = (fdf == DF_NKNxKx || fdf == DF_NKN32K4);
+    // :404-406 -- the compensation vector sits behind the packed matrix; native formats have none
+    HIP_TRY(launch_bias_offsetC((const float *)bias, N, packed ? (const int32_t *)((const U8 *)filter + mat) : nullptr,
+        nullptr, scaleO, (int32_t *)t, c.stream));
+    // the reference zeroes the result (:458) and the product accumulates into it; starting the
+    // accumulation from zero without reading the buffer is the same result
+    EE e;
+    if (M == 1 && fdf != DF_NKNxKx) {  // :461-469
+        if (fdf != DF_NKN32K4) {
+            return fail(NOT_SUPPORTED, "FullyConnected expects a pre-packed filter (transform_filter)");
+        }
+        GemvArgs g;
+        memset(&g, 0, sizeof(g));
+        g.W = (const int8_t *)filter;
+        g.ldw = align_up(K, 8);
+        g.x = (const uint8_t *)input;
+        g.K = K;
+        g.N = N;
+        g.ob = (const int32_t *)t;
+        g.comp = (const int32_t *)((const U8 *)filter + mat);
+        g.y = dst;
+        g.epi = epi_from_scale(cdt == DT_I32 ? nullptr : scale);
+        HIP_TRY(launch_gemv_s8u8(g, c.stream));
+    } else {
+        if (fdf != DF_NKNxKx) {
+            return fail(NOT_SUPPORTED, "FullyConnected expects a pre-packed filter (transform_filter)");
+        }
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = (const uint8_t *)input;
+        g.lda = K;
+        g.Bp = (const int8_t *)filter;
+        g.M = M;
+        g.N = N;
+        g.K = K;
+        g.ob = (const int32_t *)t;
+        g.comp = (const int32_t *)((const U8 *)filter + mat);
+        g.C = dst;
+        g.epi = epi_from_scale(cdt == DT_I32 ? nullptr : scale);
+        HIP_TRY(launch_gemm_u8s8(g, c.stream));
+    }
+    e = SUCCESS;
+    if (cdt != odt) {  // :477-486 -- dynamic requantisation of the int32 result
+        float *dscale = (float *)(c.ws + 8);
+        HIP_TRY(launch_absmax_i32((const int32_t *)dst, M * N, c.ws, c.stream));
+        HIP_TRY(launch_requant_i32((const int32_t *)dst, M * N, output, 1, c.ws, *outputScale, scaleO, dscale, c.stream));
+        HIP_TRY(hipMemcpyAsync(outputScale, dscale, 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));  // the output scale is a host value in this interface
+    } else if (odt == DT_F32 || odt == DT_I32) {
+        *outputScale = scaleO;
+    }
+    return e;
+}
+
+EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScale, TensorDesc filterDesc,
+    const void *filter, F32 filterScale, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
+    TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!input || !filter || !output || !outputScale) {
+        return NULL_POINTER;
+    }
+    if (filterDesc.nDims != 2) {
+        return NOT_MATCH;
+    }
+    if (filterDesc.dt != DT_I8) {
+        return NOT_SUPPORTED;
+    }
+    if (inputDesc.dt != DT_U8_Q) {
+        return NOT_MATCH;  // CHECK_REQUIREMENT(idt == qIDesc.dt), fully_connected.cpp:395
+    }
+    const DataType odt = outputDesc.dt;
+    if (odt != DT_F32 && odt != DT_U8_Q && odt != DT_I32) {
+        return NOT_SUPPORTED;
+    }
+    U32 M, K, N;
+    fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N);
+    if (M == 0 || N == 0 || K == 0) {
+        return NOT_MATCH;
+    }
+    if (bias) {
+        if (biasDesc.nDims != 1 || biasDesc.dims[0] != N) {
+            return NOT_MATCH;  // fully_connected.cpp:444-446
+        }
+    }
+    U32 need = 0;
+    EE e = fully_connected_infer_forward_tmp_bytes_gfx950(inputDesc, filterDesc, outputDesc, &need, arch);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!tmp || tmpBytes < N * 4 + ((odt == DT_U8_Q && *outputScale <= 0) ? M * N * 4 : 0)) {
+        return tmp ? NOT_MATCH : NULL_POINTER;
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (arch == AMD_GFX950_DEVICE) {
+        if (!aligned4(tmp) || !aligned4(output) || !aligned4(filter)) {
+            return fail(NOT_SUPPORTED, "device tmp / filter / output must be 4-byte aligned");
+        }
+        return fc_device(M, K, N, input, inputScale, filterDesc.df, filter, filterScale, bias, tmp, odt, output,
+            outputScale);
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const size_t inB = (size_t)M * K, fB = (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4;
+    const size_t outB = (size_t)M * N * (odt == DT_U8_Q ? 1 : 4);
+    const size_t tB = (size_t)M * N * 4 + (size_t)N * 4 + 256;
+    void *dIn = st.get(inB), *dF = st.get(fB), *dB = bias ? st.get((size_t)N * 4) : nullptr, *dT = st.get(tB),
+         *dO = st.get(outB);
+    if (!dIn || !dF || !dT || !dO || (bias && !dB)) {
+        return fail(ALLOC_FAILED, "device staging");
+    }
+    HIP_TRY(hipMemcpyAsync(dIn, input, inB, hipMemcpyHostToDevice, c.stream));
+    HIP_TRY(hipMemcpyAsync(dF, filter, fB, hipMemcpyHostToDevice, c.stream));
+    if (bias) {
+        HIP_TRY(hipMemcpyAsync(dB, bias, (size_t)N * 4, hipMemcpyHostToDevice, c.stream));
+    }
+    e = fc_device(M, K, N, dIn, inputScale, filterDesc.df, dF, filterScale, dB, dT, odt, dO, outputScale);
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(output, dO, outB, hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return SUCCESS;
+}
+
 // ---- device-resident-scale forms ------------------------------------------------------------------
 EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode)
 {

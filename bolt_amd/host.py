@@ -191,3 +191,35 @@ def requantize(x, inScale, outScale):
     check(lib().requantize_gfx950(d, ptr(x), float(np.float32(inScale)), d, ptr(out), float(np.float32(outScale)), arch),
           "requantize")
     return out
+
+
+# ---- int8 FullyConnected ------------------------------------------------------------------------------
+def fully_connected_tmp_bytes(M, K, N, fdf, odt, arch=AMD_GFX950):
+    b = _u32()
+    idesc = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+    fdesc = tensor2df(DT_I8, fdf, K, N) if fdf == DF_NKNxKx else tensor2df(DT_I8, fdf, N, K)
+    check(lib().fully_connected_infer_forward_tmp_bytes_gfx950(idesc, fdesc, tensor2df(odt, DF_NORMAL, M, N),
+                                                               C.byref(b), arch), "fc_tmp_bytes")
+    return b.value
+
+
+def fully_connected(x, scaleI, filt, fdf, scaleW, bias, M, K, N, odt, scaleO=-1.0):
+    """x: u8 [M,K]; filt: packed blob from mmm_transform_rhs (fdf DF_NKNxKx) or mvm_transform_weight
+    (fdf DF_NKN32K4). Returns (output, output scale) like the reference's outputTensor / get_scale()."""
+    arch = arch_of(x)
+    nbytes = fully_connected_tmp_bytes(M, K, N, fdf, odt, arch)
+    tmp = _empty_like_mode(x, nbytes)
+    if _is_torch(x):
+        import torch
+        tdt = {DT_F32: torch.float32, DT_I32: torch.int32, DT_U8_Q: torch.uint8}[odt]
+        out = torch.zeros((M, N), dtype=tdt, device=x.device)
+    else:
+        out = np.zeros((M, N), NP_OF[odt])
+    so = C.c_float(float(np.float32(scaleO)))
+    idesc = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+    fdesc = tensor2df(DT_I8, fdf, K, N) if fdf == DF_NKNxKx else tensor2df(DT_I8, fdf, N, K)
+    e = lib().fully_connected_gfx950(idesc, ptr(x), float(np.float32(scaleI)), fdesc, ptr(filt),
+                                     float(np.float32(scaleW)), tensor1d(DT_F32, N), ptr(bias), nbytes, ptr(tmp),
+                                     tensor2df(odt, DF_NORMAL, M, N), ptr(out), C.byref(so), arch)
+    check(e, "fully_connected")
+    return out, np.float32(so.value)

@@ -87,6 +87,22 @@ EE quantize_bias_offsetC_gfx950(const void *bias, TensorDesc biasDesc, DataType 
 EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDesc outputDesc, INT8 *output,
     F32 outputScale, Arch arch);
 
+/* ---- tensor_computing: int8 FullyConnected ------------------------------------------- */
+/* compute/tensor/src/fully_connected.cpp:107-159  fully_connected_infer_forward_tmp_bytes */
+EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    U32 *bytes, Arch arch);
+/* compute/tensor/src/fully_connected.cpp:307-498  fully_connected, x86 int8 branch (:372-495), with
+ * the Tensor arguments unwrapped as get_ptr_from_tensor / get_scale do (tensor_auxiliary.h:26-37):
+ * input is DT_U8_Q [M, K] with scale inputScale; filter is the DT_I8 output of
+ * matrix_matrix_multiply_transform_rhs (M > 1) or matrix_vector_multiply_transform_weight (M == 1)
+ * with scale filterScale; bias is fp32 [N] or NULL. Output DT_F32: dequantised with
+ * inputScale * filterScale; DT_U8_Q with *outputScale > 0: requantised in the product's epilogue;
+ * DT_U8_Q with *outputScale <= 0: int32 result, then dynamic requantisation, new scale written to
+ * *outputScale (host); DT_I32: raw accumulators. tmp needs the bytes the query above returns. */
+EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScale, TensorDesc filterDesc,
+    const void *filter, F32 filterScale, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
+    TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch);
+
 /* ---- asynchronous forms with device-resident scales (AMD_GFX950_DEVICE only) -------- */
 /* No counterpart in the reference: Bolt keeps a tensor's scale in host memory
  * (common/memory/include/tensor.hpp:83-96). These keep it on the GPU so that

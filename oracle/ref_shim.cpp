@@ -153,4 +153,45 @@ int ref_requantize(const int8_t *in, U32 n, float inScale, int8_t *out, float ou
     return requantize_cpu(d, (INT8 *)in, inScale, d, out, outScale, X86_AVX512);
 }
 
+// int8 convolution through the reference's own sequence (compute/tensor/tests/test_convolution_int8.cpp:59-161):
+// transform_filter -> tmp bytes -> convolution_int8. Input u8 (DT_U8_Q) in `idf` (DF_NCHWC8 = 2 or
+// DF_NCHWC16 = 41), filter s8 NCHW, fp32 bias, optional fp32 eltwise input laid out like the output.
+// alg: 1 = CONVOLUTION_ALGORITHM_DIRECT, 0 = POINTWISE. scale[3] = {input, output (in/out), filter}.
+// odt: DT_F32 or DT_U8_Q; output layout is what the reference writes (NCHWC16, tail block C8).
+int ref_conv_int8(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 fw, U32 sh, U32 sw, U32 pt, U32 pb,
+    U32 pl, U32 pr, U32 dh, U32 dw, U32 oh, U32 ow, int alg, const uint8_t *in, const int8_t *filter, const float *bias,
+    const float *eltwise, float *scale, int relu, int odt, void *out)
+{
+    ConvolutionParamSpec p = createConvolutionParamSpec(
+        1, 1, fh, fw, 1, sh, sw, 0, 0, pt, pb, pl, pr, 1, dh, dw, oc, CONVOLUTION_DEPTHWISE_POINTWISE);
+    ConvolutionForwardAlgorithm a = (ConvolutionForwardAlgorithm)alg;
+    TensorDesc inputDesc = tensor4df(DT_U8_Q, (DataFormat)idf, n, ic, ih, iw);
+    TensorDesc filterDesc = tensor4df(DT_I8, DF_NCHW, oc, ic, fh, fw);
+    TensorDesc biasDesc = tensor1d(DT_F32, oc);
+    TensorDesc outputDesc = tensor4df((DataType)odt, DF_NCHWC16, n, oc, oh, ow);
+    U32 fcPad = (ic + 15) / 16 * 16;
+    U32 ftmBytes = oc * fcPad * fh * fw + oc * 4 + 32;  // cpu/x86/convolution.cpp:105-170
+    INT8 *ftm = (INT8 *)calloc(ftmBytes + 64, 1);
+    TensorDesc ftmDesc;
+    EE e = convolution_transform_filter_int8(filterDesc, filter, p, a, &ftmDesc, ftm);
+    if (e != SUCCESS) {
+        free(ftm);
+        return 1000 + e;
+    }
+    U32 tmpBytes = 0;
+    e = convolution_infer_forward_tmp_bytes_int8(inputDesc, ftmDesc, outputDesc, p, a, &tmpBytes);
+    if (e != SUCCESS) {
+        free(ftm);
+        return 2000 + e;
+    }
+    void *tmp = calloc((size_t)tmpBytes + n * oc * oh * ow * 4 + 4096, 1);
+    ActivationParamSpec act;
+    act.mode = relu ? ACTIVATION_RELU : ACTIVATION_NULL;
+    e = convolution_int8(inputDesc, (UINT8 *)in, (F32 *)eltwise, ftmDesc, ftm, p, a, biasDesc, bias, tmpBytes, tmp,
+        outputDesc, out, scale, act, X86_AVX512);
+    free(tmp);
+    free(ftm);
+    return e;
+}
+
 }  // extern "C"
