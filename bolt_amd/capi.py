@@ -53,6 +53,40 @@ def tensor1d(dt, n):
     return d
 
 
+class ConvolutionParamSpec(C.Structure):
+    """common/uni/include/parameter_spec.h:259-286"""
+    _pack_ = 8
+    _fields_ = [(k, C.c_uint32) for k in (
+        "num_outputs", "kernel_t", "kernel_h", "kernel_w", "stride_t", "stride_h", "stride_w", "pad_before", "pad_after",
+        "pad_top", "pad_bottom", "pad_left", "pad_right", "group", "dilatedRate_t", "dilatedRate_h", "dilatedRate_w",
+        "num_outputs_origin", "convolution_type", "dw_activation_type", "pw_activation_type")] + [
+        ("activation_spec", C.c_float * 2), ("round_mode", C.c_uint32), ("output_pad_t", C.c_uint32),
+        ("output_pad_h", C.c_uint32), ("output_pad_w", C.c_uint32)]
+
+
+class ActivationParamSpec(C.Structure):
+    """common/uni/include/parameter_spec.h:179-183"""
+    _pack_ = 8
+    _fields_ = [("mode", C.c_uint32), ("value", C.c_float * 4)]
+
+
+assert C.sizeof(ConvolutionParamSpec) == 108 and C.sizeof(ActivationParamSpec) == 20
+ACTIVATION_NULL, ACTIVATION_RELU = 0, 1
+CONVOLUTION_ALGORITHM_POINTWISE, CONVOLUTION_ALGORITHM_DIRECT, CONVOLUTION_ALGORITHM_BNN = 0, 1, 6
+
+
+def conv_param_spec(oc, fh, fw, stride, pad, dilation=1, group=1):
+    """createConvolutionParamSpec (parameter_spec.h:878-920) for the 2-D case."""
+    p = ConvolutionParamSpec()
+    p.num_outputs, p.kernel_t, p.kernel_h, p.kernel_w = oc, 1, fh, fw
+    p.stride_t, p.stride_h, p.stride_w = 1, stride, stride
+    p.pad_top = p.pad_bottom = p.pad_left = p.pad_right = pad
+    p.group, p.dilatedRate_t, p.dilatedRate_h, p.dilatedRate_w = group, 1, dilation, dilation
+    p.num_outputs_origin = oc
+    p.convolution_type = 3  # CONVOLUTION_DEPTHWISE_POINTWISE, what the reference's tests pass
+    return p
+
+
 _vp, _u32, _f32p, _u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
 _TDp = C.POINTER(TensorDesc)
 
@@ -88,6 +122,18 @@ SIGNATURES = {
     "fully_connected_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, _u32p, C.c_int]),
     "fully_connected_gfx950": (C.c_int, [TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_float, TensorDesc, _vp, _u32,
                                          _vp, TensorDesc, _vp, _f32p, C.c_int]),
+    "convolution_transform_filter_bytes_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, C.c_int, _u32p, C.c_int]),
+    "convolution_transform_filter_gfx950": (C.c_int, [TensorDesc, _vp, ConvolutionParamSpec, C.c_int, _TDp, _vp,
+                                                      C.c_int]),
+    "convolution_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, ConvolutionParamSpec,
+                                                             C.c_int, _u32p, C.c_int]),
+    "convolution_gfx950": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, C.c_int, TensorDesc,
+                                     _vp, _u32, _vp, TensorDesc, _vp, _f32p, ActivationParamSpec, C.c_int]),
+    "convolution_transform_filter_bytes_bnn_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
+    "convolution_transform_filter_bnn_gfx950": (C.c_int, [TensorDesc, _vp, C.POINTER(TensorDesc), _vp, C.c_int]),
+    "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),
+    "convolution_bnn_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, ConvolutionParamSpec, TensorDesc, _vp,
+                                         TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, ActivationParamSpec, C.c_int]),
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -1212,6 +1212,528 @@ EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScal
     return SUCCESS;
 }
 
+// ---- int8 convolution (compute/tensor/src/cpu/x86/int8/convolution.cpp:97-150) ---------------------
+namespace {
+
+struct ConvShape {
+    U32 n, ic, ih, iw, oc, fh, fw, oh, ow;
+    U32 sh, sw, pt, pb, pl, pr, dh, dw;
+    U32 Hp, Wp, ICp, Kp, N16;
+};
+
+EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w)
+{
+    if (d.nDims != 4) {
+        return NOT_MATCH;
+    }
+    *w = d.dims[0];
+    *h = d.dims[1];
+    *c = d.dims[2];
+    *n = d.dims[3];
+    return SUCCESS;
+}
+
+EE conv_shape(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, const ConvolutionParamSpec &p,
+    ConvShape *s)
+{
+    U32 on, fc;
+    if (get4d(inputDesc, &s->n, &s->ic, &s->ih, &s->iw) != SUCCESS || get4d(filterDesc, &s->oc, &fc, &s->fh, &s->fw) != SUCCESS ||
+        get4d(outputDesc, &on, &s->oc, &s->oh, &s->ow) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (p.group != 1) {
+        return NOT_SUPPORTED;  // depthwise / grouped int8 convolution is a different reference kernel
+    }
+    if (fc != s->ic || on != s->n || s->ic % 8 != 0 || s->oc % 8 != 0) {
+        return NOT_MATCH;
+    }
+    s->sh = p.stride_h;
+    s->sw = p.stride_w;
+    s->pt = p.pad_top;
+    s->pb = p.pad_bottom;
+    s->pl = p.pad_left;
+    s->pr = p.pad_right;
+    s->dh = p.dilatedRate_h ? p.dilatedRate_h : 1;
+    s->dw = p.dilatedRate_w ? p.dilatedRate_w : 1;
+    if (s->sh == 0 || s->sw == 0) {
+        return NOT_MATCH;
+    }
+    s->Hp = s->ih + s->pt + s->pb;
+    s->Wp = s->iw + s->pl + s->pr;
+    s->ICp = align_up(s->ic, 16);
+    s->Kp = align_up(s->fh * s->fw * s->ICp, 64);
+    s->N16 = align_up(s->oc, 16);
+    const U32 eh = (s->fh - 1) * s->dh + 1, ew = (s->fw - 1) * s->dw + 1;
+    if (s->Hp < eh || s->Wp < ew || (s->Hp - eh) / s->sh + 1 < s->oh || (s->Wp - ew) / s->sw + 1 < s->ow) {
+        return NOT_MATCH;  // the output must fit the padded input (every gather stays inside it)
+    }
+    return SUCCESS;
+}
+
+size_t conv_padded_bytes(const ConvShape &s)
+{
+    return ((size_t)s.n * s.Hp * s.Wp * s.ICp + 255) / 256 * 256;
+}
+
+size_t conv_tmp_layout(const ConvShape &s, DataType odt, size_t *tab, size_t *off, size_t *acc)
+{
+    size_t b = conv_padded_bytes(s);
+    *tab = b;
+    b += (size_t)(s.Kp / 16) * 4;
+    *off = b;
+    b += (size_t)s.oc * 4;
+    b = (b + 255) / 256 * 256;
+    *acc = b;
+    if (odt == DT_U8_Q) {
+        b += (size_t)s.n * s.oc * s.oh * s.ow * 4;
+    }
+    return b + 32;
+}
+
+void conv_pack_filter_host(const INT8 *src, const ConvShape &s, I32 *offsetC, INT8 *dst)
+{
+    const U32 fhw = s.fh * s.fw;
+    memset(dst, 0, (size_t)s.N16 * s.Kp);
+    for (U32 n = 0; n < s.oc; ++n) {
+        I32 sum = 0;
+        for (U32 c = 0; c < s.ic; ++c) {
+            for (U32 t = 0; t < fhw; ++t) {
+                const INT8 v = src[((size_t)n * s.ic + c) * fhw + t];
+                sum += v;
+                dst[mmm_packed_offset(n, t * s.ICp + c, s.Kp)] = v;
+            }
+        }
+        offsetC[n] = -128 * sum;
+    }
+}
+
+// all pointers device
+EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void *eltwise, const void *filter,
+    const void *bias, void *tmp, DataType odt, DataFormat odf, void *output, F32 *scale, int relu)
+{
+    Ctx &c = ctx();
+    size_t tabOff, offOff, accOff;
+    conv_tmp_layout(s, odt, &tabOff, &offOff, &accOff);
+    U8 *t = (U8 *)tmp;
+    const F32 scaleO = scale[0] * scale[2];  // convolution_direct.cpp:2687
+    HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
+        s.pr, (int8_t *)t, c.stream));
+    HIP_TRY(launch_conv_chunk_table((uint32_t *)(t + tabOff), s.fh, s.fw, s.dh, s.dw, s.Wp, s.ICp, 4, c.stream));
+    // filter blob = [offsetC oc*4][packed matrix] (convolution_transform.cpp:36-44 keeps the vector in front)
+    const int32_t *offC = (const int32_t *)filter;
+    const int8_t *mat = (const int8_t *)filter + (size_t)s.oc * 4;
+    HIP_TRY(launch_bias_offsetC((const float *)bias, s.oc, offC, nullptr, scaleO, (int32_t *)(t + offOff), c.stream));
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = (const uint8_t *)t;
+    g.Bp = mat;
+    g.M = s.n * s.oh * s.ow;
+    g.N = s.oc;
+    g.K = s.Kp;
+    g.ob = (const int32_t *)(t + offOff);
+    g.comp = offC;
+    g.conv.OHW = s.oh * s.ow;
+    g.conv.OW = s.ow;
+    g.conv.sh = s.sh;
+    g.conv.sw = s.sw;
+    g.conv.Hp = s.Hp;
+    g.conv.Wp = s.Wp;
+    g.conv.ICp = s.ICp;
+    g.conv.chunk_off = (const uint32_t *)(t + tabOff);
+    g.conv.out_c = (odf == DF_NCHWC8) ? 8 : 16;
+    g.conv.relu = relu;
+    if (odt == DT_F32) {
+        g.C = output;
+        g.epi.mode = EPI_F32;
+        g.epi.factor = 1 / scaleO;  // :2700-2703
+        g.conv.eltwise = (const float *)eltwise;
+        HIP_TRY(launch_conv_u8s8(g, c.stream));
+        scale[1] = scaleO;
+        return SUCCESS;
+    }
+    g.epi.mode = EPI_I32;
+    if (odt == DT_I32) {
+        g.C = output;
+        HIP_TRY(launch_conv_u8s8(g, c.stream));
+        scale[1] = scaleO;
+        return SUCCESS;
+    }
+    // u8: int32 accumulators to tmp with the running max|acc|, then the tensor-wide dynamic
+    // requantisation (:2797-2806); the new output scale goes back to the host
+    g.C = t + accOff;
+    g.conv.absmax = c.ws;
+    float *dscale = (float *)(c.ws + 8);
+    HIP_TRY(launch_fill_u32(c.ws, 1, 0, c.stream));
+    HIP_TRY(launch_conv_u8s8(g, c.stream));
+    HIP_TRY(launch_requant_i32((const int32_t *)g.C, g.M * g.N, output, 1, c.ws, -1.0f, scaleO, dscale, c.stream));
+    HIP_TRY(hipMemcpyAsync(&scale[1], dscale, 4, hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return SUCCESS;
+}
+
+}  // namespace
+
+EE convolution_transform_filter_bytes_gfx950(TensorDesc filterDesc, ConvolutionParamSpec p,
+    ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch)
+{
+    (void)algorithm;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    U32 fn, fc, fh, fw;
+    if (get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (p.group != 1 || filterDesc.dt != DT_I8) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = fn * 4 + align_up(fn, 16) * align_up(fh * fw * align_up(fc, 16), 64) + 32;
+    return SUCCESS;
+}
+
+EE convolution_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, ConvolutionParamSpec p,
+    ConvolutionForwardAlgorithm algorithm, TensorDesc *ftmDesc, void *filterTransformed, Arch arch)
+{
+    (void)algorithm;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!filter || !ftmDesc || !filterTransformed) {
+        return NULL_POINTER;
+    }
+    if (filterDesc.dt != DT_I8 || filterDesc.df != DF_NCHW || p.group != 1) {
+        return NOT_SUPPORTED;
+    }
+    ConvShape s;
+    memset(&s, 0, sizeof(s));
+    if (get4d(filterDesc, &s.oc, &s.ic, &s.fh, &s.fw) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    s.ICp = align_up(s.ic, 16);
+    s.Kp = align_up(s.fh * s.fw * s.ICp, 64);
+    s.N16 = align_up(s.oc, 16);
+    if (arch == AMD_GFX950) {
+        conv_pack_filter_host((const INT8 *)filter, s, (I32 *)filterTransformed, (INT8 *)filterTransformed + (size_t)s.oc * 4);
+    } else {
+        EE e = ensure_init();
+        if (e != SUCCESS) {
+            return e;
+        }
+        HIP_TRY(launch_conv_pack_filter((const int8_t *)filter, s.oc, s.ic, s.fh, s.fw, (int32_t *)filterTransformed,
+            (int8_t *)filterTransformed + (size_t)s.oc * 4, ctx().stream));
+    }
+    *ftmDesc = filterDesc;
+    ftmDesc->df = DF_NCHWC2NxC4;  // convolution_transform.cpp:207-211
+    return SUCCESS;
+}
+
+EE convolution_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec p, ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch)
+{
+    (void)algorithm;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    ConvShape s;
+    EE e = conv_shape(inputDesc, filterDesc, outputDesc, p, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    size_t a, b, c;
+    const size_t total = conv_tmp_layout(s, outputDesc.dt, &a, &b, &c);
+    if (total > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)total;
+    return SUCCESS;
+}
+
+EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwiseInput, TensorDesc filterDesc,
+    const void *filter, ConvolutionParamSpec p, ConvolutionForwardAlgorithm algorithm, TensorDesc biasDesc,
+    const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, F32 *scale,
+    ActivationParamSpec activationDesc, Arch arch)
+{
+    (void)algorithm;
+    (void)biasDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!input || !filter || !output || !bias || !tmp || !scale) {
+        return NULL_POINTER;  // x86/int8/convolution.cpp:114-117
+    }
+    if (outputDesc.df != DF_NCHWC16 && outputDesc.df != DF_NCHWC8) {
+        return NOT_MATCH;  // :128-130
+    }
+    if (inputDesc.dt != DT_U8_Q || filterDesc.dt != DT_I8 || filterDesc.df != DF_NCHWC2NxC4) {
+        return NOT_MATCH;  // convolution_direct.cpp:2613-2615 (activations arrive quantised on this path)
+    }
+    if (inputDesc.df != DF_NCHWC8 && inputDesc.df != DF_NCHWC16) {
+        return NOT_SUPPORTED;
+    }
+    const DataType odt = outputDesc.dt;
+    if (odt != DT_F32 && odt != DT_U8_Q && odt != DT_I32) {
+        return NOT_SUPPORTED;
+    }
+    if (activationDesc.mode != ACTIVATION_NULL && activationDesc.mode != ACTIVATION_RELU) {
+        return NOT_SUPPORTED;
+    }
+    if (eltwiseInput && odt != DT_F32) {
+        return NOT_SUPPORTED;
+    }
+    ConvShape s;
+    EE e = conv_shape(inputDesc, filterDesc, outputDesc, p, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    size_t a, b, c3;
+    const size_t need = conv_tmp_layout(s, odt, &a, &b, &c3);
+    if (tmpBytes < need) {
+        return NOT_MATCH;
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    const int relu = (activationDesc.mode == ACTIVATION_RELU);
+    if (arch == AMD_GFX950_DEVICE) {
+        if (((uintptr_t)tmp & 15) || ((uintptr_t)filter & 15) || ((uintptr_t)output & 15) || ((uintptr_t)input & 7)) {
+            return fail(NOT_SUPPORTED, "device tmp / filter / output must be 16-byte aligned, input 8-byte aligned");
+        }
+        return conv_device(s, inputDesc.df, input, eltwiseInput, filter, bias, tmp, odt, outputDesc.df, output, scale,
+            relu);
+    }
+    Ctx &cx = ctx();
+    Stage st;
+    const size_t inB = (size_t)s.n * s.ic * s.ih * s.iw;
+    const size_t fB = (size_t)s.oc * 4 + (size_t)s.N16 * s.Kp;
+    const size_t outN = (size_t)s.n * s.oc * s.oh * s.ow;
+    const size_t outB = outN * (odt == DT_U8_Q ? 1 : 4);
+    void *dIn = st.get(inB), *dF = st.get(fB), *dB = st.get((size_t)s.oc * 4), *dT = st.get(need), *dO = st.get(outB);
+    void *dE = eltwiseInput ? st.get(outN * 4) : nullptr;
+    if (!dIn || !dF || !dB || !dT || !dO || (eltwiseInput && !dE)) {
+        return fail(ALLOC_FAILED, "device staging");
+    }
+    HIP_TRY(hipMemcpyAsync(dIn, input, inB, hipMemcpyHostToDevice, cx.stream));
+    HIP_TRY(hipMemcpyAsync(dF, filter, fB, hipMemcpyHostToDevice, cx.stream));
+    HIP_TRY(hipMemcpyAsync(dB, bias, (size_t)s.oc * 4, hipMemcpyHostToDevice, cx.stream));
+    if (dE) {
+        HIP_TRY(hipMemcpyAsync(dE, eltwiseInput, outN * 4, hipMemcpyHostToDevice, cx.stream));
+    }
+    e = conv_device(s, inputDesc.df, dIn, dE, dF, dB, dT, odt, outputDesc.df, dO, scale, relu);
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(output, dO, outB, hipMemcpyDeviceToHost, cx.stream));
+    HIP_TRY(hipStreamSynchronize(cx.stream));
+    return SUCCESS;
+}
+
+// ---- 1-bit convolution (compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72) ----------------------
+EE convolution_transform_filter_bytes_bnn_gfx950(TensorDesc filterDesc, U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    U32 fn, fc, fh, fw;
+    if (get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (filterDesc.dt != DT_BIN01 && filterDesc.dt != DT_BIN11) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = fn * fc * fh * fw / 8;  // same size as the reference's DF_NCHWN16C8 blob
+    return SUCCESS;
+}
+
+EE convolution_transform_filter_bnn_gfx950(TensorDesc filterDesc, const void *filter, TensorDesc *ftmDesc,
+    void *filterTransformed, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!filter || !ftmDesc || !filterTransformed) {
+        return NULL_POINTER;  // convolution_transform_bnn.h:38-40
+    }
+    U32 fn, fc, fh, fw;
+    if (get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (filterDesc.dt != DT_BIN01 && filterDesc.dt != DT_BIN11) {
+        return NOT_SUPPORTED;
+    }
+    if (filterDesc.df != DF_NCHW && filterDesc.df != DF_NCHWN16C8) {
+        return NOT_MATCH;  // :83-84
+    }
+    if (fn % 32 != 0 || fc % 32 != 0) {
+        return NOT_SUPPORTED;  // kernel structure of the reference (convolution_xnor_A76.cpp:109,665)
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    const size_t bytes = (size_t)fn * fc * fh * fw / 8;
+    const int fmt = (filterDesc.df == DF_NCHWN16C8) ? 1 : 0;
+    if (arch == AMD_GFX950) {
+        Stage st;
+        void *a = st.get(bytes), *b = st.get(bytes);
+        if (!a || !b) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, filter, bytes, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(launch_bnn_pack_filter((const uint8_t *)a, fmt, fn, fc, fh * fw, (uint32_t *)b, c.stream));
+        HIP_TRY(hipMemcpyAsync(filterTransformed, b, bytes, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    } else {
+        if (!aligned4(filterTransformed)) {
+            return fail(NOT_SUPPORTED, "device filterTransformed must be 4-byte aligned");
+        }
+        HIP_TRY(launch_bnn_pack_filter((const uint8_t *)filter, fmt, fn, fc, fh * fw, (uint32_t *)filterTransformed, c.stream));
+    }
+    *ftmDesc = filterDesc;
+    ftmDesc->df = DF_NCHWN16C8;  // the tag the operator layer checks; the byte order inside is this library's
+    return SUCCESS;
+}
+
+EE convolution_infer_forward_tmp_bytes_bnn_gfx950(TensorDesc inputDesc, ConvolutionParamSpec p, U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    U32 n, ic, ih, iw;
+    if (get4d(inputDesc, &n, &ic, &ih, &iw) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    const size_t b = (size_t)n * (ih + p.pad_top + p.pad_bottom) * (iw + p.pad_left + p.pad_right) * (ic / 8) + 32;
+    if (b > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)b;
+    return SUCCESS;
+}
+
+EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc filterDesc, const void *filter,
+    ConvolutionParamSpec p, TensorDesc scaleDesc, const void *scale, TensorDesc biasDesc, const void *bias, U32 tmpBytes,
+    void *tmp, TensorDesc outputDesc, void *output, ActivationParamSpec activationDesc, Arch arch)
+{
+    (void)scaleDesc;
+    (void)biasDesc;
+    (void)activationDesc;  // ignored by the reference as well (bnn/convolution.cpp:35)
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!input || !filter || !output || !scale || !bias || !tmp) {
+        return NULL_POINTER;  // bnn/convolution.cpp:32-35
+    }
+    U32 n, ic, ih, iw, fn, fc, fh, fw, on, oc, oh, ow;
+    if (get4d(inputDesc, &n, &ic, &ih, &iw) != SUCCESS || get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS ||
+        get4d(outputDesc, &on, &oc, &oh, &ow) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    const DataType fdt = filterDesc.dt, idt = inputDesc.dt, odt = outputDesc.dt;
+    if (fdt != DT_BIN01 && fdt != DT_BIN11) {
+        return NOT_SUPPORTED;
+    }
+    // fp32 stands where the reference has fp16; bit-packed activations of the filter's type are also taken
+    if ((idt != DT_F32 && idt != fdt) || (odt != DT_F32 && odt != DT_I32)) {
+        return NOT_MATCH;
+    }
+    if ((idt == DT_F32 && inputDesc.df != DF_NCHWC8) || outputDesc.df != DF_NCHWC8 || filterDesc.df != DF_NCHWN16C8) {
+        return NOT_MATCH;  // :45-53
+    }
+    if (fc != ic || fn != oc || on != n || ic % 32 != 0 || oc % 32 != 0 || p.group != 1 || p.stride_h == 0 ||
+        p.stride_w == 0) {
+        return NOT_MATCH;
+    }
+    if ((p.dilatedRate_h > 1) || (p.dilatedRate_w > 1)) {
+        return NOT_SUPPORTED;
+    }
+    const U32 Hp = ih + p.pad_top + p.pad_bottom, Wp = iw + p.pad_left + p.pad_right;
+    if (Hp < fh || Wp < fw || (Hp - fh) / p.stride_h + 1 < oh || (Wp - fw) / p.stride_w + 1 < ow) {
+        return NOT_MATCH;
+    }
+    U32 need = 0;
+    EE e = convolution_infer_forward_tmp_bytes_bnn_gfx950(inputDesc, p, &need, arch);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (tmpBytes < need) {
+        return NOT_MATCH;
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const size_t inB = (idt == DT_F32) ? (size_t)n * ic * ih * iw * 4 : (size_t)n * ic * ih * iw / 8;
+    const size_t fB = (size_t)oc * ic * fh * fw / 8;
+    const size_t outN = (size_t)n * oc * oh * ow;
+    const void *dIn = input, *dF = filter, *dS = scale, *dB = bias;
+    void *dT = tmp, *dO = output;
+    if (arch == AMD_GFX950) {
+        void *a = st.get(inB), *f = st.get(fB), *s = st.get((size_t)oc * 4), *b = st.get((size_t)oc * 4);
+        dT = st.get(need);
+        dO = st.get(outN * 4);
+        if (!a || !f || !s || !b || !dT || !dO) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, input, inB, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(f, filter, fB, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(s, scale, (size_t)oc * 4, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(b, bias, (size_t)oc * 4, hipMemcpyHostToDevice, c.stream));
+        dIn = a;
+        dF = f;
+        dS = s;
+        dB = b;
+    } else if (!aligned4(tmp) || ((uintptr_t)output & 15) || !aligned4(filter)) {
+        return fail(NOT_SUPPORTED, "device tmp / filter must be 4-byte aligned, output 16-byte aligned");
+    }
+    const int xnor = (fdt == DT_BIN11);
+    HIP_TRY(launch_bnn_pack_input(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left, p.pad_right,
+        xnor ? 0.0f : 0.5f, (uint32_t *)dT, c.stream));
+    BnnArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = (const uint32_t *)dT;
+    a.w = (const uint32_t *)dF;
+    a.M = n * oh * ow;
+    a.OHW = oh * ow;
+    a.OW = ow;
+    a.sh = p.stride_h;
+    a.sw = p.stride_w;
+    a.Hp = Hp;
+    a.Wp = Wp;
+    a.IC = ic;
+    a.OC = oc;
+    a.fh = fh;
+    a.fw = fw;
+    a.scale = (const float *)dS;
+    a.bias = (const float *)dB;
+    if (odt == DT_I32) {
+        a.sums = (int32_t *)dO;
+    } else {
+        a.out = (float *)dO;
+    }
+    HIP_TRY(launch_bnn_conv(a, xnor, c.stream));
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(output, dO, outN * 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
 // ---- device-resident-scale forms ------------------------------------------------------------------
 EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode)
 {

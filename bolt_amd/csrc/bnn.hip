@@ -1,0 +1,207 @@
+// 1-bit (XNOR / DoReFa) convolution on the vector ALU: bit-packed +-1 / {0,1} operands, XOR (or AND)
+// and population count, no matrix cores.
+// (Bolt: compute/tensor/src/cpu/arm/bnn/convolution_xnor_A76.cpp:17-724, convolution_dorefa_A76.cpp,
+//  naive form compute/tensor/src/cpu/general/convolution.cpp:141-178.)
+//   XNOR   (DT_BIN11): bit 1 = +1, bit 0 = -1, padding = bit 0;  S = fh*fw*ic - 2 * popcount(x ^ w)
+//   DoReFa (DT_BIN01): bit 1 = 1,  bit 0 = 0,  padding = 0;      S = popcount(x & w)
+//   out = fma(S, scale[oc], bias[oc])
+//
+// Data layout on the GPU: activations are re-laid pixel-major, [n][Hp][Wp][ic/32] dwords (32
+// channels per dword, zero-bit border), so one tap of one pixel is ic/32 consecutive dwords.
+// Weights are re-laid [oc/32][tap][ic/32][32] dwords: for a fixed (tap, channel dword) the 32
+// output channels a wave works on are 32 consecutive dwords, which are wave-uniform and therefore
+// fetched with scalar loads. A wave owns 64 output pixels (one per lane) x 32 output channels:
+// per activation dword it issues 32 x (v_xor_b32 with an SGPR operand + v_bcnt_u32_b32 with the
+// accumulator as addend) = 2 VALU instructions per 32 binary multiply-accumulates per lane.
+#include "device_common.h"
+#include "kernels.h"
+#include "layout.h"
+
+namespace bg {
+
+// fp32 NCHWC8 (or already bit-packed [n][ic/8][h][w] bytes, MSB = first channel of the 8) ->
+// pixel-major padded dwords. One thread per output dword.
+template <int FROM_F32>
+__global__ __launch_bounds__(256) void bnn_pack_input_kernel(const void *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
+    uint32_t W, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, float thr, uint32_t *__restrict__ out)
+{
+    const uint32_t cw = C / 32;
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (uint64_t)N * Hp * Wp * cw) {
+        return;
+    }
+    const uint32_t j = (uint32_t)(id % cw);
+    uint64_t p = id / cw;
+    const uint32_t wp = (uint32_t)(p % Wp);
+    p /= Wp;
+    const uint32_t hp = (uint32_t)(p % Hp);
+    const uint32_t n = (uint32_t)(p / Hp);
+    uint32_t word = 0;
+    if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W) {
+        const uint32_t h = hp - pt, w = wp - pl;
+#pragma unroll
+        for (uint32_t b = 0; b < 4; ++b) {
+            const uint32_t c8 = j * 4 + b;
+            const size_t pix = (((size_t)n * (C / 8) + c8) * H + h) * W + w;
+            uint32_t byte = 0;
+            if (FROM_F32) {
+                const float *f = (const float *)in + pix * 8;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    byte |= (f[k] >= thr) ? (1u << (7 - k)) : 0u;  // common/uni/include/data_type.h:213-221
+                }
+            } else {
+                byte = ((const uint8_t *)in)[pix];
+            }
+            word |= byte << (8 * b);
+        }
+    }
+    out[id] = word;
+}
+
+hipError_t launch_bnn_pack_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, float thr, uint32_t *out, hipStream_t st)
+{
+    const uint32_t Hp = H + pt + pb, Wp = W + pl + pr;
+    const uint64_t total = (uint64_t)N * Hp * Wp * (C / 32);
+    if (total == 0) {
+        return hipSuccess;
+    }
+    const dim3 grid((uint32_t)((total + 255) / 256));
+    if (from_f32) {
+        hipLaunchKernelGGL((bnn_pack_input_kernel<1>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, out);
+    } else {
+        hipLaunchKernelGGL((bnn_pack_input_kernel<0>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, out);
+    }
+    return hipGetLastError();
+}
+
+// Filter bits -> [oc/32][tap][ic/32][32] dwords. src_fmt 0: DF_NCHW bit string, bit position
+// ((o * ic + c) * fhw + tap), MSB-first in each byte; 1: DF_NCHWN16C8 bytes
+// ((o/16 * ic/8 + c/8) * fhw + tap) * 16 + o%16 (convolution_transform_bnn.h:58-79). One thread per dword.
+__global__ __launch_bounds__(256) void bnn_pack_filter_kernel(const uint8_t *__restrict__ src, int src_fmt, uint32_t OC,
+    uint32_t IC, uint32_t fhw, uint32_t *__restrict__ dst)
+{
+    const uint32_t cw = IC / 32;
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (uint64_t)OC * fhw * cw) {
+        return;
+    }
+    const uint32_t o32 = (uint32_t)(id % 32);
+    uint64_t r = id / 32;
+    const uint32_t j = (uint32_t)(r % cw);
+    r /= cw;
+    const uint32_t tap = (uint32_t)(r % fhw);
+    const uint32_t o = (uint32_t)(r / fhw) * 32 + o32;
+    uint32_t word = 0;
+    for (uint32_t b = 0; b < 4; ++b) {
+        const uint32_t c8 = j * 4 + b;
+        uint32_t byte = 0;
+        if (src_fmt == 1) {
+            byte = src[(((size_t)(o / 16) * (IC / 8) + c8) * fhw + tap) * 16 + o % 16];
+        } else {
+            for (uint32_t k = 0; k < 8; ++k) {
+                const uint64_t bit = ((uint64_t)o * IC + c8 * 8 + k) * fhw + tap;
+                const uint32_t v = (src[bit >> 3] >> (7 - (bit & 7))) & 1u;
+                byte |= v << (7 - k);
+            }
+        }
+        word |= byte << (8 * b);
+    }
+    dst[id] = word;
+}
+
+hipError_t launch_bnn_pack_filter(const uint8_t *src, int src_fmt, uint32_t OC, uint32_t IC, uint32_t fhw, uint32_t *dst,
+    hipStream_t st)
+{
+    const uint64_t total = (uint64_t)OC * fhw * (IC / 32);
+    if (total == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(bnn_pack_filter_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, src, src_fmt, OC, IC,
+        fhw, dst);
+    return hipGetLastError();
+}
+
+// One wave: 64 output pixels (lane = pixel) x 32 output channels.
+template <int XNOR>
+__global__ __launch_bounds__(256) void bnn_conv_kernel(BnnArgs a)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t ob = blockIdx.y * 4 + wave;  // block of 32 output channels
+    if (ob * 32 >= a.OC) {
+        return;
+    }
+    const uint32_t cw = a.IC / 32;
+    uint32_t pix = blockIdx.x * 64 + lane;
+    const bool live = pix < a.M;
+    pix = live ? pix : a.M - 1;
+    const uint32_t img = pix / a.OHW, r = pix % a.OHW;
+    const uint32_t oy = r / a.OW, ox = r % a.OW;
+    const uint32_t *xp = a.x + (size_t)((img * a.Hp + oy * a.sh) * a.Wp + ox * a.sw) * cw;
+    const uint32_t *wp = a.w + (size_t)ob * a.fh * a.fw * cw * 32;
+
+    int acc[32];
+#pragma unroll
+    for (int o = 0; o < 32; ++o) {
+        acc[o] = 0;
+    }
+    for (uint32_t kh = 0; kh < a.fh; ++kh) {
+        for (uint32_t kw = 0; kw < a.fw; ++kw) {
+            const uint32_t *xt = xp + (size_t)(kh * a.Wp + kw) * cw;
+            for (uint32_t j = 0; j < cw; ++j) {
+                const uint32_t xv = xt[j];
+#pragma unroll
+                for (int o = 0; o < 32; ++o) {
+                    const uint32_t wv = wp[o];  // wave-uniform address: scalar load
+                    acc[o] += __builtin_popcount(XNOR ? (xv ^ wv) : (xv & wv));
+                }
+                wp += 32;
+            }
+        }
+    }
+    if (!live) {
+        return;
+    }
+    const int base = (int)(a.fh * a.fw * a.IC);
+#pragma unroll
+    for (int o8 = 0; o8 < 4; ++o8) {
+        const uint32_t oc0 = ob * 32 + o8 * 8;
+        const size_t idx = (((size_t)img * (a.OC / 8) + oc0 / 8) * a.OHW + r) * 8;  // NCHWC8
+        int s[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            s[k] = XNOR ? base - 2 * acc[o8 * 8 + k] : acc[o8 * 8 + k];
+        }
+        if (a.sums) {
+            *(v4i *)(a.sums + idx) = (v4i){s[0], s[1], s[2], s[3]};
+            *(v4i *)(a.sums + idx + 4) = (v4i){s[4], s[5], s[6], s[7]};
+        }
+        if (a.out) {
+            float f[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                f[k] = __builtin_fmaf((float)s[k], a.scale[oc0 + k], a.bias[oc0 + k]);  // vfmaq in the reference
+            }
+            *(v4f *)(a.out + idx) = (v4f){f[0], f[1], f[2], f[3]};
+            *(v4f *)(a.out + idx + 4) = (v4f){f[4], f[5], f[6], f[7]};
+        }
+    }
+}
+
+hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st)
+{
+    if (a.M == 0 || a.OC == 0) {
+        return hipSuccess;
+    }
+    const dim3 grid((a.M + 63) / 64, (a.OC / 32 + 3) / 4);
+    if (xnor) {
+        hipLaunchKernelGGL((bnn_conv_kernel<1>), grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bnn_conv_kernel<0>), grid, dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace bg

@@ -1,0 +1,156 @@
+// int8 convolution as implicit GEMM on the matrix cores (no im2col buffer is ever materialised).
+//
+//   acc[n, oc, oy, ox] = offsetC[oc] + round(bias[oc] * sI * sF) + sum_{c, kh, kw} in_u8 * w_s8,
+//   border reads 128          (Bolt x86: compute/tensor/src/cpu/x86/int8/avx512/convolution_direct.cpp:2584-2809)
+// = round(bias * s) + sum over taps inside the image of (in_u8 - 128) * w_s8.
+//
+// Three launches:
+//   1. conv_pad_kernel      u8 NCHWC8 / NCHWC16 activations -> s8 (x - 128), zero-padded border and
+//                           channel tail, channel-innermost [n][Hp][Wp][ICp]. After this the 16
+//                           K-bytes a lane feeds to one MFMA are 16 consecutive channels of one tap:
+//                           one contiguous 16-byte load, no bounds checks, no re-bias in the loop.
+//   2. the pipelined GEMM kernel of gemm.hip in convolution mode (rows = output pixels, K ordered
+//      (kh, kw, c), a [K/16] table gives each 16-channel chunk's offset from the pixel's base).
+//      Epilogue: folded bias, integer ReLU + running max|acc| (int32 out) or dequantise + eltwise +
+//      fp32 ReLU (fp32 out), written in the reference's NCHWC16 / NCHWC8 output order.
+//   3. for u8 output: the tensor-wide dynamic requantisation of quantize.hip.
+#include "device_common.h"
+#include "kernels.h"
+#include "layout.h"
+
+namespace bg {
+
+// one thread per 8 output bytes (8 channels of one padded pixel); consecutive threads write
+// consecutive bytes
+__global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
+    uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out)
+{
+    const uint32_t c8n = ICp / 8;
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t total = (uint64_t)N * Hp * Wp * c8n;
+    if (id >= total) {
+        return;
+    }
+    const uint32_t c8 = (uint32_t)(id % c8n);
+    uint64_t p = id / c8n;
+    const uint32_t wp = (uint32_t)(p % Wp);
+    p /= Wp;
+    const uint32_t hp = (uint32_t)(p % Hp);
+    const uint32_t n = (uint32_t)(p / Hp);
+    v2i v = {0, 0};
+    const uint32_t c0 = c8 * 8;
+    if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W && c0 < C) {
+        const uint32_t h = hp - pt, w = wp - pl;
+        // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
+        // 8 channels starting at c0 are contiguous for x = 8 and x = 16; a trailing block of an
+        // NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
+        const uint32_t blk = c0 / cx;
+        uint32_t bw = C - blk * cx;
+        bw = bw < cx ? bw : cx;
+        const size_t src = (size_t)n * C * H * W + (size_t)blk * cx * H * W + ((size_t)h * W + w) * bw + c0 % cx;
+        v = *(const v2i *)(in + src);
+        v ^= (v2i){(int)0x80808080, (int)0x80808080};
+    }
+    *(v2i *)(out + id * 8) = v;
+}
+
+hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st)
+{
+    const uint32_t Hp = H + pt + pb, Wp = W + pl + pr, ICp = align_up(C, 16);
+    const uint64_t total = (uint64_t)N * Hp * Wp * (ICp / 8);
+    if (total == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, in, N, C, H, W, cx, pt,
+        pl, Hp, Wp, ICp, out);
+    return hipGetLastError();
+}
+
+// chunk q = tap * (ICp / 16) + c16  ->  byte offset of that 16-channel chunk from the pixel's base
+__global__ void conv_chunk_table_kernel(uint32_t *tab, uint32_t chunks, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
+    uint32_t ICp)
+{
+    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= chunks) {
+        return;
+    }
+    const uint32_t cpt = ICp / 16;
+    const uint32_t tap = q / cpt, c16 = q % cpt;
+    const uint32_t kh = tap / fw, kw = tap % fw;
+    tab[q] = ((kh * dh) * Wp + kw * dw) * ICp + c16 * 16;
+}
+
+hipError_t launch_conv_chunk_table(uint32_t *tab, uint32_t fh, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
+    uint32_t ICp, uint32_t pad_to, hipStream_t st)
+{
+    // the K loop walks whole 64-byte tiles: chunks past fh*fw*ICp/16 (K not a multiple of 64) repeat
+    // the last valid offset; their filter bytes are zero
+    const uint32_t chunks = fh * fw * (ICp / 16);
+    const uint32_t padded = align_up(chunks, pad_to);
+    hipLaunchKernelGGL(conv_chunk_table_kernel, dim3((chunks + 63) / 64), dim3(64), 0, st, tab, chunks, fw, dh, dw, Wp, ICp);
+    if (padded > chunks) {
+        hipLaunchKernelGGL(conv_chunk_table_kernel, dim3(1), dim3(64), 0, st, tab + chunks, padded - chunks, 1u, 0u, 0u,
+            Wp, 16u);  // tap 0, c16 = 0..: any in-range offset does
+    }
+    return hipGetLastError();
+}
+
+// Filter s8 NCHW [oc][ic][fh][fw] -> MFMA-fragment layout over K = (kh, kw, c) with c padded to ICp
+// and K padded to a multiple of 64, N padded to 16. One thread per 8 packed bytes.
+__global__ __launch_bounds__(256) void conv_pack_filter_kernel(const int8_t *__restrict__ src, uint32_t OC, uint32_t IC,
+    uint32_t fhw, uint32_t ICp, uint32_t Kp, uint32_t N16, int8_t *__restrict__ dst)
+{
+    const uint32_t k8 = Kp / 8;
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (uint64_t)N16 * k8) {
+        return;
+    }
+    const uint32_t n = (uint32_t)(id / k8);
+    const uint32_t k0 = (uint32_t)(id % k8) * 8;
+    uint32_t lo = 0, hi = 0;
+    const uint32_t tap = k0 / ICp, c0 = k0 % ICp;
+    if (n < OC && tap < fhw) {
+        for (uint32_t b = 0; b < 8 && c0 + b < IC; ++b) {
+            const uint32_t v = (uint8_t)src[((size_t)n * IC + c0 + b) * fhw + tap];
+            if (b < 4) {
+                lo |= v << (8 * b);
+            } else {
+                hi |= v << (8 * (b - 4));
+            }
+        }
+    }
+    *(v2i *)(dst + mmm_packed_offset(n, k0, Kp)) = (v2i){(int)lo, (int)hi};
+}
+
+// offsetC[oc] = -128 * sum over ALL taps and channels (convolution_transform.cpp:38-44): one wave per oc
+__global__ __launch_bounds__(256) void conv_offsetC_kernel(const int8_t *__restrict__ src, uint32_t OC, uint32_t len,
+    int32_t *__restrict__ out)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t n = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (n >= OC) {
+        return;
+    }
+    int s = 0;
+    for (uint32_t i = lane; i < len; i += 64) {
+        s += (int)src[(size_t)n * len + i];
+    }
+    s = wave_reduce_add(s);
+    if (lane == 0) {
+        out[n] = s * (-128);
+    }
+}
+
+hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, uint32_t fh, uint32_t fw, int32_t *offsetC,
+    int8_t *dst, hipStream_t st)
+{
+    const uint32_t ICp = align_up(IC, 16), Kp = align_up(fh * fw * ICp, 64), N16 = align_up(OC, 16);
+    const uint64_t threads = (uint64_t)N16 * (Kp / 8);
+    hipLaunchKernelGGL(conv_pack_filter_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, st, src, OC, IC,
+        fh * fw, ICp, Kp, N16, dst);
+    hipLaunchKernelGGL(conv_offsetC_kernel, dim3((OC + 3) / 4), dim3(256), 0, st, src, OC, IC * fh * fw, offsetC);
+    return hipGetLastError();
+}
+
+}  // namespace bg

@@ -154,7 +154,7 @@ struct GemmTile {
 // elements per row. The per-column terms (offsetC - compensation, channel scale, bias) are loaded
 // once per lane; the C_in loads of a panel are all issued before the first store so their latency
 // overlaps. Call after the last K-loop barrier.
-template <int MODE, int WM, int WN, int TM, int TN>
+template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
@@ -170,8 +170,17 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     const uint32_t cl = (lane % kLanesPerRow) * 4;
     const uint32_t r0 = lane / kLanesPerRow;
     const uint32_t n = n0 + wn * kCols + cl;
-    const bool vec = (n + 4 <= a.N) && ((a.N & 3) == 0);
-    const bool use_cin = a.add_cin && MODE != EPI_U8;
+    // convolution output: blocks of out_c channels per pixel, so 4 channels starting at a multiple
+    // of 4 are always contiguous and 16-byte aligned
+    const bool vec = CONV ? (n + 4 <= a.N) : ((n + 4 <= a.N) && ((a.N & 3) == 0));
+    const bool use_cin = !CONV && a.add_cin && MODE != EPI_U8;
+    int lane_max = 0;
+    uint32_t cblk_off = 0, cblk_w = 1;
+    if (CONV) {
+        const uint32_t x = a.conv.out_c, blk = n / x;
+        cblk_w = (a.N - blk * x < x) ? a.N - blk * x : x;              // trailing narrower block
+        cblk_off = blk * x * a.conv.OHW + (n % x);
+    }
 
     uint32_t base[4];
     float sw[4], bs[4];
@@ -232,7 +241,26 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             for (int c = 0; c < 4; ++c) {
                 t[c] = (int)((uint32_t)v[c] + base[c] + (uint32_t)cin[it][c]);  // int32 wrap
             }
-            const size_t idx = (size_t)m * a.N + n;
+            size_t idx = (size_t)m * a.N + n;
+            if (CONV) {
+                const uint32_t img = m / a.conv.OHW, r = m % a.conv.OHW;
+                idx = (size_t)img * a.N * a.conv.OHW + cblk_off + (size_t)r * cblk_w;
+                if (MODE == EPI_I32 && a.conv.relu) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        t[c] = t[c] < 0 ? 0 : t[c];  // integer ReLU (convolution_direct.cpp:2406)
+                    }
+                }
+                if (MODE == EPI_I32) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        if (n + c < a.N) {
+                            const int av = (t[c] == (int)0x80000000) ? t[c] : (t[c] < 0 ? -t[c] : t[c]);
+                            lane_max = av > lane_max ? av : lane_max;
+                        }
+                    }
+                }
+            }
             if (MODE == EPI_I32) {
                 if (vec) {
                     *(v4i *)((int32_t *)a.C + idx) = (v4i){t[0], t[1], t[2], t[3]};
@@ -260,6 +288,14 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 for (int c = 0; c < 4; ++c) {
                     if (MODE == EPI_F32) {
                         f[c] = (float)t[c] * factor;
+                        if (CONV) {  // cvt * (1/s), + eltwise, fp32 ReLU (convolution_direct.cpp:2410-2422)
+                            if (a.conv.eltwise && n + c < a.N) {
+                                f[c] = f[c] + a.conv.eltwise[idx + c];
+                            }
+                            if (a.conv.relu && !(f[c] > 0.0f)) {
+                                f[c] = 0.0f;
+                            }
+                        }
                     } else {
                         const float s = sI * sw[c];
                         const float q = 1.0f / s;
@@ -280,25 +316,40 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // panel reads done before the next pair of row-blocks overwrites it
     }
+    if (CONV && MODE == EPI_I32 && a.conv.absmax) {
+        // max |acc| of the whole output tensor, for the dynamic requantisation that follows
+        lane_max = wave_reduce_max_i(lane_max);
+        if (lane == 0 && lane_max != 0) {
+            atomicMax((int *)a.conv.absmax, lane_max);
+        }
+    }
 }
 
-template <int WM, int WN, int TM, int TN>
+template <int WM, int WN, int TM, int TN, bool CONV = false>
 __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes)
 {
     (void)lds_bytes;
+    if (CONV) {
+        if (a.epi.mode == EPI_I32) {
+            epilogue_rows<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+        } else {
+            epilogue_rows<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+        }
+        return;
+    }
     switch (a.epi.mode) {
         case EPI_I32:
-            epilogue_rows<EPI_I32, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_rows<EPI_I32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         case EPI_F32:
-            epilogue_rows<EPI_F32, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_rows<EPI_F32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         case EPI_U8:
-            epilogue_rows<EPI_U8, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_rows<EPI_U8, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         default:
-            epilogue_rows<EPI_F32_CH, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_rows<EPI_F32_CH, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
     }
 }
@@ -454,7 +505,7 @@ __device__ __forceinline__ constexpr int vmcnt_imm(int n)
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE>
+template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE, bool CONV = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
@@ -504,7 +555,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         if (q < kQA) {
             uint32_t row = m0 + (wave + q * T::kWaves) * 16 + i;
             row = row < a.M ? row : a.M - 1;
-            off[q] = row * a.lda + g * 16;
+            if (CONV) {
+                // implicit GEMM: row = output pixel; its receptive field starts at this offset of the
+                // padded, channel-innermost s8 image; the tap / channel-chunk offset comes per K tile
+                const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
+                const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
+                off[q] = ((img * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * a.conv.ICp;
+            } else {
+                off[q] = row * a.lda + g * 16;
+            }
         } else {
             uint32_t nb = (n0 >> 4) + (wave + (q - kQA) * T::kWaves);
             nb = nb < nblocks ? nb : nblocks - 1;
@@ -517,21 +576,24 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 // schedule keeps issuing (slot advances, tile is clamped to the last one) so that the number of
 // loads in flight, and with it every vmcnt wait, is the same in every step; the refetched tile
 // lands in a buffer nobody reads any more.
-#define BG_ISSUE(slot, tile)                                                                             \
+#define BG_ISSUE(slot, tile, aoff)                                                                       \
     {                                                                                                    \
         uint8_t *st_ = smem + ((slot) % STAGES) * T::kStageBytes;                                        \
         _Pragma("unroll") for (int q = 0; q < T::kLoads; ++q)                                            \
         {                                                                                                \
-            const uint8_t *base_ = (q < kQA) ? a.A + (size_t)(tile)*64 : (const uint8_t *)a.Bp + (size_t)(tile)*1024; \
+            const uint8_t *base_ = (q < kQA) ? a.A + (aoff) : (const uint8_t *)a.Bp + (size_t)(tile)*1024;          \
             const int f_ = (q < kQA) ? (wave + q * T::kWaves) : (T::kAFrags + wave + (q - kQA) * T::kWaves);       \
             __builtin_amdgcn_global_load_lds((gptr_t)(base_ + off[q]), (lptr_t)(st_ + f_ * 1024), 16, 0, 0);         \
         }                                                                                                \
     }
 #define BG_CLAMP(tile) ((tile) < ksteps ? (tile) : ksteps - 1)
+// offset of K tile `tile` inside an A row: 64 bytes per tile for a matrix (scalar); for a convolution
+// the 16-byte chunk this lane's K-group covers belongs to tap / channel block chunk_off[4*tile + g]
+#define BG_AOFF(tile) (CONV ? (size_t)a.conv.chunk_off[(tile)*4 + g] : (size_t)(tile)*64)
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
-        BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s));
+        BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s), BG_AOFF(BG_CLAMP((uint32_t)s)));
     }
     if constexpr (!PIPE) {
         for (uint32_t t = 0; t < ksteps; ++t) {
@@ -545,7 +607,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             if (t + (STAGES - 1) < ksteps) {
-                BG_ISSUE(t + (STAGES - 1), t + (STAGES - 1));
+                BG_ISSUE(t + (STAGES - 1), t + (STAGES - 1), BG_AOFF(t + (STAGES - 1)));
             }
             const uint8_t *sA = smem + (t % STAGES) * T::kStageBytes;
             const uint8_t *sB = sA + T::kAFrags * 1024;
@@ -556,7 +618,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             }
 #pragma unroll
             for (int x = 0; x < TM; ++x) {
-                const v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16) ^ flip;
+                v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16);
+                if (!CONV) {
+                    fa ^= flip;
+                }
 #pragma unroll
                 for (int y = 0; y < TN; ++y) {
                     acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[y], acc[x][y], 0, 0, 0);
@@ -590,11 +655,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         asm volatile("" ::: "memory");                                                       \
         __builtin_amdgcn_s_barrier();                                                        \
         asm volatile("" ::: "memory");                                                       \
-        BG_ISSUE((tt) + (STAGES - 1), BG_CLAMP((tt) + (STAGES - 1)));                        \
+        BG_ISSUE((tt) + (STAGES - 1), BG_CLAMP((tt) + (STAGES - 1)), aoff_next);             \
+        aoff_next = BG_AOFF(BG_CLAMP((tt) + STAGES)); /* convolution: table load, one step ahead */ \
         BG_READ_FRAGS(BG_CLAMP((tt) + 1), NA, NB);                                           \
         _Pragma("unroll") for (int x = 0; x < TM; ++x)                                       \
         {                                                                                    \
-            const v4i fx_ = FA[x] ^ flip; /* re-bias at use: the read itself stays in flight */ \
+            const v4i fx_ = CONV ? FA[x] : (FA[x] ^ flip); /* re-bias at use: the read stays in flight */ \
             _Pragma("unroll") for (int y = 0; y < TN; ++y)                                   \
             {                                                                                \
                 acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx_, FB[y], acc[x][y], 0, 0, 0); \
@@ -616,9 +682,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         BG_READ_FRAGS(0u, fa0, fb0);
-        for (uint32_t t = 0; t < ksteps; t += 2) {  // ksteps is even here (K % 128 == 0)
+        size_t aoff_next = BG_AOFF(BG_CLAMP((uint32_t)(STAGES - 1)));
+        uint32_t t = 0;
+        for (; t + 1 < ksteps; t += 2) {
             BG_STEP(t, fa0, fb0, fa1, fb1);
             BG_STEP(t + 1, fa1, fb1, fa0, fb0);
+        }
+        if (t < ksteps) {  // odd tile count: the register sets are back in their initial roles
+            BG_STEP(t, fa0, fb0, fa1, fb1);
         }
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches before the buffers are reused
 #undef BG_STEP
@@ -626,19 +697,20 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     }
 #undef BG_ISSUE
 #undef BG_CLAMP
+#undef BG_AOFF
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();  // every wave is done with the K-loop buffers before they become the panel
     asm volatile("" ::: "memory");
-    epilogue_panel<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+    epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE = false>
+template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE = false, bool CONV = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     static_assert(WM * WN * 32 * (TN * 16 + 4) * 4 <= T::kLdsBytes, "epilogue panel must fit the K-loop LDS");
     static bool attr_set = false;
-    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE>;
+    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
         if (e != hipSuccess) {
@@ -667,6 +739,18 @@ static hipError_t launch_tiled(const GemmArgs &a, hipStream_t st)
     dim3 grid((a.N + T::kBN - 1) / T::kBN, (a.M + T::kBM - 1) / T::kBM);
     hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), T::kLdsBytes, st, a);
     return hipGetLastError();
+}
+
+// Implicit-GEMM convolution: same pipeline, A rows are output pixels gathered from the padded image.
+hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
+{
+    if (a.M == 0 || a.N == 0) {
+        return hipSuccess;
+    }
+    if (a.N <= 64) {
+        return launch_dma<2, 1, 8, 4, 4, true, true>(a, st);  // 256 pixels x 64 channels, 2 waves
+    }
+    return launch_dma<2, 2, 8, 4, 4, true, true>(a, st);      // 256 pixels x 128 channels
 }
 
 static int g_force_tile = -1;  // test hook: -1 = heuristic
@@ -702,9 +786,6 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     const bool dma_ok = tiled_ok && (a.K % 64 == 0);
     if (tile >= 3 && !dma_ok) {
         tile = tiled_ok ? 2 : 0;
-    }
-    if (tile >= 7 && a.K % 128 != 0) {
-        tile = 4;  // the fragment-prefetch schedule walks K in pairs of 64-wide tiles
     }
     switch (tile) {
         case 1:

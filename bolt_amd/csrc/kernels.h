@@ -34,6 +34,19 @@ hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const i
     void *y, const Epilogue &epi, hipStream_t st);
 
 // ---- GEMM ---------------------------------------------------------------------------------------
+// Geometry of an implicit-GEMM convolution (GemmArgs::conv), all in elements / bytes of the padded,
+// channel-innermost s8 image [n][Hp][Wp][ICp] that conv_pad produces.
+struct ConvGeom {
+    uint32_t OHW, OW;          // output pixels per image, output width
+    uint32_t sh, sw;           // strides
+    uint32_t Hp, Wp, ICp;      // padded image height / width, channels rounded up to 16
+    const uint32_t *chunk_off; // [K / 16] byte offset of 16-channel chunk q = tap * ICp/16 + c16 from the pixel base
+    uint32_t out_c;            // channel block of the output layout: 16 (NCHWC16) or 8 (NCHWC8)
+    int relu;
+    const float *eltwise;      // optional fp32 tensor added before the ReLU (fp32 output only)
+    uint32_t *absmax;          // optional: max |acc| over the whole output (int32 output only)
+};
+
 struct GemmArgs {
     const uint8_t *A;    // u8 activations
     uint32_t lda;        // bytes between consecutive m (transA = 0) or consecutive k (transA = 1)
@@ -45,10 +58,40 @@ struct GemmArgs {
     void *C;             // [M][N] row-major
     int add_cin;         // accumulate into the int32 bits already in C
     Epilogue epi;
+    ConvGeom conv;       // used by launch_conv_u8s8 only
 };
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
+// A = padded s8 image, M = n * OH * OW output pixels, N = output channels, K = fh * fw * ICp
+hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
 // tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
 void gemm_force_tile(int tile);
+
+// ---- convolution helpers (conv.hip) -------------------------------------------------------------
+// u8 NCHWC8 (cx = 8) / NCHWC16 (cx = 16) -> s8 (x - 128), zero padded, [n][H+pt+pb][W+pl+pr][ALIGN(C,16)]
+hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st);
+hipError_t launch_conv_chunk_table(uint32_t *tab, uint32_t fh, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
+    uint32_t ICp, uint32_t pad_to, hipStream_t st);
+// s8 NCHW filter -> offsetC[OC] and the fragment-layout matrix over K = (kh, kw, c)
+hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, uint32_t fh, uint32_t fw, int32_t *offsetC,
+    int8_t *dst, hipStream_t st);
+
+// ---- 1-bit convolution (bnn.hip) ----------------------------------------------------------------
+struct BnnArgs {
+    const uint32_t *x;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded
+    const uint32_t *w;     // [OC/32][fh*fw][IC/32][32] dwords
+    uint32_t M;            // n * OH * OW output pixels
+    uint32_t OHW, OW, sh, sw, Hp, Wp, IC, OC, fh, fw;
+    int32_t *sums;         // optional int32 sums, NCHWC8
+    float *out;            // optional fma(S, scale[oc], bias[oc]), NCHWC8
+    const float *scale, *bias;
+};
+hipError_t launch_bnn_pack_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, float thr, uint32_t *out, hipStream_t st);
+// src_fmt 0: DF_NCHW bit string, 1: DF_NCHWN16C8 bytes
+hipError_t launch_bnn_pack_filter(const uint8_t *src, int src_fmt, uint32_t OC, uint32_t IC, uint32_t fhw, uint32_t *dst,
+    hipStream_t st);
+hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st);
 
 // ---- weight pack --------------------------------------------------------------------------------
 // src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].

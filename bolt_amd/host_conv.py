@@ -1,0 +1,103 @@
+"""Python host-side mirror of the reference's convolution call sequence
+(compute/tensor/tests/test_convolution_int8.cpp:59-161, inference/engine/include/cpu/convolution_cpu.hpp:454-523):
+transform_filter_bytes -> transform_filter -> infer_forward_tmp_bytes -> convolution. numpy buffers use
+the host-pointer convention, torch CUDA tensors the device-pointer one. All arithmetic is in
+libbolt_gfx950.so."""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .capi import (ACTIVATION_NULL, ACTIVATION_RELU, CONVOLUTION_ALGORITHM_DIRECT, DF_NCHW, DF_NCHWC8, DF_NCHWC16,
+                   DF_NCHWC2NxC4, DT_F32, DT_I8, DT_I32, DT_U8_Q, ActivationParamSpec, TensorDesc, check, conv_param_spec,
+                   lib, tensor1d, tensor4df)
+from .host import NP_OF, _empty_like_mode, _is_torch, arch_of, ptr
+
+
+def conv_out_hw(ih, iw, fh, fw, stride, pad, dilation=1):
+    oh = (ih + 2 * pad - ((fh - 1) * dilation + 1)) // stride + 1
+    ow = (iw + 2 * pad - ((fw - 1) * dilation + 1)) // stride + 1
+    return oh, ow
+
+
+def transform_filter(filt_nchw, oc, ic, fh, fw, p):
+    arch = arch_of(filt_nchw)
+    fdesc = tensor4df(DT_I8, DF_NCHW, oc, ic, fh, fw)
+    b = C.c_uint32(0)
+    check(lib().convolution_transform_filter_bytes_gfx950(fdesc, p, CONVOLUTION_ALGORITHM_DIRECT, C.byref(b), arch),
+          "conv_filter_bytes")
+    blob = _empty_like_mode(filt_nchw, b.value)
+    ftm = TensorDesc()
+    check(lib().convolution_transform_filter_gfx950(fdesc, ptr(filt_nchw), p, CONVOLUTION_ALGORITHM_DIRECT, C.byref(ftm),
+                                                    ptr(blob), arch), "conv_transform_filter")
+    return blob, ftm
+
+
+def convolution(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias, scale, relu, odt, odf=DF_NCHWC16,
+                eltwise=None, dilation=1):
+    """x: u8 activations in `idf`; blob / ftm from transform_filter; scale = [sI, sO, sF] (list, sO updated).
+    Returns the output buffer in `odf` order."""
+    arch = arch_of(x)
+    p = conv_param_spec(oc, fh, fw, stride, pad, dilation)
+    oh, ow = conv_out_hw(ih, iw, fh, fw, stride, pad, dilation)
+    idesc = tensor4df(DT_U8_Q, idf, n, ic, ih, iw)
+    odesc = tensor4df(odt, odf, n, oc, oh, ow)
+    b = C.c_uint32(0)
+    check(lib().convolution_infer_forward_tmp_bytes_gfx950(idesc, ftm, odesc, p, CONVOLUTION_ALGORITHM_DIRECT, C.byref(b),
+                                                           arch), "conv_tmp_bytes")
+    tmp = _empty_like_mode(x, b.value)
+    count = n * oc * oh * ow
+    if _is_torch(x):
+        import torch
+        tdt = {DT_F32: torch.float32, DT_I32: torch.int32, DT_U8_Q: torch.uint8}[odt]
+        out = torch.zeros(count, dtype=tdt, device=x.device)
+    else:
+        out = np.zeros(count, NP_OF[odt])
+    sarr = (C.c_float * 3)(*[float(np.float32(v)) for v in scale])
+    act = ActivationParamSpec()
+    act.mode = ACTIVATION_RELU if relu else ACTIVATION_NULL
+    e = lib().convolution_gfx950(idesc, ptr(x), ptr(eltwise), ftm, ptr(blob), p, CONVOLUTION_ALGORITHM_DIRECT,
+                                 tensor1d(DT_F32, oc), ptr(bias), b.value, ptr(tmp), odesc, ptr(out), sarr, act, arch)
+    check(e, "convolution")
+    for i in range(3):
+        scale[i] = np.float32(sarr[i])
+    return out
+
+
+def bnn_transform_filter(filt_bits, fdt, fdf, oc, ic, fh, fw):
+    """1-bit filter (DF_NCHW bit string or DF_NCHWN16C8 bytes) -> this library's blob
+    (compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86)."""
+    arch = arch_of(filt_bits)
+    fdesc = tensor4df(fdt, fdf, oc, ic, fh, fw)
+    b = C.c_uint32(0)
+    check(lib().convolution_transform_filter_bytes_bnn_gfx950(fdesc, C.byref(b), arch), "bnn_filter_bytes")
+    blob = _empty_like_mode(filt_bits, b.value)
+    ftm = TensorDesc()
+    check(lib().convolution_transform_filter_bnn_gfx950(fdesc, ptr(filt_bits), C.byref(ftm), ptr(blob), arch),
+          "bnn_transform_filter")
+    return blob, ftm
+
+
+def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, scale, bias, odt=DT_F32):
+    """x: fp32 NCHWC8 activations (idt = DT_F32) or packed bits (idt = the filter's type); scale / bias fp32 [oc].
+    Mirrors convolution_bnn (compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72). Output NCHWC8."""
+    arch = arch_of(x)
+    p = conv_param_spec(oc, fh, fw, stride, pad)
+    oh, ow = conv_out_hw(ih, iw, fh, fw, stride, pad)
+    idesc = tensor4df(idt, DF_NCHWC8, n, ic, ih, iw)
+    odesc = tensor4df(odt, DF_NCHWC8, n, oc, oh, ow)
+    b = C.c_uint32(0)
+    check(lib().convolution_infer_forward_tmp_bytes_bnn_gfx950(idesc, p, C.byref(b), arch), "bnn_tmp_bytes")
+    tmp = _empty_like_mode(x, b.value)
+    count = n * oc * oh * ow
+    if _is_torch(x):
+        import torch
+        out = torch.zeros(count, dtype={DT_F32: torch.float32, DT_I32: torch.int32}[odt], device=x.device)
+    else:
+        out = np.zeros(count, NP_OF[odt])
+    act = ActivationParamSpec()
+    act.mode = ACTIVATION_NULL
+    e = lib().convolution_bnn_gfx950(idesc, ptr(x), ftm, ptr(blob), p, tensor1d(DT_F32, oc), ptr(scale),
+                                     tensor1d(DT_F32, oc), ptr(bias), b.value, ptr(tmp), odesc, ptr(out), act, arch)
+    check(e, "convolution_bnn")
+    return out

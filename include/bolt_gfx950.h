@@ -103,6 +103,56 @@ EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScal
     const void *filter, F32 filterScale, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
     TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch);
 
+/* ---- tensor_computing: int8 convolution ---------------------------------------------- */
+/* The inner (TensorDesc + pointer) forms the reference's convolution*() reach on x86:
+ *   convolution_transform_filter_bytes_x86   compute/tensor/src/cpu/x86/convolution.cpp:105-170
+ *   convolution_transform_filter_int8        compute/tensor/src/cpu/x86/int8/convolution_transform.cpp:192-238
+ *   convolution_infer_forward_tmp_bytes_int8 compute/tensor/src/cpu/x86/int8/convolution.cpp:17-95
+ *   convolution_int8                         compute/tensor/src/cpu/x86/int8/convolution.cpp:97-150
+ * Sizes are this back end's own (a back end answers its own size queries); callers allocate what
+ * the queries return, exactly as ConvolutionCPU does (convolution_cpu.hpp:454-523).
+ * Filter: DT_I8 DF_NCHW [oc, ic, fh, fw] -> blob tagged DF_NCHWC2NxC4 = [offsetC oc*4 | packed].
+ * Input: DT_U8_Q in DF_NCHWC8 or DF_NCHWC16. Output DF_NCHWC16 (what the reference produces; a
+ * trailing block is 8 wide when oc % 16 == 8) or DF_NCHWC8; DT_F32 (optionally + eltwiseInput, laid
+ * out like the output), DT_I32, or DT_U8_Q with the tensor-wide dynamic output scale.
+ * scale[3] = {input scale, output scale (written), filter scale}, host memory. group must be 1. */
+EE convolution_transform_filter_bytes_gfx950(TensorDesc filterDesc, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch);
+EE convolution_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, TensorDesc *ftmDesc, void *filterTransformed, Arch arch);
+EE convolution_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec convParamSpec, ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch);
+EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwiseInput, TensorDesc filterDesc,
+    const void *filter, ConvolutionParamSpec convParamSpec, ConvolutionForwardAlgorithm algorithm, TensorDesc biasDesc,
+    const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, F32 *scale,
+    ActivationParamSpec activationDesc, Arch arch);
+
+/* ---- 1-bit (XNOR / DoReFa) convolution ---------------------------------------------- */
+/* compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72 (convolution_bnn), filter transform
+ * compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86, tmp bytes
+ * compute/tensor/src/cpu/arm/convolution.cpp:413-455, naive semantics
+ * compute/tensor/src/cpu/general/convolution.cpp:141-178. The reference reaches these through the
+ * same convolution_* dispatchers when filterDesc.dt is DT_BIN01 / DT_BIN11; here they are separate
+ * symbols with convolution_bnn's own argument list (+ Arch).
+ *   filter : DT_BIN11 (bit 1 = +1, bit 0 = -1) or DT_BIN01 (bit = value), [oc, ic, fh, fw], MSB first;
+ *            DF_NCHW bit string or the reference's DF_NCHWN16C8 bytes -> blob tagged DF_NCHWN16C8,
+ *            oc*ic*fh*fw/8 bytes (the reference's size; the byte order inside is this library's).
+ *   input  : DF_NCHWC8, DT_F32 (binarised on the fly: x >= 0 for BIN11, x >= 0.5 for BIN01, the
+ *            thresholds of the reference's fp16 packing) or already packed bits of the filter's type,
+ *            [n][ic/8][ih][iw] bytes, MSB = first channel of each 8.
+ *   output : DF_NCHWC8, DT_F32 = fma(S, scale[oc], bias[oc]) or DT_I32 = S, the integer sum
+ *            (XNOR: fh*fw*ic - 2*popcount(x ^ w) with padding counted as -1; DoReFa: popcount(x & w)).
+ *   fp32 stands where the reference's ARM kernels use fp16. ic and oc must be multiples of 32,
+ *   group 1, no dilation. scale / bias: fp32 [oc], same pointer convention as the other buffers. */
+EE convolution_transform_filter_bytes_bnn_gfx950(TensorDesc filterDesc, U32 *bytes, Arch arch);
+EE convolution_transform_filter_bnn_gfx950(TensorDesc filterDesc, const void *filter, TensorDesc *ftmDesc,
+    void *filterTransformed, Arch arch);
+EE convolution_infer_forward_tmp_bytes_bnn_gfx950(TensorDesc inputDesc, ConvolutionParamSpec convParamSpec, U32 *bytes,
+    Arch arch);
+EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc filterDesc, const void *filter,
+    ConvolutionParamSpec convParamSpec, TensorDesc scaleDesc, const void *scale, TensorDesc biasDesc, const void *bias,
+    U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, ActivationParamSpec activationDesc, Arch arch);
+
 /* ---- asynchronous forms with device-resident scales (AMD_GFX950_DEVICE only) -------- */
 /* No counterpart in the reference: Bolt keeps a tensor's scale in host memory
  * (common/memory/include/tensor.hpp:83-96). These keep it on the GPU so that

@@ -186,6 +186,71 @@ typedef enum {
     CONVOLUTION_ALGORITHM_FORCE_U32 = 0x7fffffff
 } ConvolutionForwardAlgorithm;
 
+/* common/uni/include/parameter_spec.h:94-101, :25-34, :230-247, :259-286 (all inside #pragma pack(8),
+ * every member 4 bytes wide except the 8-byte ActivationSpec union) */
+typedef enum {
+    CONVOLUTION_POINTWISE = 0,
+    CONVOLUTION_DILATION = 1,
+    CONVOLUTION_DEPTHWISE = 2,
+    CONVOLUTION_DEPTHWISE_POINTWISE = 3,
+    CONVOLUTION_DECONVOLUTION = 4,
+    CONVOLUTION_DEPTHWISE_DECONVOLUTION = 5,
+    CONVOLUTION_MODE_FORCE_U32 = 0x7fffffff
+} ConvolutionMode;
+
+typedef enum {
+    ROUND_CEIL = 0,
+    ROUND_FLOOR = 1,
+    ROUND_TF_SAME = 2,
+    ROUND_TF_VALID = 3,
+    ROUND_PREFER_FLOOR = 4,
+    ROUND_PREFER_CEIL = 5,
+    ROUND_SAME_UPPER = 6,
+    ROUND_SAME_LOWER = 7,
+    ROUND_MODE_FORCE_U32 = 0x7fffffff
+} RoundMode;
+
+typedef union {
+    struct {
+        float neg_slope;
+    } relu_spec;
+    struct {
+        float min;
+        float max;
+    } clip_spec;
+} ActivationSpec;
+
+#pragma pack(8)
+typedef struct {
+    U32 num_outputs;
+    U32 kernel_t;
+    U32 kernel_h;
+    U32 kernel_w;
+    U32 stride_t;
+    U32 stride_h;
+    U32 stride_w;
+    U32 pad_before;
+    U32 pad_after;
+    U32 pad_top;
+    U32 pad_bottom;
+    U32 pad_left;
+    U32 pad_right;
+    U32 group;
+    U32 dilatedRate_t;
+    U32 dilatedRate_h;
+    U32 dilatedRate_w;
+    U32 num_outputs_origin;
+    ConvolutionMode convolution_type;
+    ActivationMode dw_activation_type;
+    ActivationMode pw_activation_type;
+    ActivationSpec activation_spec;
+    RoundMode round_mode;
+    U32 output_pad_t;
+    U32 output_pad_h;
+    U32 output_pad_w;
+} ConvolutionParamSpec;
+#pragma pack()
+
 static inline U32 bolt_align(U32 x, U32 a)
 {
     return a == 0 ? 0 : (x + a - 1) / a * a;
