@@ -1,0 +1,118 @@
+"""The HIP path against the committed golden vectors (bytes returned by the reference's compiled x86
+AVX-512-VNNI path for seeded inputs, tests/golden/*.npz), through the C-ABI, bit for bit."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from bolt_amd import capi, host, host_conv  # noqa: E402
+from bolt_amd.capi import (DF_NCHWC8, DF_NCHWC16, DF_NKN32K4, DF_NKNxKx, DF_NORMAL, DF_TRANSPOSE, DT_F32, DT_I8, DT_I32,
+                           DT_U8_Q)  # noqa: E402
+from test_golden import load, same  # noqa: E402
+from test_gpu_blas import dev, run_mmm, run_mvm, torch_mod  # noqa: E402,F401
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_mmm_golden(torch_mod, device_mode):
+    g = load("mmm")
+    for i, (M, K, N) in enumerate(g["shapes"]):
+        M, K, N = int(M), int(K), int(N)
+        print("mmm golden", device_mode, M, K, N, flush=True)
+        A, W, off, ob, cin, s = g[f"A{i}"], g[f"W{i}"], g[f"offsetC{i}"], g[f"ob{i}"], g[f"cin{i}"], g[f"s{i}"]
+        blob, _, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+        assert same(blob[rhs:rhs + 4 * N].view(np.int32), off)
+        assert same(host.quantize_bias_offsetC(g[f"bias{i}"], off, s, N), ob)
+        r = lambda *a: run_mmm(torch_mod, device_mode, *a)     # noqa: E731
+        assert same(r(A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, ob, cin, DT_I32, None), g[f"i32_{i}"])
+        assert same(r(A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, ob, np.zeros((M, N), np.float32), DT_F32, [s]), g[f"f32_{i}"])
+        if f"i32_tA_{i}" in g.files:
+            assert same(r(np.ascontiguousarray(A.T), DF_TRANSPOSE, blob, DF_NKNxKx, M, K, N, off, cin, DT_I32, None),
+                        g[f"i32_tA_{i}"])
+        assert same(r(A, DF_NORMAL, np.ascontiguousarray(W.T), DF_NORMAL, M, K, N, None, cin, DT_I32, None),
+                    g[f"i32_unpacked_{i}"])
+        assert same(r(A, DF_NORMAL, blob, DF_NKNxKx, M, K, N, ob, np.zeros((M, N), np.uint8), DT_U8_Q,
+                      [-1.0, float(g[f"u8scale{i}"])]), g[f"u8_{i}"])
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_mvm_golden(torch_mod, device_mode):
+    g = load("mvm")
+    for i, (N, K) in enumerate(g["shapes"]):
+        N, K = int(N), int(K)
+        print("mvm golden", device_mode, N, K, flush=True)
+        W, x, off, yin, s = g[f"W{i}"], g[f"x{i}"], g[f"offsetC{i}"], g[f"yin{i}"], g[f"s{i}"]
+        blob, _ = host.mvm_transform_weight(W, DF_NORMAL, N, K)
+        pd = host.mvm_desc(DF_NKN32K4, N, K)
+        r = lambda *a, **k: run_mvm(torch_mod, device_mode, *a, **k)     # noqa: E731
+        assert same(r(blob, pd, x, N, K, off, yin, None), g[f"i32_{i}"])
+        assert same(r(blob, pd, x, N, K, off, np.zeros(N, np.float32), [s], ydt=DT_F32), g[f"f32_{i}"])
+        assert same(r(W, host.mvm_desc(DF_NORMAL, N, K), x, N, K, None, yin, None), g[f"i32_unpacked_{i}"])
+        assert same(r(np.ascontiguousarray(W.T), host.mvm_desc(DF_TRANSPOSE, N, K), x, N, K, None, yin, None),
+                    g[f"i32_unpackedT_{i}"])
+        assert same(r(blob, pd, x, N, K, off, np.zeros(N, np.uint8), [-1.0, float(g[f"u8scale{i}"])], ydt=DT_U8_Q),
+                    g[f"u8_{i}"])
+        assert same(r(g[f"uA{i}"], host.mvm_desc(DF_NORMAL, N, K, DT_U8_Q), g[f"uv{i}"], N, K, None, yin, None, vdt=DT_I8),
+                    g[f"u8mat_i32_{i}"])
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_quantize_golden(torch_mod, device_mode):
+    torch = torch_mod
+    g = load("quantize")
+
+    def put(a):
+        return dev(torch, a) if device_mode else np.ascontiguousarray(a)
+
+    def get(t):
+        if device_mode:
+            capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+            return t.cpu().numpy()
+        return t
+
+    for i, n in enumerate(g["ns"]):
+        print("quantize golden", device_mode, int(n), flush=True)
+        x, acc, u = g[f"x{i}"], g[f"acc{i}"], g[f"u{i}"]
+        for nm, qdt in (("u8", DT_U8_Q), ("i8", DT_I8)):
+            for tag, sc, mode in (("dyn", -1.0, 0), ("static", 20.0, 1), ("floor", 1000.0, 0)):
+                s = [sc]
+                q = get(host.quantize(put(x), DT_F32, qdt, s, mode))
+                assert same(q, g[f"{nm}_{tag}_{i}"]) and s[0] == g[f"{nm}_{tag}_s{i}"][0], (nm, tag, n)
+            for tag, s0 in (("i32dyn", -1.0), ("i32static", 0.02)):
+                s = [s0, 37.5]
+                q = get(host.quantize(put(acc), DT_I32, qdt, s))
+                assert same(q, g[f"{nm}_{tag}_{i}"]) and same(np.array(s, np.float32), g[f"{nm}_{tag}_s{i}"]), (nm, tag, n)
+        assert same(get(host.quantize(put(u), DT_U8_Q, DT_I8, [1.0])), g[f"u_to_i8_{i}"])
+        assert same(get(host.dequantize(put(acc), DT_I32, 37.5)), g[f"deq_i32_{i}"])
+        assert same(get(host.dequantize(put(u), DT_U8_Q, 11.25)), g[f"deq_u8_{i}"])
+        assert same(get(host.quantize_bias_offsetC(put(g[f"b{i}"]), put(g[f"o{i}"]), 123.456, int(n))), g[f"bias_offsetC_{i}"])
+        assert same(get(host.quantize_bias_offsetC(put(g[f"b{i}"]), None, 123.456, int(n))), g[f"bias_only_{i}"])
+        assert same(get(host.requantize(put(g[f"r{i}"]), 10.0, 7.3)), g[f"requant_{i}"])
+    for nm, qdt in (("u8", DT_U8_Q), ("i8", DT_I8)):
+        s = [-1.0]
+        q = get(host.quantize(put(g["ties"]), DT_F32, qdt, s))
+        assert s[0] == 1.0 and same(q, g[f"ties_{nm}"])
+    assert same(get(host.quantize_bias_offsetC(put(g["bias_ties"]), None, 8.0, 256)), g["bias_ties_out"])
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_conv_golden(torch_mod, device_mode):
+    torch = torch_mod
+    g = load("conv_int8")
+    for i, case in enumerate(g["cases"]):
+        n, ic, ih, iw, oc, fh, fw, stride, pad = (int(v) for v in case)
+        print("conv golden", device_mode, case, flush=True)
+        p = capi.conv_param_spec(oc, fh, fw, stride, pad)
+
+        def put(a):
+            return dev(torch, a) if device_mode else np.ascontiguousarray(a)
+        blob, ftm = host_conv.transform_filter(put(g[f"W{i}"]), oc, ic, fh, fw, p)
+        for relu in (0, 1):
+            for nm, odt in (("u8", DT_U8_Q), ("f32", DT_F32)):
+                sc = [g[f"sI{i}"], -1.0, g[f"sF{i}"]]
+                out = host_conv.convolution(put(g[f"xq{i}"]), DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad,
+                                            put(g[f"bias{i}"]), sc, bool(relu), odt, DF_NCHWC16)
+                if device_mode:
+                    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+                    out = out.cpu().numpy()
+                assert same(np.array(sc, np.float32), g[f"{nm}_relu{relu}_scale{i}"]), (case, nm, relu)
+                assert same(out, g[f"{nm}_relu{relu}_{i}"]), (case, nm, relu)
