@@ -16,7 +16,11 @@
 #ifndef BOLT_GFX950_H
 #define BOLT_GFX950_H
 
+/* Inside Bolt, whose own headers already define TensorDesc, EE, Arch ..., define
+ * BOLT_GFX950_NO_TYPES before including this file so only the prototypes are taken. */
+#ifndef BOLT_GFX950_NO_TYPES
 #include "bolt_types.h"
+#endif
 #include <stddef.h>
 
 #ifdef __cplusplus
@@ -30,8 +34,10 @@ EE bolt_gfx950_init(void);
 EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
-/* Tuning knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1 = 256x256 block
- * tiles, 2 = 128x128 block tiles (tiled kernels need K % 16 == 0; otherwise the general one runs). */
+/* Tuning / test knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1-2 the
+ * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 3-10 the LDS-DMA kernel
+ * variants (need K % 64 == 0); a variant whose shape requirement fails falls back to the general
+ * kernel. Every variant returns the same bytes. */
 EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);
