@@ -69,7 +69,7 @@ EE ensure_init()
     if (e != hipSuccess || n == 0) {
         return fail(NOT_SUPPORTED, "no HIP device available", e);
     }
-    e = hipMalloc((void **)&c.ws, 256);
+    e = hipMalloc((void **)&c.ws, (kWsWords + 64) * sizeof(uint32_t));
     if (e != hipSuccess) {
         return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
     }
@@ -821,7 +821,7 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     } else if (!aligned4(data) && ddt != DT_U8_Q) {
         return fail(NOT_SUPPORTED, "device data must be 4-byte aligned");
     }
-    float *dscale = (float *)(c.ws + 8);
+    float *dscale = (float *)(c.ws + kWsWords);
     bool read_back = false;
     if (f32in) {
         const bool dynamic = (!mode || *scale <= 0);
@@ -1125,7 +1125,7 @@ static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataForm
     }
     e = SUCCESS;
     if (cdt != odt) {  // :477-486 -- dynamic requantisation of the int32 result
-        float *dscale = (float *)(c.ws + 8);
+        float *dscale = (float *)(c.ws + kWsWords);
         HIP_TRY(launch_absmax_i32((const int32_t *)dst, M * N, c.ws, c.stream));
         HIP_TRY(launch_requant_i32((const int32_t *)dst, M * N, output, 1, c.ws, *outputScale, scaleO, dscale, c.stream));
         HIP_TRY(hipMemcpyAsync(outputScale, dscale, 4, hipMemcpyDeviceToHost, c.stream));
@@ -1362,8 +1362,8 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // requantisation (:2797-2806); the new output scale goes back to the host
     g.C = t + accOff;
     g.conv.absmax = c.ws;
-    float *dscale = (float *)(c.ws + 8);
-    HIP_TRY(launch_fill_u32(c.ws, 1, 0, c.stream));
+    float *dscale = (float *)(c.ws + kWsWords);
+    HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
     HIP_TRY(launch_conv_u8s8(g, c.stream));
     HIP_TRY(launch_requant_i32((const int32_t *)g.C, g.M * g.N, output, 1, c.ws, -1.0f, scaleO, dscale, c.stream));
     HIP_TRY(hipMemcpyAsync(&scale[1], dscale, 4, hipMemcpyDeviceToHost, c.stream));

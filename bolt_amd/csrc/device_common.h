@@ -114,4 +114,42 @@ __device__ __forceinline__ int wave_reduce_max_i(int v)
     return v;
 }
 
+// ---- tensor-wide max through device scratch words --------------------------------------------------
+// Atomics from many workgroups to ONE address serialise at the memory side (the eight XCDs' L2s
+// are not coherent with each other), ~10 ns apiece. The running max is therefore spread over
+// kWsSlots words, one per 64-byte line; a producer workgroup folds its result into slot
+// (workgroup % kWsSlots), every consumer wave reads all slots with one load per lane.
+constexpr uint32_t kWsSlots = 64, kWsStride = 16, kWsWords = kWsSlots * kWsStride;
+
+__device__ __forceinline__ void ws_fold_max(uint32_t *ws, uint32_t group, int v)
+{
+    if (v != 0) {
+        atomicMax((int *)ws + (group % kWsSlots) * kWsStride, v);
+    }
+}
+
+// Workgroup-wide max of non-negative ints, folded into the slot of this workgroup. `red` = one
+// LDS word per wave. Values are non-negative floats' bit patterns or non-negative ints, so the
+// integer order is the wanted order either way.
+__device__ __forceinline__ void ws_block_fold_max(uint32_t *ws, int v, int *red)
+{
+    v = wave_reduce_max_i(v);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+    if (lane == 0) {
+        red[wave] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < waves; ++w) {
+            v = red[w] > v ? red[w] : v;
+        }
+        ws_fold_max(ws, blockIdx.x + blockIdx.y * gridDim.x, v);
+    }
+}
+
+__device__ __forceinline__ int ws_read_max(const uint32_t *ws)
+{
+    return wave_reduce_max_i((int)ws[(threadIdx.x & (kWsSlots - 1)) * kWsStride]);
+}
+
 }  // namespace bg

@@ -319,8 +319,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     if (CONV && MODE == EPI_I32 && a.conv.absmax) {
         // max |acc| of the whole output tensor, for the dynamic requantisation that follows
         lane_max = wave_reduce_max_i(lane_max);
-        if (lane == 0 && lane_max != 0) {
-            atomicMax((int *)a.conv.absmax, lane_max);
+        if (lane == 0) {
+            ws_fold_max(a.conv.absmax, blockIdx.x * 8 + wave, lane_max);
         }
     }
 }

@@ -46,44 +46,48 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st)
 template <int VEC>
 __global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict__ x, uint32_t n, uint32_t *ws)
 {
+    __shared__ int red[4];
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t stride = gridDim.x * blockDim.x;
     float m = 0.0f;
+#define BG_AMAX(v)                 \
+    {                              \
+        float a_ = fabsf(v);       \
+        m = (a_ > m) ? a_ : m;     \
+    }
     if (VEC) {
         const uint32_t n4 = n / 4;
         const v4f *x4 = (const v4f *)x;
-        for (uint32_t i = tid; i < n4; i += stride) {
-            v4f v = x4[i];
-            float a = fabsf(v.x), b = fabsf(v.y), c = fabsf(v.z), d = fabsf(v.w);
-            m = (a > m) ? a : m;
-            m = (b > m) ? b : m;
-            m = (c > m) ? c : m;
-            m = (d > m) ? d : m;
+        uint32_t i = tid;
+        for (; i + 3 * stride < n4; i += 4 * stride) {  // four independent 16-byte loads in flight
+            v4f a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
+            BG_AMAX(a.x) BG_AMAX(a.y) BG_AMAX(a.z) BG_AMAX(a.w) BG_AMAX(b.x) BG_AMAX(b.y) BG_AMAX(b.z) BG_AMAX(b.w)
+            BG_AMAX(c.x) BG_AMAX(c.y) BG_AMAX(c.z) BG_AMAX(c.w) BG_AMAX(d.x) BG_AMAX(d.y) BG_AMAX(d.z) BG_AMAX(d.w)
         }
-        for (uint32_t i = n4 * 4 + tid; i < n; i += stride) {
-            float a = fabsf(x[i]);
-            m = (a > m) ? a : m;
+        for (; i < n4; i += stride) {
+            v4f v = x4[i];
+            BG_AMAX(v.x) BG_AMAX(v.y) BG_AMAX(v.z) BG_AMAX(v.w)
+        }
+        for (uint32_t j = n4 * 4 + tid; j < n; j += stride) {
+            BG_AMAX(x[j])
         }
     } else {
         for (uint32_t i = tid; i < n; i += stride) {
-            float a = fabsf(x[i]);
-            m = (a > m) ? a : m;
+            BG_AMAX(x[i])
         }
     }
-    uint32_t bits = __float_as_uint(m);
-    bits = (uint32_t)wave_reduce_max_i((int)bits);  // non-negative floats: integer order == float order
-    if ((threadIdx.x & 63) == 0 && bits != 0) {
-        atomicMax(ws, bits);
-    }
+#undef BG_AMAX
+    // non-negative floats: integer order == float order
+    ws_block_fold_max(ws, (int)__float_as_uint(m), red);
 }
 
 hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st)
 {
-    hipError_t e = launch_fill_u32(ws, 1, 0, st);
+    hipError_t e = launch_fill_u32(ws, kWsWords, 0, st);
     if (e != hipSuccess || n == 0) {
         return e;
     }
-    const uint32_t blocks = grid_for(n, 16, 256, 2048);
+    const uint32_t blocks = grid_for(n, 16, 256, 1024);
     if (((uintptr_t)x & 15) == 0) {
         hipLaunchKernelGGL((absmax_f32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, ws);
     } else {
@@ -95,27 +99,48 @@ hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream
 // avx512/quantize.cpp:70-119: vpabsd + vpmaxsd, so |INT32_MIN| stays negative and never wins.
 __global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t *__restrict__ x, uint32_t n, uint32_t *ws)
 {
+    __shared__ int red[4];
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t stride = gridDim.x * blockDim.x;
     int m = 0;
-    for (uint32_t i = tid; i < n; i += stride) {
-        int v = x[i];
-        int a = (v == (int)0x80000000) ? v : (v < 0 ? -v : v);
-        m = (a > m) ? a : m;
+#define BG_AMAX(v)                                                       \
+    {                                                                    \
+        int v_ = (v);                                                    \
+        int a_ = (v_ == (int)0x80000000) ? v_ : (v_ < 0 ? -v_ : v_);     \
+        m = (a_ > m) ? a_ : m;                                           \
     }
-    m = wave_reduce_max_i(m);
-    if ((threadIdx.x & 63) == 0 && m != 0) {
-        atomicMax((int *)ws, m);
+    if (((uintptr_t)x & 15) == 0) {
+        const uint32_t n4 = n / 4;
+        const v4i *x4 = (const v4i *)x;
+        uint32_t i = tid;
+        for (; i + 3 * stride < n4; i += 4 * stride) {
+            v4i a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
+            BG_AMAX(a.x) BG_AMAX(a.y) BG_AMAX(a.z) BG_AMAX(a.w) BG_AMAX(b.x) BG_AMAX(b.y) BG_AMAX(b.z) BG_AMAX(b.w)
+            BG_AMAX(c.x) BG_AMAX(c.y) BG_AMAX(c.z) BG_AMAX(c.w) BG_AMAX(d.x) BG_AMAX(d.y) BG_AMAX(d.z) BG_AMAX(d.w)
+        }
+        for (; i < n4; i += stride) {
+            v4i v = x4[i];
+            BG_AMAX(v.x) BG_AMAX(v.y) BG_AMAX(v.z) BG_AMAX(v.w)
+        }
+        for (uint32_t j = n4 * 4 + tid; j < n; j += stride) {
+            BG_AMAX(x[j])
+        }
+    } else {
+        for (uint32_t i = tid; i < n; i += stride) {
+            BG_AMAX(x[i])
+        }
     }
+#undef BG_AMAX
+    ws_block_fold_max(ws, m, red);
 }
 
 hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st)
 {
-    hipError_t e = launch_fill_u32(ws, 1, 0, st);
+    hipError_t e = launch_fill_u32(ws, kWsWords, 0, st);
     if (e != hipSuccess || n == 0) {
         return e;
     }
-    hipLaunchKernelGGL(absmax_i32_kernel, dim3(grid_for(n, 8, 256, 2048)), dim3(256), 0, st, x, n, ws);
+    hipLaunchKernelGGL(absmax_i32_kernel, dim3(grid_for(n, 16, 256, 1024)), dim3(256), 0, st, x, n, ws);
     return hipGetLastError();
 }
 
@@ -154,7 +179,7 @@ __device__ __forceinline__ unsigned q4(v4f v, float s)
 __device__ __forceinline__ float resolve_scale(float s_in, int mode, const uint32_t *ws)
 {
     if (!mode || s_in <= 0) {
-        float m = __uint_as_float(ws[0]);
+        float m = __uint_as_float((uint32_t)ws_read_max(ws));
         float dyn = (m == 0.0f) ? 1.0f : 127.0f / m;
         return (s_in > dyn) ? s_in : dyn;
     }
@@ -226,7 +251,7 @@ __global__ __launch_bounds__(256) void requant_i32_kernel(const int32_t *__restr
     float r = 0.0f;
     float out0 = s0;
     if (s0 < 0 && s1 > 0) {
-        int m = (int)ws[0];
+        int m = ws_read_max(ws);
         r = (m == 0) ? 1.0f : 127.0f / (float)m;
         out0 = s1 * r;
     } else if (s0 > 0 && s1 > 0) {
@@ -237,21 +262,31 @@ __global__ __launch_bounds__(256) void requant_i32_kernel(const int32_t *__restr
         *ds_out = out0;
     }
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = tid; i < n; i += stride) {
-        float t = (float)x[i] * r;
-        if (TO_U8) {
-            float u = t + 128.0f;
-            q[i] = (uint8_t)usat8_u(rne_i32(u));
-        } else {
-            q[i] = (uint8_t)ssat8(rne_i32(t));
+#define BG_RQ(v) ((unsigned)(TO_U8 ? usat8_u(rne_i32((float)(v) * r + 128.0f)) : ssat8(rne_i32((float)(v) * r))) & 0xffu)
+#define BG_RQ4(v) (BG_RQ(v.x) | (BG_RQ(v.y) << 8) | (BG_RQ(v.z) << 16) | (BG_RQ(v.w) << 24))
+    uint32_t done = 0;
+    if ((((uintptr_t)x | (uintptr_t)q) & 15) == 0) {
+        const uint32_t n16 = n / 16;
+        const v4i *x4 = (const v4i *)x;
+        v4i *q16 = (v4i *)q;
+        for (uint32_t i = tid; i < n16; i += stride) {
+            v4i a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+            v4i o = {(int)BG_RQ4(a), (int)BG_RQ4(b), (int)BG_RQ4(c), (int)BG_RQ4(d)};
+            q16[i] = o;
         }
+        done = n16 * 16;
     }
+    for (uint32_t i = done + tid; i < n; i += stride) {
+        q[i] = (uint8_t)BG_RQ(x[i]);
+    }
+#undef BG_RQ4
+#undef BG_RQ
 }
 
 hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s0,
     float s1, float *ds_out, hipStream_t st)
 {
-    const uint32_t blocks = grid_for(n, 4, 256, 8192);
+    const uint32_t blocks = grid_for(n, 16, 256, 8192);
     if (to_u8) {
         hipLaunchKernelGGL((requant_i32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s0, s1,
             ds_out);
