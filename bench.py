@@ -170,6 +170,29 @@ def other_kernels(L, capi, host, torch, dev):
     res["bnn_c5_xnor"] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
                           "gbps": 53061632 / t / 1e6}
 
+    # -- C4: BERT-base int8 encoder layer, batch 32 x seq 128 (4096 tokens), one C call per layer
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import encoder_layer as ref_layer
+    from bolt_amd.host_encoder import EncoderLayer
+    rs = np.random.default_rng(20240604)
+    batch, seq, hidden, heads, ffn = 32, 128, 768, 12, 3072
+    P = {}
+    for name, Nn, Kk in (("qkv", 3 * hidden, hidden), ("o", hidden, hidden), ("1", ffn, hidden), ("2", hidden, ffn)):
+        P["w" + name], P["s" + name] = ref_layer.quantize_weight_per_channel(   # load-time weight quantisation
+            (rs.standard_normal((Nn, Kk)) * 0.02).astype(np.float32))
+        P["b" + name] = np.zeros(Nn, np.float32)
+    for k in ("ln1", "ln2"):
+        P[k + "_g"], P[k + "_b"] = np.ones(hidden, np.float32), np.zeros(hidden, np.float32)
+    layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
+    hx = torch.randn((batch * seq, hidden), device=dev, generator=g)
+    hy = torch.empty_like(hx)
+    t = timed(lambda: layer(hx, hy), 50)
+    gemm_ops = 2.0 * batch * seq * hidden * (3 * hidden + hidden + 2 * ffn)
+    res["bert_base_layer_c4"] = {"ms": t, "tokens_per_s": batch * seq / (t * 1e-3), "int8_gemm_tops": gemm_ops / t / 1e9,
+                                 "config": "hidden 768, 12 heads, FFN 3072, seq 128, batch 32; int8 GEMMs with per-channel "
+                                           "weight scales, dynamic per-tensor activation quantisation, fp32 attention / "
+                                           "LayerNorm / GELU"}
+
     # -- quantize family at the BERT FFN size (4096 x 3072)
     cnt = 4096 * 3072
     xf = torch.randn(cnt, device=dev, generator=g)

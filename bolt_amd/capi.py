@@ -91,6 +91,13 @@ _vp, _u32, _f32p, _u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTE
 _TDp = C.POINTER(TensorDesc)
 
 # name -> (restype, argtypes); every symbol include/bolt_gfx950.h declares
+class BoltEncoderLayerInt8(C.Structure):
+    _fields_ = ([(n, C.c_uint32) for n in ("batch", "seq", "hidden", "heads", "ffn")] +
+                [(n, C.c_void_p) for n in ("wqkv", "wo", "w1", "w2")] +
+                [(n, C.POINTER(C.c_float)) for n in ("sqkv", "so", "s1", "s2", "bqkv", "bo", "b1", "b2", "ln1_gamma",
+                                                     "ln1_beta", "ln2_gamma", "ln2_beta")])
+
+
 SIGNATURES = {
     "bolt_gfx950_init": (C.c_int, []),
     "bolt_gfx950_set_stream": (C.c_int, [_vp]),
@@ -134,6 +141,14 @@ SIGNATURES = {
     "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),
     "convolution_bnn_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, ConvolutionParamSpec, TensorDesc, _vp,
                                          TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, ActivationParamSpec, C.c_int]),
+    "bolt_gfx950_encoder_layer_int8_workspace_bytes": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),
+                                                                 C.POINTER(C.c_size_t)]),
+    "bolt_gfx950_encoder_layer_int8_workspace_layout": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),
+                                                                  C.POINTER(C.c_size_t)]),
+    "bolt_gfx950_encoder_layer_int8": (C.c_int, [C.POINTER(BoltEncoderLayerInt8), _vp, _vp, _vp, C.c_size_t]),
+    "bolt_gfx950_attention_f32": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _vp]),
+    "bolt_gfx950_add_layernorm_f32": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "bolt_gfx950_gelu_f32": (C.c_int, [_vp, C.c_size_t]),
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

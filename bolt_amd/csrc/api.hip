@@ -1734,6 +1734,205 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     return SUCCESS;
 }
 
+// ---- BERT-style int8 encoder layer --------------------------------------------------------------------
+namespace {
+struct EncoderPlan {
+    size_t ws, scales, xq, qkv, ctx, ao, h1, f, o, total;
+};
+
+EncoderPlan encoder_plan(const BoltEncoderLayerInt8 &L)
+{
+    const size_t T = (size_t)L.batch * L.seq, H = L.hidden, F = L.ffn;
+    EncoderPlan p;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t at = off;
+        off += (bytes + 255) / 256 * 256;
+        return at;
+    };
+    p.ws = take(4 * kWsWords * sizeof(uint32_t));
+    p.scales = take(64);
+    p.xq = take(T * (F > H ? F : H));  // one u8 buffer reused by the four quantised activations
+    p.qkv = take(T * 3 * H * 4);
+    p.ctx = take(T * H * 4);
+    p.ao = take(T * H * 4);
+    p.h1 = take(T * H * 4);
+    p.f = take(T * F * 4);
+    p.o = take(T * H * 4);
+    p.total = off;
+    return p;
+}
+
+EE encoder_check(const BoltEncoderLayerInt8 *L)
+{
+    if (!L) {
+        return NULL_POINTER;
+    }
+    if (!L->wqkv || !L->wo || !L->w1 || !L->w2 || !L->sqkv || !L->so || !L->s1 || !L->s2 || !L->ln1_gamma || !L->ln1_beta ||
+        !L->ln2_gamma || !L->ln2_beta) {
+        return NULL_POINTER;
+    }
+    if (L->batch == 0 || L->seq == 0 || L->heads == 0 || L->hidden != L->heads * 64 || L->ffn == 0 || L->ffn % 4 != 0 ||
+        L->hidden > 2048) {
+        return NOT_SUPPORTED;
+    }
+    if ((uint64_t)L->batch * L->seq * (L->ffn > 3 * L->hidden ? L->ffn : 3 * L->hidden) > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    return SUCCESS;
+}
+}  // namespace
+
+EE bolt_gfx950_encoder_layer_int8_workspace_bytes(const BoltEncoderLayerInt8 *layer, size_t *bytes)
+{
+    EE e = encoder_check(layer);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    *bytes = encoder_plan(*layer).total;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_encoder_layer_int8_workspace_layout(const BoltEncoderLayerInt8 *layer, size_t *offsets)
+{
+    EE e = encoder_check(layer);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!offsets) {
+        return NULL_POINTER;
+    }
+    const EncoderPlan p = encoder_plan(*layer);
+    offsets[0] = p.qkv;
+    offsets[1] = p.ctx;
+    offsets[2] = p.ao;
+    offsets[3] = p.h1;
+    offsets[4] = p.f;
+    offsets[5] = p.o;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float *hidden, float *out, void *workspace,
+    size_t workspaceBytes)
+{
+    EE e = encoder_check(layer);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!hidden || !out || !workspace) {
+        return NULL_POINTER;
+    }
+    const BoltEncoderLayerInt8 &L = *layer;
+    const EncoderPlan p = encoder_plan(L);
+    if (workspaceBytes < p.total) {
+        return NOT_MATCH;
+    }
+    if (((uintptr_t)workspace & 255) || ((uintptr_t)hidden & 15) || ((uintptr_t)out & 15)) {
+        return fail(NOT_SUPPORTED, "workspace must be 256-byte aligned, hidden / out 16-byte aligned");
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    hipStream_t st = ctx().stream;
+    U8 *w = (U8 *)workspace;
+    const U32 T = L.batch * L.seq, H = L.hidden, F = L.ffn;
+    uint32_t *ws0 = (uint32_t *)(w + p.ws), *ws1 = ws0 + kWsWords, *ws2 = ws1 + kWsWords, *ws3 = ws2 + kWsWords;
+    float *sc = (float *)(w + p.scales);
+    uint8_t *xq = w + p.xq;
+    float *qkv = (float *)(w + p.qkv), *cx = (float *)(w + p.ctx), *ao = (float *)(w + p.ao), *h1 = (float *)(w + p.h1),
+          *f = (float *)(w + p.f), *o = (float *)(w + p.o);
+
+    auto gemm = [&](const uint8_t *A, const void *blob, U32 N, U32 K, const float *dsI, const float *sW, const float *bias,
+                    float *C) -> hipError_t {
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = A;
+        g.lda = K;
+        g.Bp = (const int8_t *)blob;
+        g.M = T;
+        g.N = N;
+        g.K = K;
+        g.comp = (const int32_t *)((const U8 *)blob + packed_matrix_bytes(N, K));
+        g.ob = g.comp;  // no folded bias: the fp32 bias is added in the epilogue
+        g.C = C;
+        g.epi.mode = EPI_F32_CH;
+        g.epi.scaleI = dsI;
+        g.epi.scaleW = sW;
+        g.epi.bias = bias;
+        return launch_gemm_u8s8(g, st);
+    };
+
+    HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
+    // x -> u8 (dynamic per-tensor scale), one quantisation shared by Q, K and V
+    HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st));
+    HIP_TRY(launch_quantize_f32(hidden, T * H, xq, 1, ws0, 0.0f, nullptr, 0, sc + 0, st));
+    HIP_TRY(gemm(xq, L.wqkv, 3 * H, H, sc + 0, L.sqkv, L.bqkv, qkv));
+    HIP_TRY(launch_attention_f32(qkv, L.batch, L.seq, H, L.heads, cx, ws1, st));
+    HIP_TRY(launch_quantize_f32(cx, T * H, xq, 1, ws1, 0.0f, nullptr, 0, sc + 1, st));
+    HIP_TRY(gemm(xq, L.wo, H, H, sc + 1, L.so, L.bo, ao));
+    HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st));
+    HIP_TRY(launch_quantize_f32(h1, T * H, xq, 1, ws2, 0.0f, nullptr, 0, sc + 2, st));
+    HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
+    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st));
+    HIP_TRY(launch_quantize_f32(f, T * F, xq, 1, ws3, 0.0f, nullptr, 0, sc + 3, st));
+    HIP_TRY(gemm(xq, L.w2, H, F, sc + 3, L.s2, L.b2, o));
+    HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_attention_f32(const float *qkv, U32 batch, U32 seq, U32 hidden, U32 heads, float *context)
+{
+    if (!qkv || !context) {
+        return NULL_POINTER;
+    }
+    if (heads == 0 || hidden != heads * 64) {
+        return NOT_SUPPORTED;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(launch_attention_f32(qkv, batch, seq, hidden, heads, context, nullptr, ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_add_layernorm_f32(const float *a, const float *b, const float *gamma, const float *beta, U32 rows,
+    U32 hidden, float *out)
+{
+    if (!a || !gamma || !beta || !out) {
+        return NULL_POINTER;
+    }
+    if (hidden % 4 != 0 || hidden > 2048) {
+        return NOT_SUPPORTED;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(launch_add_layernorm(a, b, gamma, beta, rows, hidden, out, nullptr, ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_gelu_f32(float *x, size_t n)
+{
+    if (!x) {
+        return NULL_POINTER;
+    }
+    if (n % 4 != 0) {
+        return NOT_SUPPORTED;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(launch_gelu_f32(x, n, nullptr, ctx().stream));
+    return SUCCESS;
+}
+
 // ---- device-resident-scale forms ------------------------------------------------------------------
 EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode)
 {

@@ -104,6 +104,15 @@ __device__ __forceinline__ float wave_reduce_max(float v)
     return v;
 }
 
+__device__ __forceinline__ float wave_reduce_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
 __device__ __forceinline__ int wave_reduce_max_i(int v)
 {
 #pragma unroll

@@ -93,6 +93,16 @@ hipError_t launch_bnn_pack_filter(const uint8_t *src, int src_fmt, uint32_t OC, 
     hipStream_t st);
 hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st);
 
+// ---- fp32 neighbours of the int8 GEMMs in an encoder layer (encoder.hip) --------------------------
+// Each takes an optional `ws` (kWsWords scratch words, zeroed by the caller) into which max|out| is folded.
+// qkv rows are [Q | K | V] of 3*H floats; head size 64 (H == heads * 64).
+hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, uint32_t H, uint32_t heads, float *ctx,
+    uint32_t *ws, hipStream_t st);
+// out = LayerNorm(a + b) (b may be null); H % 4 == 0, H <= 2048
+hipError_t launch_add_layernorm(const float *a, const float *b, const float *gamma, const float *beta, uint32_t rows,
+    uint32_t H, float *out, uint32_t *ws, hipStream_t st);
+hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st);
+
 // ---- weight pack --------------------------------------------------------------------------------
 // src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].
 hipError_t launch_pack_mmm(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t K, uint32_t N, int8_t *dst,

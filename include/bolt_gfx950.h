@@ -159,6 +159,46 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     ConvolutionParamSpec convParamSpec, TensorDesc scaleDesc, const void *scale, TensorDesc biasDesc, const void *bias,
     U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, ActivationParamSpec activationDesc, Arch arch);
 
+/* ---- BERT-style int8 encoder layer (device pointers only, asynchronous) ------------- */
+/* One post-LayerNorm transformer encoder layer as Bolt runs it for an int8 BERT model: the four
+ * FullyConnected operators (QKV merged into one, as model_tools' FC+FC merge does for BERT,
+ * model_tools/include/OPOptimizers/FCFCOptimizer.hpp) are int8 GEMMs on activations quantised
+ * per tensor, dynamically (scale 127 / max|x|, quantize_x86 F32 -> U8_Q), with per-output-channel
+ * weight scales; attention scores / softmax / context, residual adds, LayerNorm
+ * (compute/tensor/src/cpu/x86/fp32/layer_norm.cpp:21-67, eps 1e-6) and tanh-GELU
+ * (x86_functions_fp32.h:127-149) are fp32. Head size 64; no attention mask.
+ *   hidden, out : fp32 [batch * seq, hidden]
+ *   w*          : outputs of matrix_matrix_multiply_transform_rhs_gfx950 for [K, N] =
+ *                 [hidden, 3*hidden] (Q | K | V columns), [hidden, hidden], [hidden, ffn], [ffn, hidden]
+ *   s*          : fp32 [N] weight scales, Bolt convention (quantised = real * scale)
+ *   b*          : fp32 [N] biases or NULL;  ln*: fp32 [hidden]
+ * All pointers are device pointers except `layer` itself; the call enqueues ~15 kernels on the
+ * library stream and returns. workspace: 256-byte aligned, size from the query. */
+typedef struct {
+    U32 batch, seq, hidden, heads, ffn;
+    const void *wqkv, *wo, *w1, *w2;
+    const float *sqkv, *so, *s1, *s2;
+    const float *bqkv, *bo, *b1, *b2;
+    const float *ln1_gamma, *ln1_beta, *ln2_gamma, *ln2_beta;
+} BoltEncoderLayerInt8;
+EE bolt_gfx950_encoder_layer_int8_workspace_bytes(const BoltEncoderLayerInt8 *layer, size_t *bytes);
+EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float *hidden, float *out, void *workspace,
+    size_t workspaceBytes);
+/* Inspection hook: byte offsets inside `workspace` of the fp32 intermediates a call leaves behind, in
+ * this order: qkv [T, 3*hidden], attention context [T, hidden], attention output projection
+ * [T, hidden], first LayerNorm output [T, hidden], FFN activation after GELU [T, ffn], FFN output
+ * [T, hidden]. */
+EE bolt_gfx950_encoder_layer_int8_workspace_layout(const BoltEncoderLayerInt8 *layer, size_t *offsets);
+
+/* The layer's fp32 pieces on their own (device pointers, asynchronous):
+ *   attention: qkv rows [Q | K | V] of 3*hidden floats -> ctx = softmax(Q K^T / 8) V per head of 64
+ *   add_layernorm: out = LayerNorm(a + b) (b may be NULL), hidden % 4 == 0, hidden <= 2048
+ *   gelu: in place, n % 4 == 0 */
+EE bolt_gfx950_attention_f32(const float *qkv, U32 batch, U32 seq, U32 hidden, U32 heads, float *ctx);
+EE bolt_gfx950_add_layernorm_f32(const float *a, const float *b, const float *gamma, const float *beta, U32 rows,
+    U32 hidden, float *out);
+EE bolt_gfx950_gelu_f32(float *x, size_t n);
+
 /* ---- asynchronous forms with device-resident scales (AMD_GFX950_DEVICE only) -------- */
 /* No counterpart in the reference: Bolt keeps a tensor's scale in host memory
  * (common/memory/include/tensor.hpp:83-96). These keep it on the GPU so that
