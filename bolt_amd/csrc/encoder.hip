@@ -13,89 +13,148 @@ namespace bg {
 
 // ---- attention ------------------------------------------------------------------------------------
 // qkv: [batch * S][3 * H] fp32 rows (Q | K | V), head h owns columns h*64 .. h*64+63 of each third.
-// One wave = 64 query rows of one (batch, head); a lane keeps its query row and its output row in
-// registers. Key / value rows are the same for every lane of the wave, so they come in through the
-// scalar cache and feed v_fmac as SGPR operands; the dot products run over d = 0..63 in order.
-// Softmax is the streaming form over blocks of 16 keys (running max and sum), mathematically the
-// max-subtracted softmax of the reference.
+// fp32 matrix cores (v_mfma_f32_16x16x4_f32), no LDS: a wave owns 32 queries of one (batch, head) and
+// walks the keys in chunks of 128.
+//   scores^T = K . Q^T   : M = key, N = query, contraction over d. A lane (c = lane % 16, g = lane / 16)
+//                          feeds K[key c][16 s + 4 g + t] and Q[query c][16 s + 4 g + t] for step (s, t):
+//                          one 16-byte load covers four steps, and both operands permute d the same way.
+//   the accumulator of key tile kt then holds score(key 16 kt + 4 g + i, query c), i = 0..3, so the
+//   softmax statistics of a query are an in-lane reduction plus two cross-lane steps (xor 16, 32);
+//   out^T = V^T . P^T    : M = d, N = query, contraction over keys in the order the accumulators
+//                          already have them: step (kt, t) takes P from element t of tile kt and
+//                          V[key 16 kt + 4 g + t][d c] -- no transposition through LDS.
+// Chunks are merged with the streaming (running max / running sum) form of the max-subtracted softmax.
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+
 template <int D>
-__global__ __launch_bounds__(64) void attention_f32_kernel(const float *__restrict__ qkv, uint32_t S, uint32_t H,
+__global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__restrict__ qkv, uint32_t S, uint32_t H,
     float qscale, float *__restrict__ ctx, uint32_t *ws)
 {
-    const uint32_t lane = threadIdx.x;
+    static_assert(D == 64, "head size 64");
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t c = lane & 15, g = lane >> 4;
     const uint32_t h = blockIdx.y, b = blockIdx.z;
-    uint32_t r = blockIdx.x * 64 + lane;
-    const bool live = r < S;
-    r = live ? r : S - 1;
+    const uint32_t q0 = blockIdx.x * 128 + wave * 32;
+    if (q0 >= S) {
+        return;
+    }
     const size_t ld = 3 * (size_t)H;
-    const float *base = qkv + (size_t)b * S * ld + (size_t)h * D;
-    float q[D], o[D];
-    {
-        const v4f *qp = (const v4f *)(base + (size_t)r * ld);
+    const float *Qb = qkv + (size_t)b * S * ld + (size_t)h * D;
+    const float *Kb = Qb + H, *Vb = Qb + 2 * (size_t)H;
+
+    v4f_t qf[2][4];
 #pragma unroll
-        for (int d4 = 0; d4 < D / 4; ++d4) {
-            v4f v = qp[d4];
-            q[4 * d4] = v.x * qscale;
-            q[4 * d4 + 1] = v.y * qscale;
-            q[4 * d4 + 2] = v.z * qscale;
-            q[4 * d4 + 3] = v.w * qscale;
+    for (int nt = 0; nt < 2; ++nt) {
+        uint32_t q = q0 + nt * 16 + c;
+        q = q < S ? q : S - 1;
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+            v4f_t v = *(const v4f_t *)(Qb + (size_t)q * ld + 16 * s4 + 4 * g);
+            qf[nt][s4] = v * qscale;
         }
     }
+    v4f_t o[4][2];
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        o[d] = 0.0f;
+    for (int mt = 0; mt < 4; ++mt) {
+        o[mt][0] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
+        o[mt][1] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
     }
-    float m = -INFINITY, l = 0.0f;
-    constexpr int JB = 16;
-    for (uint32_t j0 = 0; j0 < S; j0 += JB) {
-        float s[JB];
-        float mx = m;
+    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.0f, 0.0f};
+
+    for (uint32_t k0 = 0; k0 < S; k0 += 128) {
+        v4f_t s[8][2];
 #pragma unroll
-        for (int jj = 0; jj < JB; ++jj) {
-            const uint32_t j = (j0 + jj < S) ? j0 + jj : S - 1;
-            const float *kp = base + H + (size_t)j * ld;  // wave-uniform address
-            float acc = 0.0f;
+        for (int kt = 0; kt < 8; ++kt) {
+            s[kt][0] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
+            s[kt][1] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
+            uint32_t key = k0 + kt * 16 + c;
+            key = key < S ? key : S - 1;
+            const float *kp = Kb + (size_t)key * ld + 4 * g;
 #pragma unroll
-            for (int d = 0; d < D; ++d) {
-                acc = __builtin_fmaf(q[d], kp[d], acc);
-            }
-            s[jj] = (j0 + jj < S) ? acc : -INFINITY;
-            mx = fmaxf(mx, s[jj]);
-        }
-        const float corr = __expf(m - mx);  // exp(-inf) = 0 on the first block
-        l *= corr;
+            for (int s4 = 0; s4 < 4; ++s4) {
+                const v4f_t kf = *(const v4f_t *)(kp + 16 * s4);
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            o[d] *= corr;
-        }
-#pragma unroll
-        for (int jj = 0; jj < JB; ++jj) {
-            const uint32_t j = (j0 + jj < S) ? j0 + jj : S - 1;
-            const float p = __expf(s[jj] - mx);
-            l += p;
-            const float *vp = base + 2 * (size_t)H + (size_t)j * ld;
-#pragma unroll
-            for (int d = 0; d < D; ++d) {
-                o[d] = __builtin_fmaf(p, vp[d], o[d]);
+                for (int t = 0; t < 4; ++t) {
+                    s[kt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t], qf[0][s4][t], s[kt][0], 0, 0, 0);
+                    s[kt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t], qf[1][s4][t], s[kt][1], 0, 0, 0);
+                }
             }
         }
-        m = mx;
+        // keys past the end of the sequence do not take part
+#pragma unroll
+        for (int kt = 0; kt < 8; ++kt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (k0 + kt * 16 + 4 * g + i >= S) {
+                    s[kt][0][i] = -INFINITY;
+                    s[kt][1][i] = -INFINITY;
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            float mx = m[nt];
+#pragma unroll
+            for (int kt = 0; kt < 8; ++kt) {
+                mx = fmaxf(mx, fmaxf(fmaxf(s[kt][nt][0], s[kt][nt][1]), fmaxf(s[kt][nt][2], s[kt][nt][3])));
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float corr = __expf(m[nt] - mx);  // exp(-inf) = 0 on the first chunk
+            float sum = 0.0f;
+#pragma unroll
+            for (int kt = 0; kt < 8; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float p = __expf(s[kt][nt][i] - mx);
+                    s[kt][nt][i] = p;
+                    sum += p;
+                }
+            }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            l[nt] = l[nt] * corr + sum;
+            m[nt] = mx;
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                o[mt][nt] = o[mt][nt] * corr;
+            }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 8; ++kt) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                uint32_t key = k0 + kt * 16 + 4 * g + t;
+                key = key < S ? key : S - 1;  // its probability is 0
+                const float *vp = Vb + (size_t)key * ld + c;
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) {
+                    const float vv = vp[16 * mt];
+                    o[mt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, s[kt][0][t], o[mt][0], 0, 0, 0);
+                    o[mt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, s[kt][1][t], o[mt][1], 0, 0, 0);
+                }
+            }
+        }
     }
-    const float inv = 1.0f / l;
     float amax = 0.0f;
-    v4f *op = (v4f *)(ctx + ((size_t)b * S + r) * H + (size_t)h * D);
 #pragma unroll
-    for (int d4 = 0; d4 < D / 4; ++d4) {
-        v4f v = {o[4 * d4] * inv, o[4 * d4 + 1] * inv, o[4 * d4 + 2] * inv, o[4 * d4 + 3] * inv};
-        if (live) {
-            op[d4] = v;
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    for (int nt = 0; nt < 2; ++nt) {
+        const uint32_t q = q0 + nt * 16 + c;
+        const float inv = 1.0f / l[nt];
+        if (q < S) {
+            float *op = ctx + ((size_t)b * S + q) * H + (size_t)h * D + 4 * g;
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                const v4f_t v = o[mt][nt] * inv;
+                *(v4f_t *)(op + 16 * mt) = v;
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+            }
         }
     }
     if (ws) {
         const int bits = wave_reduce_max_i((int)__float_as_uint(amax));
         if (lane == 0) {
-            ws_fold_max(ws, blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), bits);
+            ws_fold_max(ws, (blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 4 + wave, bits);
         }
     }
 }
@@ -109,8 +168,8 @@ hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, ui
     if (H != heads * 64) {
         return hipErrorInvalidValue;
     }
-    const dim3 grid((S + 63) / 64, heads, batch);
-    hipLaunchKernelGGL((attention_f32_kernel<64>), grid, dim3(64), 0, st, qkv, S, H, 0.125f, ctx, ws);
+    const dim3 grid((S + 127) / 128, heads, batch);
+    hipLaunchKernelGGL((attention_f32_kernel<64>), grid, dim3(256), 0, st, qkv, S, H, 0.125f, ctx, ws);
     return hipGetLastError();
 }
 
