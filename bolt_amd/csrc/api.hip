@@ -1318,7 +1318,6 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     const F32 scaleO = scale[0] * scale[2];  // convolution_direct.cpp:2687
     HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
         s.pr, (int8_t *)t, c.stream));
-    HIP_TRY(launch_conv_chunk_table((uint32_t *)(t + tabOff), s.fh, s.fw, s.dh, s.dw, s.Wp, s.ICp, 4, c.stream));
     // filter blob = [offsetC oc*4][packed matrix] (convolution_transform.cpp:36-44 keeps the vector in front)
     const int32_t *offC = (const int32_t *)filter;
     const int8_t *mat = (const int8_t *)filter + (size_t)s.oc * 4;
@@ -1339,7 +1338,10 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     g.conv.Hp = s.Hp;
     g.conv.Wp = s.Wp;
     g.conv.ICp = s.ICp;
-    g.conv.chunk_off = (const uint32_t *)(t + tabOff);
+    g.conv.fh = s.fh;
+    g.conv.fw = s.fw;
+    g.conv.dh = s.dh;
+    g.conv.dw = s.dw;
     g.conv.out_c = (odf == DF_NCHWC8) ? 8 : 16;
     g.conv.relu = relu;
     if (odt == DT_F32) {
@@ -1358,14 +1360,21 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
         scale[1] = scaleO;
         return SUCCESS;
     }
-    // u8: int32 accumulators to tmp with the running max|acc|, then the tensor-wide dynamic
-    // requantisation (:2797-2806); the new output scale goes back to the host
-    g.C = t + accOff;
+    // u8 with the tensor-wide dynamic output scale (:2797-2806). The reference parks int32 accumulators
+    // in tmp, takes their abs-max and requantises; here the convolution runs twice instead -- once
+    // folding max|acc| into the scratch slots without storing anything, once writing u8 with the scale
+    // that maximum gives. The arithmetic per element is the same; the int32 tensor (4 bytes per output,
+    // written and read back) never exists, which is worth more than the repeated matrix work.
+    g.C = nullptr;
     g.conv.absmax = c.ws;
     float *dscale = (float *)(c.ws + kWsWords);
     HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
     HIP_TRY(launch_conv_u8s8(g, c.stream));
-    HIP_TRY(launch_requant_i32((const int32_t *)g.C, g.M * g.N, output, 1, c.ws, -1.0f, scaleO, dscale, c.stream));
+    g.C = output;
+    g.epi.mode = EPI_U8;
+    g.conv.scaleO = scaleO;
+    g.conv.dscale_out = dscale;
+    HIP_TRY(launch_conv_u8s8(g, c.stream));
     HIP_TRY(hipMemcpyAsync(&scale[1], dscale, 4, hipMemcpyDeviceToHost, c.stream));
     HIP_TRY(hipStreamSynchronize(c.stream));
     return SUCCESS;

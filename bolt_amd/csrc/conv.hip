@@ -67,34 +67,6 @@ hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H
     return hipGetLastError();
 }
 
-// chunk q = tap * (ICp / 16) + c16  ->  byte offset of that 16-channel chunk from the pixel's base
-__global__ void conv_chunk_table_kernel(uint32_t *tab, uint32_t chunks, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
-    uint32_t ICp)
-{
-    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= chunks) {
-        return;
-    }
-    const uint32_t cpt = ICp / 16;
-    const uint32_t tap = q / cpt, c16 = q % cpt;
-    const uint32_t kh = tap / fw, kw = tap % fw;
-    tab[q] = ((kh * dh) * Wp + kw * dw) * ICp + c16 * 16;
-}
-
-hipError_t launch_conv_chunk_table(uint32_t *tab, uint32_t fh, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
-    uint32_t ICp, uint32_t pad_to, hipStream_t st)
-{
-    // the K loop walks whole 64-byte tiles: chunks past fh*fw*ICp/16 (K not a multiple of 64) repeat
-    // the last valid offset; their filter bytes are zero
-    const uint32_t chunks = fh * fw * (ICp / 16);
-    const uint32_t padded = align_up(chunks, pad_to);
-    hipLaunchKernelGGL(conv_chunk_table_kernel, dim3((chunks + 63) / 64), dim3(64), 0, st, tab, chunks, fw, dh, dw, Wp, ICp);
-    if (padded > chunks) {
-        hipLaunchKernelGGL(conv_chunk_table_kernel, dim3(1), dim3(64), 0, st, tab + chunks, padded - chunks, 1u, 0u, 0u,
-            Wp, 16u);  // tap 0, c16 = 0..: any in-range offset does
-    }
-    return hipGetLastError();
-}
 
 // Filter s8 NCHW [oc][ic][fh][fw] -> MFMA-fragment layout over K = (kh, kw, c) with c padded to ICp
 // and K padded to a multiple of 64, N padded to 16. One thread per 8 packed bytes.

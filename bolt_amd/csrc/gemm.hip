@@ -148,104 +148,121 @@ struct GemmTile {
     static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-// Epilogue through LDS. Each wave parks 2 row-blocks (32 rows) of its tile at a time in its own LDS
-// region as a row-major int32 panel, then walks it so that every lane owns 4 consecutive columns
-// and every global access (C_in load, result store) of a wave is a contiguous run of TN*16
-// elements per row. The per-column terms (offsetC - compensation, channel scale, bias) are loaded
-// once per lane; the C_in loads of a panel are all issued before the first store so their latency
-// overlaps. Call after the last K-loop barrier.
+// Epilogue straight from the accumulators. The tiled kernels feed the matrix instruction with the
+// operands swapped (B fragment first), so a tile's accumulator is the TRANSPOSE of the usual layout:
+// lane (i = lane % 16, g = lane / 16) holds C[row i][cols 4g .. 4g+3] of its 16 x 16 tile, four
+// consecutive columns of one row. Every result store and C_in load is then one 16-byte access per
+// lane with no pass through LDS; a wave covers 16 rows x 64 bytes per access for a matrix, and for
+// a convolution (NCHWC16: a pixel's 16 channels are contiguous, consecutive pixels follow each
+// other) one contiguous KiB. The per-column terms (offsetC - compensation, reciprocal channel
+// scale, bias) depend only on the lane and the tile column and are set up once.
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
+    (void)smem;
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
-    constexpr int kCols = TN * 16;
-    constexpr int kPitch = kCols + 4;  // words; +4 keeps the 4 row groups of a tile on different banks
-    constexpr int kXPer = (TM < 2) ? TM : 2;
-    constexpr int kLanesPerRow = kCols / 4;
-    constexpr int kRowsPerIter = 64 / kLanesPerRow;
-    constexpr int kIters = kXPer * 16 / kRowsPerIter;
-    int32_t *panel = (int32_t *)smem + wave * 32 * kPitch;
-    const uint32_t cl = (lane % kLanesPerRow) * 4;
-    const uint32_t r0 = lane / kLanesPerRow;
-    const uint32_t n = n0 + wn * kCols + cl;
-    // convolution output: blocks of out_c channels per pixel, so 4 channels starting at a multiple
-    // of 4 are always contiguous and 16-byte aligned
-    const bool vec = CONV ? (n + 4 <= a.N) : ((n + 4 <= a.N) && ((a.N & 3) == 0));
     const bool use_cin = !CONV && a.add_cin && MODE != EPI_U8;
+    const bool n_vec = CONV || ((a.N & 3) == 0);
     int lane_max = 0;
-    uint32_t cblk_off = 0, cblk_w = 1;
-    if (CONV) {
-        const uint32_t x = a.conv.out_c, blk = n / x;
-        cblk_w = (a.N - blk * x < x) ? a.N - blk * x : x;              // trailing narrower block
-        cblk_off = blk * x * a.conv.OHW + (n % x);
-    }
 
-    uint32_t base[4];
-    float sw[4], bs[4];
     float factor = 0.0f, sI = 0.0f;
-    if (MODE == EPI_F32 || MODE == EPI_U8) {
+    if (CONV && MODE == EPI_U8) {
+        // tensor-wide dynamic requantisation (avx512/quantize.cpp:364-416 after the abs-max of :70-119)
+        const int mx = ws_read_max(a.conv.absmax);
+        factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
+        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+            *a.conv.dscale_out = a.conv.scaleO * factor;
+        }
+    } else if (MODE == EPI_F32 || MODE == EPI_U8) {
         factor = epi_factor(a.epi);
     } else if (MODE == EPI_F32_CH) {
         sI = *a.epi.scaleI;
     }
+
+    uint32_t base[TN][4];
+    float qs[TN][4], bs[TN][4];
+    uint32_t cblk_off[TN], cblk_w[TN];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const bool ok = n + c < a.N;
-        base[c] = ok ? (uint32_t)a.ob[n + c] - (uint32_t)a.comp[n + c] : 0u;
-        sw[c] = (MODE == EPI_F32_CH && ok) ? a.epi.scaleW[n + c] : 1.0f;
-        bs[c] = (MODE == EPI_F32_CH && ok && a.epi.bias) ? a.epi.bias[n + c] : 0.0f;
+    for (int y = 0; y < TN; ++y) {
+        const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const bool ok = n + c < a.N;
+            base[y][c] = ok ? (uint32_t)a.ob[n + c] - (uint32_t)a.comp[n + c] : 0u;
+            qs[y][c] = 1.0f;
+            bs[y][c] = 0.0f;
+            if (MODE == EPI_F32_CH && ok) {
+                const float s = sI * a.epi.scaleW[n + c];
+                qs[y][c] = 1.0f / s;
+                bs[y][c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
+            }
+        }
+        cblk_off[y] = 0;
+        cblk_w[y] = 1;
+        if (CONV) {
+            // output blocks of out_c channels per pixel (a trailing block may be narrower); 4 channels
+            // starting at a multiple of 4 never straddle a block
+            const uint32_t xc = a.conv.out_c, blk = n / xc;
+            cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
+            cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+        }
     }
 
+    v4i cin[2][TN];
+#define BG_LOAD_CIN(xx, buf)                                                              \
+    if (use_cin) {                                                                        \
+        const uint32_t m_ = m0 + (wm * TM + (xx)) * 16 + i;                               \
+        _Pragma("unroll") for (int y = 0; y < TN; ++y)                                    \
+        {                                                                                 \
+            const uint32_t n_ = n0 + (wn * TN + y) * 16 + 4 * g;                          \
+            cin[buf][y] = (v4i){0, 0, 0, 0};                                              \
+            if (m_ < a.M && n_ < a.N) {                                                   \
+                const int32_t *p_ = (const int32_t *)a.C + (size_t)m_ * a.N + n_;         \
+                if (n_vec && n_ + 4 <= a.N) {                                             \
+                    cin[buf][y] = *(const v4i *)p_;                                       \
+                } else {                                                                  \
+                    for (int c = 0; c < 4 && n_ + c < a.N; ++c) {                         \
+                        cin[buf][y][c] = p_[c];                                           \
+                    }                                                                     \
+                }                                                                         \
+            }                                                                             \
+        }                                                                                 \
+    }
+    BG_LOAD_CIN(0, 0);
 #pragma unroll
-    for (int xh = 0; xh < TM; xh += kXPer) {
-#pragma unroll
-        for (int x = 0; x < kXPer; ++x) {
-#pragma unroll
-            for (int y = 0; y < TN; ++y) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    panel[(x * 16 + 4 * g + r) * kPitch + y * 16 + i] = acc[xh + x][y][r];
-                }
-            }
+    for (int x = 0; x < TM; ++x) {
+        if (x + 1 < TM) {
+            BG_LOAD_CIN(x + 1, (x + 1) & 1);  // the next row block's C_in is in flight while this one is stored
         }
-        v4i cin[kIters];
-#pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            const uint32_t m = m0 + (wm * TM + xh) * 16 + r0 + it * kRowsPerIter;
-            cin[it] = (v4i){0, 0, 0, 0};
-            if (use_cin && m < a.M && n < a.N) {
-                const int32_t *p = (const int32_t *)a.C + (size_t)m * a.N + n;
-                if (vec) {
-                    cin[it] = *(const v4i *)p;
-                } else {
-                    for (int c = 0; c < 4 && n + c < a.N; ++c) {
-                        cin[it][c] = p[c];
-                    }
-                }
-            }
+        const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+        if (m >= a.M) {
+            continue;
         }
-        // the same wave wrote the panel and reads it back: LDS operations of one wave complete in order
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        size_t rowbase = (size_t)m * a.N;
+        uint32_t pix = 0;
+        if (CONV) {
+            const uint32_t img = m / a.conv.OHW;
+            pix = m - img * a.conv.OHW;
+            rowbase = (size_t)img * a.N * a.conv.OHW;
+        }
 #pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            const uint32_t rr = r0 + it * kRowsPerIter;
-            const uint32_t m = m0 + (wm * TM + xh) * 16 + rr;
-            if (m >= a.M || n >= a.N) {
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+            if (n >= a.N) {
                 continue;
             }
-            const v4i v = *(const v4i *)(panel + rr * kPitch + cl);
+            const bool vec = n_vec && (n + 4 <= a.N);
             int t[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                t[c] = (int)((uint32_t)v[c] + base[c] + (uint32_t)cin[it][c]);  // int32 wrap
+                t[c] = (int)((uint32_t)acc[x][y][c] + base[y][c] + (use_cin ? (uint32_t)cin[x & 1][y][c] : 0u));  // int32 wrap
             }
-            size_t idx = (size_t)m * a.N + n;
+            size_t idx = rowbase + n;
             if (CONV) {
-                const uint32_t img = m / a.conv.OHW, r = m % a.conv.OHW;
-                idx = (size_t)img * a.N * a.conv.OHW + cblk_off + (size_t)r * cblk_w;
-                if (MODE == EPI_I32 && a.conv.relu) {
+                idx = rowbase + cblk_off[y] + (size_t)pix * cblk_w[y];
+                if ((MODE == EPI_I32 || MODE == EPI_U8) && a.conv.relu) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         t[c] = t[c] < 0 ? 0 : t[c];  // integer ReLU (convolution_direct.cpp:2406)
@@ -262,7 +279,9 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 }
             }
             if (MODE == EPI_I32) {
-                if (vec) {
+                if (CONV && !a.C) {
+                    // abs-max pass only
+                } else if (vec) {
                     *(v4i *)((int32_t *)a.C + idx) = (v4i){t[0], t[1], t[2], t[3]};
                 } else {
                     for (int c = 0; c < 4 && n + c < a.N; ++c) {
@@ -273,7 +292,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 unsigned b[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    b[c] = epi_u8(t[c], factor);
+                    // stand-alone requantisation adds 128.0f before rounding, the GEMM's own u8 mode after
+                    b[c] = CONV ? usat8_u(rne_i32((float)t[c] * factor + 128.0f)) : epi_u8(t[c], factor);
                 }
                 if (vec) {
                     *(uint32_t *)((uint8_t *)a.C + idx) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
@@ -297,11 +317,9 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                             }
                         }
                     } else {
-                        const float s = sI * sw[c];
-                        const float q = 1.0f / s;
-                        f[c] = (float)t[c] * q;
+                        f[c] = (float)t[c] * qs[y][c];
                         if (a.epi.bias) {
-                            f[c] = f[c] + bs[c];
+                            f[c] = f[c] + bs[y][c];
                         }
                     }
                 }
@@ -314,8 +332,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 }
             }
         }
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // panel reads done before the next pair of row-blocks overwrites it
     }
+#undef BG_LOAD_CIN
     if (CONV && MODE == EPI_I32 && a.conv.absmax) {
         // max |acc| of the whole output tensor, for the dynamic requantisation that follows
         lane_max = wave_reduce_max_i(lane_max);
@@ -333,6 +351,8 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
     if (CONV) {
         if (a.epi.mode == EPI_I32) {
             epilogue_rows<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+        } else if (a.epi.mode == EPI_U8) {
+            epilogue_rows<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else {
             epilogue_rows<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         }
@@ -456,7 +476,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_tiled_kernel(GemmArgs a
             for (int x = 0; x < TM; ++x) {
 #pragma unroll
                 for (int y = 0; y < TN; ++y) {
-                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[x], fb[y], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[x], acc[x][y], 0, 0, 0);  // B first: transposed accumulator
                 }
             }
         }
@@ -587,13 +607,44 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         }                                                                                                \
     }
 #define BG_CLAMP(tile) ((tile) < ksteps ? (tile) : ksteps - 1)
-// offset of K tile `tile` inside an A row: 64 bytes per tile for a matrix (scalar); for a convolution
-// the 16-byte chunk this lane's K-group covers belongs to tap / channel block chunk_off[4*tile + g]
-#define BG_AOFF(tile) (CONV ? (size_t)a.conv.chunk_off[(tile)*4 + g] : (size_t)(tile)*64)
+// Offset of K tile `tile` inside an A row: 64 bytes per tile for a matrix (scalar). For a
+// convolution K runs over (kh, kw, c) in 16-channel chunks and this lane's K-group g covers chunk
+// 4 * tile + g; its (kh, kw, c16) is carried in registers and stepped by four chunks per tile --
+// a table in memory would put a vector load, and with it a wait on every tile fetch in flight,
+// into each step. Chunks past the last tap (K padded to 64) read the pixel base; their weights are 0.
+#define BG_AOFF(tile) ((size_t)(tile)*64)
+    static_assert(!CONV || PIPE, "the convolution walk is wired into the fragment-prefetch loop");
+    uint32_t cv_c16 = 0, cv_kw = 0, cv_kh = 0;
+    const uint32_t cv_cpc = CONV ? a.conv.ICp / 16 : 1;
+    if (CONV) {
+        const uint32_t tap = g / cv_cpc;
+        cv_c16 = g % cv_cpc;
+        cv_kh = tap / a.conv.fw;
+        cv_kw = tap % a.conv.fw;
+    }
+#define BG_CV_OFF()                                                                                            \
+    ((cv_kh < a.conv.fh) ? (size_t)((cv_kh * a.conv.dh * a.conv.Wp + cv_kw * a.conv.dw) * a.conv.ICp + cv_c16 * 16) \
+                         : (size_t)0)
+#define BG_CV_ADVANCE()                                      \
+    {                                                        \
+        cv_c16 += 4;                                         \
+        _Pragma("unroll") for (int w_ = 0; w_ < 4; ++w_)     \
+        {                                                    \
+            const bool wr_ = cv_c16 >= cv_cpc;               \
+            cv_c16 -= wr_ ? cv_cpc : 0u;                     \
+            cv_kw += wr_ ? 1u : 0u;                          \
+            const bool w2_ = cv_kw >= a.conv.fw;             \
+            cv_kw = w2_ ? 0u : cv_kw;                        \
+            cv_kh += w2_ ? 1u : 0u;                          \
+        }                                                    \
+    }
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
-        BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s), BG_AOFF(BG_CLAMP((uint32_t)s)));
+        BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s), (CONV ? BG_CV_OFF() : BG_AOFF(BG_CLAMP((uint32_t)s))));
+        if (CONV && (uint32_t)s + 1 < ksteps) {
+            BG_CV_ADVANCE();
+        }
     }
     if constexpr (!PIPE) {
         for (uint32_t t = 0; t < ksteps; ++t) {
@@ -624,7 +675,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
                 }
 #pragma unroll
                 for (int y = 0; y < TN; ++y) {
-                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[y], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa, acc[x][y], 0, 0, 0);  // B first: transposed accumulator
                 }
             }
         }
@@ -656,14 +707,21 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         __builtin_amdgcn_s_barrier();                                                        \
         asm volatile("" ::: "memory");                                                       \
         BG_ISSUE((tt) + (STAGES - 1), BG_CLAMP((tt) + (STAGES - 1)), aoff_next);             \
-        aoff_next = BG_AOFF(BG_CLAMP((tt) + STAGES)); /* convolution: table load, one step ahead */ \
+        if (CONV) {                                                                          \
+            if ((tt) + STAGES < ksteps) {                                                    \
+                BG_CV_ADVANCE();                                                             \
+            }                                                                                \
+            aoff_next = BG_CV_OFF();                                                         \
+        } else {                                                                             \
+            aoff_next = BG_AOFF(BG_CLAMP((tt) + STAGES));                                    \
+        }                                                                                    \
         BG_READ_FRAGS(BG_CLAMP((tt) + 1), NA, NB);                                           \
         _Pragma("unroll") for (int x = 0; x < TM; ++x)                                       \
         {                                                                                    \
             const v4i fx_ = CONV ? FA[x] : (FA[x] ^ flip); /* re-bias at use: the read stays in flight */ \
             _Pragma("unroll") for (int y = 0; y < TN; ++y)                                   \
             {                                                                                \
-                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx_, FB[y], acc[x][y], 0, 0, 0); \
+                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(FB[y], fx_, acc[x][y], 0, 0, 0); \
             }                                                                                \
         }                                                                                    \
         /* issue order for the scheduler: the tile fetches first, then one LDS fragment read */ \
@@ -682,7 +740,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         BG_READ_FRAGS(0u, fa0, fb0);
-        size_t aoff_next = BG_AOFF(BG_CLAMP((uint32_t)(STAGES - 1)));
+        size_t aoff_next = CONV ? BG_CV_OFF() : BG_AOFF(BG_CLAMP((uint32_t)(STAGES - 1)));
         uint32_t t = 0;
         for (; t + 1 < ksteps; t += 2) {
             BG_STEP(t, fa0, fb0, fa1, fb1);
@@ -698,6 +756,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 #undef BG_ISSUE
 #undef BG_CLAMP
 #undef BG_AOFF
+#undef BG_CV_OFF
+#undef BG_CV_ADVANCE
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();  // every wave is done with the K-loop buffers before they become the panel
     asm volatile("" ::: "memory");

@@ -40,11 +40,14 @@ struct ConvGeom {
     uint32_t OHW, OW;          // output pixels per image, output width
     uint32_t sh, sw;           // strides
     uint32_t Hp, Wp, ICp;      // padded image height / width, channels rounded up to 16
-    const uint32_t *chunk_off; // [K / 16] byte offset of 16-channel chunk q = tap * ICp/16 + c16 from the pixel base
+    uint32_t fh, fw, dh, dw;   // filter taps and dilation: K runs over (kh, kw, c) in 16-channel chunks
     uint32_t out_c;            // channel block of the output layout: 16 (NCHWC16) or 8 (NCHWC8)
     int relu;
     const float *eltwise;      // optional fp32 tensor added before the ReLU (fp32 output only)
-    uint32_t *absmax;          // optional: max |acc| over the whole output (int32 output only)
+    uint32_t *absmax;          // scratch slots: int32 mode folds max |acc| into them (C may then be null:
+                               // nothing is stored); u8 mode reads them for the tensor-wide dynamic scale
+    float scaleO;              // u8 mode: scale of the accumulators (input scale * filter scale)
+    float *dscale_out;         // u8 mode: device word that receives the resulting output scale
 };
 
 struct GemmArgs {
@@ -70,8 +73,6 @@ void gemm_force_tile(int tile);
 // u8 NCHWC8 (cx = 8) / NCHWC16 (cx = 16) -> s8 (x - 128), zero padded, [n][H+pt+pb][W+pl+pr][ALIGN(C,16)]
 hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
     uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st);
-hipError_t launch_conv_chunk_table(uint32_t *tab, uint32_t fh, uint32_t fw, uint32_t dh, uint32_t dw, uint32_t Wp,
-    uint32_t ICp, uint32_t pad_to, hipStream_t st);
 // s8 NCHW filter -> offsetC[OC] and the fragment-layout matrix over K = (kh, kw, c)
 hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, uint32_t fh, uint32_t fw, int32_t *offsetC,
     int8_t *dst, hipStream_t st);
