@@ -129,12 +129,14 @@ __global__ __launch_bounds__(256) void bnn_conv_kernel(BnnArgs a)
 {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t ob = blockIdx.y * 4 + wave;  // block of 32 output channels
-    if (ob * 32 >= a.OC) {
+    // the four waves of a workgroup share one block of 32 output channels (the same weight stream in
+    // the scalar cache) and take 64 pixels each
+    const uint32_t ob = blockIdx.y;
+    const uint32_t cw = a.IC / 32;
+    uint32_t pix = (blockIdx.x * 4 + wave) * 64 + lane;
+    if ((blockIdx.x * 4 + wave) * 64 >= a.M) {
         return;
     }
-    const uint32_t cw = a.IC / 32;
-    uint32_t pix = blockIdx.x * 64 + lane;
     const bool live = pix < a.M;
     pix = live ? pix : a.M - 1;
     const uint32_t img = pix / a.OHW, r = pix % a.OHW;
@@ -147,17 +149,65 @@ __global__ __launch_bounds__(256) void bnn_conv_kernel(BnnArgs a)
     for (int o = 0; o < 32; ++o) {
         acc[o] = 0;
     }
-    for (uint32_t kh = 0; kh < a.fh; ++kh) {
-        for (uint32_t kw = 0; kw < a.fw; ++kw) {
-            const uint32_t *xt = xp + (size_t)(kh * a.Wp + kw) * cw;
-            for (uint32_t j = 0; j < cw; ++j) {
-                const uint32_t xv = xt[j];
+    if ((cw & 3) == 0) {
+        // 128 channels (one 16-byte load) per step; the load of the next step is issued before the
+        // 4 x 64 VALU instructions of this one, so its latency never stalls the wave. The step
+        // counters are wave-uniform (scalar ALU).
+        const uint32_t cw4 = cw >> 2, steps = a.fh * a.fw * cw4;
+        uint32_t j4 = 0, kw = 0, kh = 0;
+        v4i nxt = *(const v4i *)xp;
+        // the 32 weights of the next 32-channel group are fetched (scalar loads) while the VALU works
+        // through the current group: two SGPR sets in flight
+        uint32_t wc[32], wn[32];
+#pragma unroll
+        for (int o = 0; o < 32; ++o) {
+            wc[o] = wp[o];
+        }
+        for (uint32_t it = 0; it < steps; ++it) {
+            const v4i cur = nxt;
+            if (++j4 == cw4) {
+                j4 = 0;
+                if (++kw == a.fw) {
+                    kw = 0;
+                    ++kh;
+                }
+            }
+            const bool more = it + 1 < steps;
+            if (more) {
+                nxt = *(const v4i *)(xp + (size_t)(kh * a.Wp + kw) * cw + j4 * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t xv = (uint32_t)cur[u];
+                const uint32_t *wq = (u < 3 || more) ? wp + (u + 1) * 32 : wp;  // past the end: any valid address
 #pragma unroll
                 for (int o = 0; o < 32; ++o) {
-                    const uint32_t wv = wp[o];  // wave-uniform address: scalar load
-                    acc[o] += __builtin_popcount(XNOR ? (xv ^ wv) : (xv & wv));
+                    wn[o] = wq[o];
                 }
-                wp += 32;
+#pragma unroll
+                for (int o = 0; o < 32; ++o) {
+                    acc[o] += __builtin_popcount(XNOR ? (xv ^ wc[o]) : (xv & wc[o]));
+                }
+#pragma unroll
+                for (int o = 0; o < 32; ++o) {
+                    wc[o] = wn[o];
+                }
+            }
+            wp += 128;
+        }
+    } else {
+        for (uint32_t kh = 0; kh < a.fh; ++kh) {
+            for (uint32_t kw = 0; kw < a.fw; ++kw) {
+                const uint32_t *xt = xp + (size_t)(kh * a.Wp + kw) * cw;
+                for (uint32_t j = 0; j < cw; ++j) {
+                    const uint32_t xv = xt[j];
+#pragma unroll
+                    for (int o = 0; o < 32; ++o) {
+                        const uint32_t wv = wp[o];  // wave-uniform address: scalar load
+                        acc[o] += __builtin_popcount(XNOR ? (xv ^ wv) : (xv & wv));
+                    }
+                    wp += 32;
+                }
             }
         }
     }
@@ -195,7 +245,7 @@ hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st)
     if (a.M == 0 || a.OC == 0) {
         return hipSuccess;
     }
-    const dim3 grid((a.M + 63) / 64, (a.OC / 32 + 3) / 4);
+    const dim3 grid((a.M + 255) / 256, a.OC / 32);
     if (xnor) {
         hipLaunchKernelGGL((bnn_conv_kernel<1>), grid, dim3(256), 0, st, a);
     } else {
