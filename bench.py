@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--only", choices=["gemm", "fc", "conv", "bnn", "encoder", "quantize"],
+                    help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
     return ap.parse_args()
@@ -94,7 +96,7 @@ def cpu_baseline(W, xq, sI, sW0, seconds):
 MFMA_PEAK_TOPS = 5000.0
 
 
-def other_kernels(L, capi, host, torch, dev):
+def other_kernels(L, capi, host, torch, dev, only=None):
     """Secondary measurements of the same hot path, each timed with HIP events on the library stream
     over `reps` back-to-back calls with operands resident in HBM. Python issues every call, so shapes
     whose kernel runs under ~15 us (C1) are bound by call overhead, which is what a caller sees."""
@@ -105,6 +107,9 @@ def other_kernels(L, capi, host, torch, dev):
                                DT_I32, DT_U8_Q, tensor2df)
     g = torch.Generator(device=dev).manual_seed(20240601)
     res = {}
+
+    def want(name):
+        return only is None or only == name
 
     def timed(fn, reps, warm=3):
         for _ in range(warm):
@@ -118,98 +123,104 @@ def other_kernels(L, capi, host, torch, dev):
         return ms.value / reps
 
     # -- int8 GEMM: square sweep + the BERT-base layer shapes (fp32 out = FullyConnected epilogue; int32 out = C += A.B)
-    gemm = []
-    for (M, K, N, reps) in ((2048, 2048, 2048, 50), (4096, 4096, 4096, 30), (8192, 8192, 8192, 10), (4096, 768, 768, 50),
-                            (4096, 768, 3072, 50), (4096, 3072, 768, 50)):
-        A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
-        W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
-        blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
-        off = blob[rhs:rhs + 4 * N].clone()
-        ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
-        for cdt, tdt, sc, nm in ((DT_F32, torch.float32, [37.25], "f32"), (DT_I32, torch.int32, None, "i32_accumulate")):
-            Cb = torch.zeros((M, N), dtype=tdt, device=dev)
-            cd = tensor2df(cdt, DF_NORMAL, M, N)
-            t = timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps)
-            tops = 2.0 * M * N * K / t / 1e9
-            gemm.append({"M": M, "K": K, "N": N, "out": nm, "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
-        del A, W, blob, Cb
-    res["gemm_int8"] = gemm
-
+    if want("gemm"):
+        gemm = []
+        for (M, K, N, reps) in ((2048, 2048, 2048, 50), (4096, 4096, 4096, 30), (8192, 8192, 8192, 10), (4096, 768, 768, 50),
+                                (4096, 768, 3072, 50), (4096, 3072, 768, 50)):
+            A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
+            W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
+            blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            off = blob[rhs:rhs + 4 * N].clone()
+            ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+            for cdt, tdt, sc, nm in ((DT_F32, torch.float32, [37.25], "f32"), (DT_I32, torch.int32, None, "i32_accumulate")):
+                Cb = torch.zeros((M, N), dtype=tdt, device=dev)
+                cd = tensor2df(cdt, DF_NORMAL, M, N)
+                t = timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps)
+                tops = 2.0 * M * N * K / t / 1e9
+                gemm.append({"M": M, "K": K, "N": N, "out": nm, "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
+            del A, W, blob, Cb
+        res["gemm_int8"] = gemm
     # -- C1: FullyConnected M=64 K=1024 N=1024, fp32 out
-    M, K, N = 64, 1024, 1024
-    x = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
-    W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
-    blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
-    bias = torch.randn(N, device=dev, generator=g) * 0.1
-    t = timed(lambda: host.fully_connected(x, 30.0, blob, DF_NKNxKx, 100.0, bias, M, K, N, DT_F32), 200)
-    res["fc_c1"] = {"ms": t, "tops": 2.0 * M * N * K / t / 1e9, "algorithmic_bytes": 1380352,
-                    "gbps": 1380352 / t / 1e6, "note": "call-overhead bound: includes tmp/out allocation by the Python wrapper"}
-
+    if want("fc"):
+        M, K, N = 64, 1024, 1024
+        x = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
+        W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
+        blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+        bias = torch.randn(N, device=dev, generator=g) * 0.1
+        t = timed(lambda: host.fully_connected(x, 30.0, blob, DF_NKNxKx, 100.0, bias, M, K, N, DT_F32), 200)
+        res["fc_c1"] = {"ms": t, "tops": 2.0 * M * N * K / t / 1e9, "algorithmic_bytes": 1380352,
+                        "gbps": 1380352 / t / 1e6, "note": "call-overhead bound: includes tmp/out allocation by the Python wrapper"}
     # -- C3: int8 3x3 convolution 32x64x56x56 -> 64, ReLU, u8 out with dynamic output scale
-    n, ic, ih, iw, oc = 32, 64, 56, 56, 64
-    xq = torch.randint(128, 256, (n * ic * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
-    Wc = torch.randint(-127, 128, (oc, ic, 3, 3), dtype=torch.int8, device=dev, generator=g)
-    p = capi.conv_param_spec(oc, 3, 3, 1, 1)
-    cblob, ftm = host_conv.transform_filter(Wc, oc, ic, 3, 3, p)
-    cb = torch.randn(oc, device=dev, generator=g) * 0.1
-    ops = 2.0 * n * ih * iw * oc * ic * 9
-    for odt, nm in ((DT_U8_Q, "u8_dynamic_scale"), (DT_I32, "i32")):
-        t = timed(lambda: host_conv.convolution(xq, DF_NCHWC8, n, ic, ih, iw, cblob, ftm, oc, 3, 3, 1, 1, cb,
-                                                [40.0, -1.0, 80.0], True, odt, DF_NCHWC16), 20)
-        res["conv_c3_" + nm] = {"ms": t, "tops": ops / t / 1e9, "frac_mfma_peak": ops / t / 1e9 / MFMA_PEAK_TOPS,
-                                "algorithmic_bytes": 12882432 if odt == DT_U8_Q else 6422528 * 5 + 36864 + 512}
-
+    if want("conv"):
+        n, ic, ih, iw, oc = 32, 64, 56, 56, 64
+        xq = torch.randint(128, 256, (n * ic * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
+        Wc = torch.randint(-127, 128, (oc, ic, 3, 3), dtype=torch.int8, device=dev, generator=g)
+        p = capi.conv_param_spec(oc, 3, 3, 1, 1)
+        cblob, ftm = host_conv.transform_filter(Wc, oc, ic, 3, 3, p)
+        cb = torch.randn(oc, device=dev, generator=g) * 0.1
+        ops = 2.0 * n * ih * iw * oc * ic * 9
+        ctmp = torch.empty(64 << 20, dtype=torch.uint8, device=dev)      # reused across calls, as an engine's shared tmp is
+        for odt, nm, tdt in ((DT_U8_Q, "u8_dynamic_scale", torch.uint8), (DT_I32, "i32", torch.int32)):
+            cout = torch.empty(n * oc * ih * iw, dtype=tdt, device=dev)
+            t = timed(lambda: host_conv.convolution(xq, DF_NCHWC8, n, ic, ih, iw, cblob, ftm, oc, 3, 3, 1, 1, cb,
+                                                    [40.0, -1.0, 80.0], True, odt, DF_NCHWC16, tmp=ctmp, out=cout), 20)
+            res["conv_c3_" + nm] = {"ms": t, "tops": ops / t / 1e9, "frac_mfma_peak": ops / t / 1e9 / MFMA_PEAK_TOPS,
+                                    "algorithmic_bytes": 12882432 if odt == DT_U8_Q else 6422528 * 5 + 36864 + 512}
     # -- C5: XNOR convolution 64x256x28x28 -> 256, fp32 out
-    n, ic, ih, iw, oc = 64, 256, 28, 28, 256
-    xb = torch.randint(0, 256, (n * ic // 8 * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
-    wb = torch.randint(0, 256, (oc * ic * 9 // 8,), dtype=torch.uint8, device=dev, generator=g)
-    bblob, bftm = host_conv.bnn_transform_filter(wb, DT_BIN11, DF_NCHWN16C8, oc, ic, 3, 3)
-    bs, bb = torch.rand(oc, device=dev, generator=g) + 0.5, torch.randn(oc, device=dev, generator=g) * 0.1
-    t = timed(lambda: host_conv.convolution_bnn(xb, DT_BIN11, n, ic, ih, iw, bblob, bftm, oc, 3, 3, 1, 1, bs, bb, DT_F32), 20)
-    macs = float(n) * ih * iw * oc * ic * 9
-    res["bnn_c5_xnor"] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
-                          "gbps": 53061632 / t / 1e6}
-
+    if want("bnn"):
+        n, ic, ih, iw, oc = 64, 256, 28, 28, 256
+        xb = torch.randint(0, 256, (n * ic // 8 * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
+        wb = torch.randint(0, 256, (oc * ic * 9 // 8,), dtype=torch.uint8, device=dev, generator=g)
+        bblob, bftm = host_conv.bnn_transform_filter(wb, DT_BIN11, DF_NCHWN16C8, oc, ic, 3, 3)
+        bs, bb = torch.rand(oc, device=dev, generator=g) + 0.5, torch.randn(oc, device=dev, generator=g) * 0.1
+        btmp = torch.empty(8 << 20, dtype=torch.uint8, device=dev)
+        bout = torch.empty(n * oc * ih * iw, dtype=torch.float32, device=dev)
+        t = timed(lambda: host_conv.convolution_bnn(xb, DT_BIN11, n, ic, ih, iw, bblob, bftm, oc, 3, 3, 1, 1, bs, bb, DT_F32,
+                                                    tmp=btmp, out=bout), 20)
+        macs = float(n) * ih * iw * oc * ic * 9
+        res["bnn_c5_xnor"] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
+                              "gbps": 53061632 / t / 1e6}
     # -- C4: BERT-base int8 encoder layer, batch 32 x seq 128 (4096 tokens), one C call per layer
-    sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    import encoder_layer as ref_layer
-    from bolt_amd.host_encoder import EncoderLayer
-    rs = np.random.default_rng(20240604)
-    batch, seq, hidden, heads, ffn = 32, 128, 768, 12, 3072
-    P = {}
-    for name, Nn, Kk in (("qkv", 3 * hidden, hidden), ("o", hidden, hidden), ("1", ffn, hidden), ("2", hidden, ffn)):
-        P["w" + name], P["s" + name] = ref_layer.quantize_weight_per_channel(   # load-time weight quantisation
-            (rs.standard_normal((Nn, Kk)) * 0.02).astype(np.float32))
-        P["b" + name] = np.zeros(Nn, np.float32)
-    for k in ("ln1", "ln2"):
-        P[k + "_g"], P[k + "_b"] = np.ones(hidden, np.float32), np.zeros(hidden, np.float32)
-    layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
-    hx = torch.randn((batch * seq, hidden), device=dev, generator=g)
-    hy = torch.empty_like(hx)
-    t = timed(lambda: layer(hx, hy), 50)
-    gemm_ops = 2.0 * batch * seq * hidden * (3 * hidden + hidden + 2 * ffn)
-    res["bert_base_layer_c4"] = {"ms": t, "tokens_per_s": batch * seq / (t * 1e-3), "int8_gemm_tops": gemm_ops / t / 1e9,
-                                 "config": "hidden 768, 12 heads, FFN 3072, seq 128, batch 32; int8 GEMMs with per-channel "
-                                           "weight scales, dynamic per-tensor activation quantisation, fp32 attention / "
-                                           "LayerNorm / GELU"}
-
+    if want("encoder"):
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import encoder_layer as ref_layer
+        from bolt_amd.host_encoder import EncoderLayer
+        rs = np.random.default_rng(20240604)
+        batch, seq, hidden, heads, ffn = 32, 128, 768, 12, 3072
+        P = {}
+        for name, Nn, Kk in (("qkv", 3 * hidden, hidden), ("o", hidden, hidden), ("1", ffn, hidden), ("2", hidden, ffn)):
+            P["w" + name], P["s" + name] = ref_layer.quantize_weight_per_channel(   # load-time weight quantisation
+                (rs.standard_normal((Nn, Kk)) * 0.02).astype(np.float32))
+            P["b" + name] = np.zeros(Nn, np.float32)
+        for k in ("ln1", "ln2"):
+            P[k + "_g"], P[k + "_b"] = np.ones(hidden, np.float32), np.zeros(hidden, np.float32)
+        layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
+        hx = torch.randn((batch * seq, hidden), device=dev, generator=g)
+        hy = torch.empty_like(hx)
+        t = timed(lambda: layer(hx, hy), 50)
+        gemm_ops = 2.0 * batch * seq * hidden * (3 * hidden + hidden + 2 * ffn)
+        res["bert_base_layer_c4"] = {"ms": t, "tokens_per_s": batch * seq / (t * 1e-3), "int8_gemm_tops": gemm_ops / t / 1e9,
+                                     "config": "hidden 768, 12 heads, FFN 3072, seq 128, batch 32; int8 GEMMs with per-channel "
+                                               "weight scales, dynamic per-tensor activation quantisation, fp32 attention / "
+                                               "LayerNorm / GELU"}
     # -- quantize family at the BERT FFN size (4096 x 3072)
-    cnt = 4096 * 3072
-    xf = torch.randn(cnt, device=dev, generator=g)
-    q8 = torch.empty(cnt, dtype=torch.uint8, device=dev)
-    dsc = torch.full((1,), -1.0, device=dev)
-    t = timed(lambda: capi.check(L.bolt_gfx950_quantize_f32_async(xf.data_ptr(), cnt, DT_U8_Q, q8.data_ptr(),
-                                                                  dsc.data_ptr(), 0), "q"), 50)
-    res["quantize_f32_u8_dynamic"] = {"n": cnt, "ms": t, "algorithmic_bytes": 9 * cnt, "gbps": 9 * cnt / t / 1e6,
-                                      "frac_hbm_peak": 9 * cnt / t / 1e6 / HBM_PEAK_GBS}
-    acc = torch.randint(-200000, 200000, (cnt,), dtype=torch.int32, device=dev, generator=g)
-    fo = torch.empty(cnt, dtype=torch.float32, device=dev)
-    t = timed(lambda: host.dequantize(acc, DT_I32, 37.5, out=fo), 50)
-    res["dequantize_i32_f32"] = {"n": cnt, "ms": t, "algorithmic_bytes": 8 * cnt, "gbps": 8 * cnt / t / 1e6,
-                                 "frac_hbm_peak": 8 * cnt / t / 1e6 / HBM_PEAK_GBS}
-    t = timed(lambda: host.quantize(acc, DT_I32, DT_U8_Q, [0.02, 37.5], out=q8), 50)
-    res["requantize_i32_u8_static"] = {"n": cnt, "ms": t, "algorithmic_bytes": 5 * cnt, "gbps": 5 * cnt / t / 1e6,
-                                       "frac_hbm_peak": 5 * cnt / t / 1e6 / HBM_PEAK_GBS}
+    if want("quantize"):
+        cnt = 4096 * 3072
+        xf = torch.randn(cnt, device=dev, generator=g)
+        q8 = torch.empty(cnt, dtype=torch.uint8, device=dev)
+        dsc = torch.full((1,), -1.0, device=dev)
+        t = timed(lambda: capi.check(L.bolt_gfx950_quantize_f32_async(xf.data_ptr(), cnt, DT_U8_Q, q8.data_ptr(),
+                                                                      dsc.data_ptr(), 0), "q"), 50)
+        res["quantize_f32_u8_dynamic"] = {"n": cnt, "ms": t, "algorithmic_bytes": 9 * cnt, "gbps": 9 * cnt / t / 1e6,
+                                          "frac_hbm_peak": 9 * cnt / t / 1e6 / HBM_PEAK_GBS}
+        acc = torch.randint(-200000, 200000, (cnt,), dtype=torch.int32, device=dev, generator=g)
+        fo = torch.empty(cnt, dtype=torch.float32, device=dev)
+        t = timed(lambda: host.dequantize(acc, DT_I32, 37.5, out=fo), 50)
+        res["dequantize_i32_f32"] = {"n": cnt, "ms": t, "algorithmic_bytes": 8 * cnt, "gbps": 8 * cnt / t / 1e6,
+                                     "frac_hbm_peak": 8 * cnt / t / 1e6 / HBM_PEAK_GBS}
+        t = timed(lambda: host.quantize(acc, DT_I32, DT_U8_Q, [0.02, 37.5], out=q8), 50)
+        res["requantize_i32_u8_static"] = {"n": cnt, "ms": t, "algorithmic_bytes": 5 * cnt, "gbps": 5 * cnt / t / 1e6,
+                                           "frac_hbm_peak": 5 * cnt / t / 1e6 / HBM_PEAK_GBS}
     return res
 
 
@@ -229,6 +240,9 @@ def main():
     L = capi.lib()
     capi.check(L.bolt_gfx950_init(), "init")
     dev = torch.device("cuda:0")
+    if a.only:
+        print(json.dumps({"only": a.only, "other_kernels": other_kernels(L, capi, host, torch, dev, a.only)}), flush=True)
+        return
     rng = np.random.default_rng(20240601)
     W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
     sW = (1.0 / rng.uniform(0.005, 0.02, size=N)).astype(np.float32)      # Bolt scale = 1 / step

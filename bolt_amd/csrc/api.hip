@@ -1275,18 +1275,12 @@ size_t conv_padded_bytes(const ConvShape &s)
     return ((size_t)s.n * s.Hp * s.Wp * s.ICp + 255) / 256 * 256;
 }
 
-size_t conv_tmp_layout(const ConvShape &s, DataType odt, size_t *tab, size_t *off, size_t *acc)
+// tmp = [padded s8 image][offsetC + folded bias, oc int32]
+size_t conv_tmp_layout(const ConvShape &s, size_t *off)
 {
-    size_t b = conv_padded_bytes(s);
-    *tab = b;
-    b += (size_t)(s.Kp / 16) * 4;
+    size_t b = (conv_padded_bytes(s) + 255) / 256 * 256;
     *off = b;
     b += (size_t)s.oc * 4;
-    b = (b + 255) / 256 * 256;
-    *acc = b;
-    if (odt == DT_U8_Q) {
-        b += (size_t)s.n * s.oc * s.oh * s.ow * 4;
-    }
     return b + 32;
 }
 
@@ -1312,8 +1306,8 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     const void *bias, void *tmp, DataType odt, DataFormat odf, void *output, F32 *scale, int relu)
 {
     Ctx &c = ctx();
-    size_t tabOff, offOff, accOff;
-    conv_tmp_layout(s, odt, &tabOff, &offOff, &accOff);
+    size_t offOff;
+    conv_tmp_layout(s, &offOff);
     U8 *t = (U8 *)tmp;
     const F32 scaleO = scale[0] * scale[2];  // convolution_direct.cpp:2687
     HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
@@ -1454,8 +1448,8 @@ EE convolution_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc f
     if (e != SUCCESS) {
         return e;
     }
-    size_t a, b, c;
-    const size_t total = conv_tmp_layout(s, outputDesc.dt, &a, &b, &c);
+    size_t off;
+    const size_t total = conv_tmp_layout(s, &off);
     if (total > 0xffffffffull) {
         return NOT_SUPPORTED;
     }
@@ -1500,8 +1494,8 @@ EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwi
     if (e != SUCCESS) {
         return e;
     }
-    size_t a, b, c3;
-    const size_t need = conv_tmp_layout(s, odt, &a, &b, &c3);
+    size_t off;
+    const size_t need = conv_tmp_layout(s, &off);
     if (tmpBytes < need) {
         return NOT_MATCH;
     }

@@ -553,6 +553,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     const uint32_t K = a.K;
     const uint32_t nblocks = align_up(a.N, 16) >> 4;
     const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+    // Touch the per-column vectors the epilogue will want (offsetC, compensation) now, so that they sit
+    // in this XCD's L2 by then instead of costing an HBM round trip at the end of every block.
+    int warm = 0;
+    {
+        const uint32_t n = n0 + wn * TN * 16 + lane;
+        if (lane < TN * 16 && n < a.N) {
+            warm = a.ob[n] ^ a.comp[n];
+        }
+    }
 
     v4i acc[TM][TN];
 #pragma unroll
@@ -732,7 +741,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                               \
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                               \
         }                                                                                    \
-        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 2 * (TM + TN), 0);             \
+        __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN > 2 * (TM + TN)) ? TM * TN - 2 * (TM + TN) : 0, 0); \
     }
         // tile 0 landed everywhere
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
@@ -758,9 +767,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 #undef BG_AOFF
 #undef BG_CV_OFF
 #undef BG_CV_ADVANCE
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();  // every wave is done with the K-loop buffers before they become the panel
-    asm volatile("" ::: "memory");
+    asm volatile("" ::"v"(warm));  // keeps the warming loads alive; the value itself is not used
     epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
@@ -768,7 +775,6 @@ template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE = false, bool CO
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
-    static_assert(WM * WN * 32 * (TN * 16 + 4) * 4 <= T::kLdsBytes, "epilogue panel must fit the K-loop LDS");
     static bool attr_set = false;
     auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV>;
     if (!attr_set) {
@@ -808,7 +814,15 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
         return hipSuccess;
     }
     if (a.N <= 64) {
-        return launch_dma<2, 1, 8, 4, 4, true, true>(a, st);  // 256 pixels x 64 channels, 2 waves
+        // Few output channels: nowhere near MFMA-bound, the time is load latency, so what matters is
+        // waves per CU and that the grid fits the chip in ONE round (every block lives about as long as
+        // the whole kernel). 128-pixel blocks of 4 waves sit three to a CU (768 at once), 256-pixel
+        // blocks two to a CU (512 at once).
+        const uint32_t b128 = (a.M + 127) / 128, b256 = (a.M + 255) / 256;
+        if (b128 <= 768 || b256 > 512) {
+            return launch_dma<4, 1, 2, 4, 4, true, true>(a, st);
+        }
+        return launch_dma<4, 1, 4, 4, 4, true, true>(a, st);
     }
     return launch_dma<2, 2, 8, 4, 4, true, true>(a, st);      // 256 pixels x 128 channels
 }

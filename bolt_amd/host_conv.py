@@ -34,9 +34,9 @@ def transform_filter(filt_nchw, oc, ic, fh, fw, p):
 
 
 def convolution(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias, scale, relu, odt, odf=DF_NCHWC16,
-                eltwise=None, dilation=1):
+                eltwise=None, dilation=1, tmp=None, out=None):
     """x: u8 activations in `idf`; blob / ftm from transform_filter; scale = [sI, sO, sF] (list, sO updated).
-    Returns the output buffer in `odf` order."""
+    Returns the output buffer in `odf` order. `tmp` / `out` may be handed in to reuse buffers across calls."""
     arch = arch_of(x)
     p = conv_param_spec(oc, fh, fw, stride, pad, dilation)
     oh, ow = conv_out_hw(ih, iw, fh, fw, stride, pad, dilation)
@@ -45,9 +45,12 @@ def convolution(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias,
     b = C.c_uint32(0)
     check(lib().convolution_infer_forward_tmp_bytes_gfx950(idesc, ftm, odesc, p, CONVOLUTION_ALGORITHM_DIRECT, C.byref(b),
                                                            arch), "conv_tmp_bytes")
-    tmp = _empty_like_mode(x, b.value)
+    if tmp is None:
+        tmp = _empty_like_mode(x, b.value)
     count = n * oc * oh * ow
-    if _is_torch(x):
+    if out is not None:
+        pass
+    elif _is_torch(x):
         import torch
         tdt = {DT_F32: torch.float32, DT_I32: torch.int32, DT_U8_Q: torch.uint8}[odt]
         out = torch.zeros(count, dtype=tdt, device=x.device)
@@ -78,7 +81,8 @@ def bnn_transform_filter(filt_bits, fdt, fdf, oc, ic, fh, fw):
     return blob, ftm
 
 
-def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, scale, bias, odt=DT_F32):
+def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, scale, bias, odt=DT_F32, tmp=None,
+                    out=None):
     """x: fp32 NCHWC8 activations (idt = DT_F32) or packed bits (idt = the filter's type); scale / bias fp32 [oc].
     Mirrors convolution_bnn (compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72). Output NCHWC8."""
     arch = arch_of(x)
@@ -88,9 +92,12 @@ def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, s
     odesc = tensor4df(odt, DF_NCHWC8, n, oc, oh, ow)
     b = C.c_uint32(0)
     check(lib().convolution_infer_forward_tmp_bytes_bnn_gfx950(idesc, p, C.byref(b), arch), "bnn_tmp_bytes")
-    tmp = _empty_like_mode(x, b.value)
+    if tmp is None:
+        tmp = _empty_like_mode(x, b.value)
     count = n * oc * oh * ow
-    if _is_torch(x):
+    if out is not None:
+        pass
+    elif _is_torch(x):
         import torch
         out = torch.zeros(count, dtype={DT_F32: torch.float32, DT_I32: torch.int32}[odt], device=x.device)
     else:
