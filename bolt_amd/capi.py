@@ -129,6 +129,10 @@ SIGNATURES = {
     "fully_connected_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, _u32p, C.c_int]),
     "fully_connected_gfx950": (C.c_int, [TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_float, TensorDesc, _vp, _u32,
                                          _vp, TensorDesc, _vp, _f32p, C.c_int]),
+    "matmul_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, C.c_bool, TensorDesc, C.c_bool, TensorDesc, _u32p,
+                                                        C.c_int]),
+    "matmul_gfx950": (C.c_int, [TensorDesc, C.c_bool, _vp, C.c_float, TensorDesc, C.c_bool, _vp, C.c_float, _u32, _vp,
+                                TensorDesc, _vp, C.c_int]),
     "convolution_transform_filter_bytes_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, C.c_int, _u32p, C.c_int]),
     "convolution_transform_filter_gfx950": (C.c_int, [TensorDesc, _vp, ConvolutionParamSpec, C.c_int, _TDp, _vp,
                                                       C.c_int]),

@@ -132,6 +132,13 @@ EE get1d(TensorDesc d, DataType *dt, U32 *len)
     return SUCCESS;
 }
 
+uint32_t f32_bits(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
 bool aligned4(const void *p)
 {
     return ((uintptr_t)p & 3) == 0;
@@ -1732,6 +1739,195 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     HIP_TRY(launch_bnn_conv(a, xnor, c.stream));
     if (arch == AMD_GFX950) {
         HIP_TRY(hipMemcpyAsync(output, dO, outN * 4, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
+// ---- tensor_computing: int8 matmul (compute/tensor/src/matmul.cpp:203-300, 302-576, x86 branch) --------
+namespace {
+struct MatmulShape {
+    U32 M, K, N, batch, batchA, batchB;
+    size_t elemsA, elemsB;
+    size_t offQA, offQB, offBlob, offScale, total;  // tmp layout
+};
+
+EE matmul_shape(TensorDesc a, bool tA, TensorDesc b, bool tB, TensorDesc c, MatmulShape *s)
+{
+    if (a.nDims < 2 || b.nDims < 2 || c.nDims < 2) {
+        return NOT_SUPPORTED;
+    }
+    s->M = tA ? a.dims[0] : a.dims[1];
+    s->K = tA ? a.dims[1] : a.dims[0];
+    const U32 kb = tB ? b.dims[0] : b.dims[1];
+    s->N = tB ? b.dims[1] : b.dims[0];
+    if (kb != s->K || c.dims[0] != s->N || c.dims[1] != s->M) {
+        return NOT_MATCH;
+    }
+    auto lead = [](const TensorDesc &d) {
+        U32 n = 1;
+        for (U32 i = 2; i < d.nDims; ++i) {
+            n *= d.dims[i];
+        }
+        return n;
+    };
+    s->batchA = lead(a);
+    s->batchB = lead(b);
+    s->batch = lead(c);
+    // a 2-D operand is shared by every slice (matmul.cpp:505-528 with all leading dims 1)
+    if ((s->batchA != s->batch && s->batchA != 1) || (s->batchB != s->batch && s->batchB != 1)) {
+        return NOT_SUPPORTED;
+    }
+    s->elemsA = (size_t)s->batchA * s->M * s->K;
+    s->elemsB = (size_t)s->batchB * s->K * s->N;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t at = off;
+        off += (bytes + 255) / 256 * 256;
+        return at;
+    };
+    s->offQA = take(s->elemsA);
+    s->offQB = take(s->elemsB);
+    s->offBlob = take((size_t)s->N * 4 + packed_matrix_bytes(s->N, s->K) + 64);
+    s->offScale = take(64);
+    s->total = off;
+    return SUCCESS;
+}
+}  // namespace
+
+EE matmul_infer_forward_tmp_bytes_gfx950(TensorDesc matrixADesc, bool transposeA, TensorDesc matrixBDesc, bool transposeB,
+    TensorDesc matrixCDesc, U32 *bytes, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    MatmulShape s;
+    EE e = matmul_shape(matrixADesc, transposeA, matrixBDesc, transposeB, matrixCDesc, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (s.total > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)s.total;
+    return SUCCESS;
+}
+
+EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F32 scaleA, TensorDesc matrixBDesc,
+    bool transposeB, const void *matrixB, F32 scaleB, U32 tmpBytes, void *tmp, TensorDesc matrixCDesc, void *matrixC,
+    Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!matrixA || !matrixB || !matrixC) {
+        return NULL_POINTER;  // matmul.cpp:322-324
+    }
+    MatmulShape s;
+    EE e = matmul_shape(matrixADesc, transposeA, matrixBDesc, transposeB, matrixCDesc, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    const DataType adt = matrixADesc.dt, bdt = matrixBDesc.dt, cdt = matrixCDesc.dt;
+    const bool af32 = (adt == DT_F32 || adt == DT_F32_8Q), bf32 = (bdt == DT_F32 || bdt == DT_F32_8Q);
+    if ((!af32 && adt != DT_U8_Q) || (!bf32 && bdt != DT_I8) || (cdt != DT_F32 && cdt != DT_I32)) {
+        return NOT_SUPPORTED;
+    }
+    if (s.M == 1 || s.N == 1) {
+        // the reference quantises the operands the other way round for a vector result (A -> I8,
+        // B -> U8_Q, matmul.cpp:376-382) and goes through matrix_vector_multiply; not wired up here
+        return NOT_SUPPORTED;
+    }
+    if ((!af32 && scaleA <= 0) || (!bf32 && scaleB <= 0)) {
+        return NOT_MATCH;
+    }
+    if (s.batch == 0 || s.M == 0 || s.N == 0) {
+        return SUCCESS;
+    }
+    if (!tmp || tmpBytes < s.total) {
+        return tmp ? NOT_MATCH : NULL_POINTER;
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const void *dA = matrixA, *dB = matrixB;
+    void *dC = matrixC;
+    U8 *dT = (U8 *)tmp;
+    const size_t aB = s.elemsA * bytesOf(adt), bB = s.elemsB * bytesOf(bdt), cB = (size_t)s.batch * s.M * s.N * 4;
+    if (arch == AMD_GFX950) {
+        void *a = st.get(aB), *b = st.get(bB);
+        dC = st.get(cB);
+        dT = (U8 *)st.get(s.total);
+        if (!a || !b || !dC || !dT) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(a, matrixA, aB, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(b, matrixB, bB, hipMemcpyHostToDevice, c.stream));
+        dA = a;
+        dB = b;
+    } else if (!aligned4(matrixA) || !aligned4(matrixB) || !aligned4(matrixC) || ((uintptr_t)tmp & 15)) {
+        return fail(NOT_SUPPORTED, "device operands must be 4-byte aligned, tmp 16-byte aligned");
+    }
+    float *sc = (float *)(dT + s.offScale);  // [0] = scale of A, [1] = scale of B, [2] = their product
+    const uint8_t *qA = (const uint8_t *)dA;
+    const int8_t *qB = (const int8_t *)dB;
+    // Whole-tensor quantisation, the caller's scale as the floor (quantize_cpu with its default mode,
+    // matmul.cpp:401-421): A -> U8_Q, B -> I8.
+    if (af32) {
+        HIP_TRY(launch_absmax_f32((const float *)dA, (U32)s.elemsA, c.ws, c.stream));
+        HIP_TRY(launch_quantize_f32((const float *)dA, (U32)s.elemsA, dT + s.offQA, 1, c.ws, scaleA, nullptr, 0, sc + 0,
+            c.stream));
+        qA = dT + s.offQA;
+    } else {
+        HIP_TRY(launch_fill_u32((uint32_t *)(sc + 0), 1, f32_bits(scaleA), c.stream));
+    }
+    if (bf32) {
+        HIP_TRY(launch_absmax_f32((const float *)dB, (U32)s.elemsB, c.ws, c.stream));
+        HIP_TRY(launch_quantize_f32((const float *)dB, (U32)s.elemsB, dT + s.offQB, 0, c.ws, scaleB, nullptr, 0, sc + 1,
+            c.stream));
+        qB = (const int8_t *)(dT + s.offQB);
+    } else {
+        HIP_TRY(launch_fill_u32((uint32_t *)(sc + 1), 1, f32_bits(scaleB), c.stream));
+    }
+    HIP_TRY(launch_mul_scalars(sc + 2, sc + 0, sc + 1, c.stream));  // scaleO = sA * sB (:411-420)
+
+    // One slice at a time, B packed into tmp per slice exactly as matrix_matrix_multiply does for an
+    // unpacked right-hand side (mmm.cpp:206-218).
+    int8_t *blob = (int8_t *)(dT + s.offBlob);
+    int32_t *comp = (int32_t *)((U8 *)blob + packed_matrix_bytes(s.N, s.K));
+    for (U32 ic = 0; ic < s.batch; ++ic) {
+        const int8_t *bs = qB + (s.batchB == 1 ? 0 : (size_t)ic * s.K * s.N);
+        if (ic == 0 || s.batchB != 1) {
+            HIP_TRY(launch_pack_mmm(bs, transposeB ? 1 : s.N, transposeB ? s.K : 1, s.K, s.N, blob, comp, c.stream));
+        }
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = qA + (s.batchA == 1 ? 0 : (size_t)ic * s.M * s.K);
+        g.lda = transposeA ? s.M : s.K;
+        g.transA = transposeA ? 1 : 0;
+        g.Bp = blob;
+        g.M = s.M;
+        g.N = s.N;
+        g.K = s.K;
+        g.comp = comp;
+        g.ob = comp;
+        g.C = (U8 *)dC + (size_t)ic * s.M * s.N * 4;
+        if (cdt == DT_F32) {
+            g.epi.mode = EPI_F32;
+            g.epi.dfactor = sc + 2;
+        } else {
+            g.epi.mode = EPI_I32;
+        }
+        HIP_TRY(launch_gemm_u8s8(g, c.stream));
+    }
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(matrixC, dC, cB, hipMemcpyDeviceToHost, c.stream));
         HIP_TRY(hipStreamSynchronize(c.stream));
     }
     return SUCCESS;

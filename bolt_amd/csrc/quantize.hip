@@ -41,6 +41,17 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st)
     return hipGetLastError();
 }
 
+__global__ void mul_scalars_kernel(float *out, const float *a, const float *b)
+{
+    out[0] = a[0] * b[0];
+}
+
+hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st)
+{
+    hipLaunchKernelGGL(mul_scalars_kernel, dim3(1), dim3(1), 0, st, out, a, b);
+    return hipGetLastError();
+}
+
 // ---- |max| reductions ---------------------------------------------------------------------------
 // avx512/quantize.cpp:21-68: sign bit cleared, vmaxps (a NaN never replaces the running max).
 template <int VEC>

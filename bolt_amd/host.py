@@ -223,3 +223,32 @@ def fully_connected(x, scaleI, filt, fdf, scaleW, bias, M, K, N, odt, scaleO=-1.
                                      tensor2df(odt, DF_NORMAL, M, N), ptr(out), C.byref(so), arch)
     check(e, "fully_connected")
     return out, np.float32(so.value)
+
+
+# ---- int8 matmul ------------------------------------------------------------------------------------------
+def tensor_nd(dt, shape):
+    """TensorDesc for a row-major array of `shape` (outermost first), DF_NCHW like the reference's matmul operands."""
+    d = TensorDesc()
+    d.dt, d.df, d.nDims = dt, 0, len(shape)
+    for i, v in enumerate(reversed(shape)):
+        d.dims[i] = v
+    return d
+
+
+def matmul(A, adt, a_shape, transposeA, scaleA, B, bdt, b_shape, transposeB, scaleB, c_shape, cdt=DT_F32):
+    """Mirrors matmul (compute/tensor/src/matmul.cpp:302-576, x86 int8 branch). Shapes are the stored ones."""
+    arch = arch_of(A)
+    ad, bd, cd = tensor_nd(adt, a_shape), tensor_nd(bdt, b_shape), tensor_nd(cdt, c_shape)
+    nb = _u32()
+    check(lib().matmul_infer_forward_tmp_bytes_gfx950(ad, bool(transposeA), bd, bool(transposeB), cd, C.byref(nb), arch),
+          "matmul_tmp_bytes")
+    tmp = _empty_like_mode(A, nb.value)
+    count = int(np.prod(c_shape))
+    if _is_torch(A):
+        import torch
+        out = torch.zeros(count, dtype=torch.float32 if cdt == DT_F32 else torch.int32, device=A.device)
+    else:
+        out = np.zeros(count, NP_OF[cdt])
+    check(lib().matmul_gfx950(ad, bool(transposeA), ptr(A), float(np.float32(scaleA)), bd, bool(transposeB), ptr(B),
+                              float(np.float32(scaleB)), nb.value, ptr(tmp), cd, ptr(out), arch), "matmul")
+    return out

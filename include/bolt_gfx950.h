@@ -21,6 +21,7 @@
 #ifndef BOLT_GFX950_NO_TYPES
 #include "bolt_types.h"
 #endif
+#include <stdbool.h>
 #include <stddef.h>
 
 #ifdef __cplusplus
@@ -108,6 +109,22 @@ EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDe
 EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScale, TensorDesc filterDesc,
     const void *filter, F32 filterScale, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
     TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch);
+
+/* ---- tensor_computing: int8 matmul ---------------------------------------------------- */
+/* compute/tensor/src/matmul.cpp:203-300 (matmul_infer_forward_tmp_bytes) and :302-576 (matmul), the
+ * x86 int8 branch with the Tensor arguments unwrapped: fp32 operands are quantised as whole tensors
+ * (A -> U8_Q, B -> I8, the caller's scale as a floor; pass 0 or less for none), operands that
+ * already have those types come with their scale; every 2-D slice [.., M, K] x [.., K, N] then goes
+ * through matrix_matrix_multiply with B packed per slice, and C = cvt(acc) * (1 / (scaleA * scaleB))
+ * (DT_F32) or the raw accumulators (DT_I32). Leading dimensions of A and B must equal C's or be
+ * absent (a 2-D operand is shared by all slices). The bias copy of the reference is not part of the
+ * int8 branch's result and is left out. Vector results (M == 1 or N == 1) are NOT_SUPPORTED: the
+ * reference swaps the operand types there and uses matrix_vector_multiply. */
+EE matmul_infer_forward_tmp_bytes_gfx950(TensorDesc matrixADesc, bool transposeA, TensorDesc matrixBDesc, bool transposeB,
+    TensorDesc matrixCDesc, U32 *bytes, Arch arch);
+EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F32 scaleA, TensorDesc matrixBDesc,
+    bool transposeB, const void *matrixB, F32 scaleB, U32 tmpBytes, void *tmp, TensorDesc matrixCDesc, void *matrixC,
+    Arch arch);
 
 /* ---- tensor_computing: int8 convolution ---------------------------------------------- */
 /* The inner (TensorDesc + pointer) forms the reference's convolution*() reach on x86:
