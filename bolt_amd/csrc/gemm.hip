@@ -156,15 +156,20 @@ struct GemmTile {
 // a convolution (NCHWC16: a pixel's 16 channels are contiguous, consecutive pixels follow each
 // other) one contiguous KiB. The per-column terms (offsetC - compensation, reciprocal channel
 // scale, bias) depend only on the lane and the tile column and are set up once.
-template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
+// FULL: the block tile lies wholly inside C and rows of C are 16-byte granular, so no bounds test, no
+// scalar tail and -- what matters -- no control flow: the compiler can then count outstanding memory
+// operations exactly instead of draining them (s_waitcnt vmcnt(0)) between row blocks, which would
+// serialise every wave on the round trip of its own stores. CIN: 0 = C is not read, 1 = it is,
+// 2 = decided at run time (edge tiles).
+template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
     (void)smem;
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
-    const bool use_cin = !CONV && a.add_cin && MODE != EPI_U8;
-    const bool n_vec = CONV || ((a.N & 3) == 0);
+    const bool use_cin = (CIN == 2) ? (!CONV && a.add_cin && MODE != EPI_U8) : (CIN == 1);
+    const bool n_vec = FULL || CONV || ((a.N & 3) == 0);
     int lane_max = 0;
 
     float factor = 0.0f, sI = 0.0f;
@@ -189,7 +194,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const bool ok = n + c < a.N;
+            const bool ok = FULL || (n + c < a.N);
             base[y][c] = ok ? (uint32_t)a.ob[n + c] - (uint32_t)a.comp[n + c] : 0u;
             qs[y][c] = 1.0f;
             bs[y][c] = 0.0f;
@@ -218,9 +223,9 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         {                                                                                 \
             const uint32_t n_ = n0 + (wn * TN + y) * 16 + 4 * g;                          \
             cin[buf][y] = (v4i){0, 0, 0, 0};                                              \
-            if (m_ < a.M && n_ < a.N) {                                                   \
+            if (FULL || (m_ < a.M && n_ < a.N)) {                                         \
                 const int32_t *p_ = (const int32_t *)a.C + (size_t)m_ * a.N + n_;         \
-                if (n_vec && n_ + 4 <= a.N) {                                             \
+                if (FULL || (n_vec && n_ + 4 <= a.N)) {                                   \
                     cin[buf][y] = *(const v4i *)p_;                                       \
                 } else {                                                                  \
                     for (int c = 0; c < 4 && n_ + c < a.N; ++c) {                         \
@@ -237,7 +242,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             BG_LOAD_CIN(x + 1, (x + 1) & 1);  // the next row block's C_in is in flight while this one is stored
         }
         const uint32_t m = m0 + (wm * TM + x) * 16 + i;
-        if (m >= a.M) {
+        if (!FULL && m >= a.M) {
             continue;
         }
         size_t rowbase = (size_t)m * a.N;
@@ -250,10 +255,10 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 #pragma unroll
         for (int y = 0; y < TN; ++y) {
             const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
-            if (n >= a.N) {
+            if (!FULL && n >= a.N) {
                 continue;
             }
-            const bool vec = n_vec && (n + 4 <= a.N);
+            const bool vec = FULL || (n_vec && (n + 4 <= a.N));
             int t[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -271,7 +276,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 if (MODE == EPI_I32) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        if (n + c < a.N) {
+                        if (FULL || n + c < a.N) {
                             const int av = (t[c] == (int)0x80000000) ? t[c] : (t[c] < 0 ? -t[c] : t[c]);
                             lane_max = av > lane_max ? av : lane_max;
                         }
@@ -309,7 +314,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                     if (MODE == EPI_F32) {
                         f[c] = (float)t[c] * factor;
                         if (CONV) {  // cvt * (1/s), + eltwise, fp32 ReLU (convolution_direct.cpp:2410-2422)
-                            if (a.conv.eltwise && n + c < a.N) {
+                            if (a.conv.eltwise && (FULL || n + c < a.N)) {
                                 f[c] = f[c] + a.conv.eltwise[idx + c];
                             }
                             if (a.conv.relu && !(f[c] > 0.0f)) {
@@ -343,6 +348,21 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     }
 }
 
+template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
+{
+    const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
+    const bool cin = !CONV && a.add_cin && MODE != EPI_U8;
+    if (full && !cin) {
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0);
+    } else if (full && MODE != EPI_U8 && !CONV) {
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1>(a, acc, smem, lane, wave, m0, n0);
+    } else {
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2>(a, acc, smem, lane, wave, m0, n0);
+    }
+}
+
 template <int WM, int WN, int TM, int TN, bool CONV = false>
 __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes)
@@ -350,26 +370,26 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
     (void)lds_bytes;
     if (CONV) {
         if (a.epi.mode == EPI_I32) {
-            epilogue_rows<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else if (a.epi.mode == EPI_U8) {
-            epilogue_rows<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else {
-            epilogue_rows<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         }
         return;
     }
     switch (a.epi.mode) {
         case EPI_I32:
-            epilogue_rows<EPI_I32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_I32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         case EPI_F32:
-            epilogue_rows<EPI_F32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_F32, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         case EPI_U8:
-            epilogue_rows<EPI_U8, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_U8, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         default:
-            epilogue_rows<EPI_F32_CH, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_F32_CH, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
     }
 }
