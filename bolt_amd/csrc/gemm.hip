@@ -545,7 +545,7 @@ __device__ __forceinline__ constexpr int vmcnt_imm(int n)
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE, bool CONV = false>
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
@@ -642,7 +642,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 // a table in memory would put a vector load, and with it a wait on every tile fetch in flight,
 // into each step. Chunks past the last tap (K padded to 64) read the pixel base; their weights are 0.
 #define BG_AOFF(tile) ((size_t)(tile)*64)
-    static_assert(!CONV || PIPE, "the convolution walk is wired into the fragment-prefetch loop");
+    static_assert(!CONV || PIPE == 1, "the convolution walk is wired into the fragment-prefetch loop");
     uint32_t cv_c16 = 0, cv_kw = 0, cv_kh = 0;
     const uint32_t cv_cpc = CONV ? a.conv.ICp / 16 : 1;
     if (CONV) {
@@ -675,7 +675,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             BG_CV_ADVANCE();
         }
     }
-    if constexpr (!PIPE) {
+    if constexpr (PIPE == 0) {
         for (uint32_t t = 0; t < ksteps; ++t) {
             // tile t is the oldest batch in flight; up to STAGES-2 younger ones may stay outstanding
             if (t + (STAGES - 2) < ksteps) {
@@ -708,6 +708,75 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
                 }
             }
         }
+    } else if constexpr (PIPE == 2) {
+        // Ping-pong schedule for 8 waves = two per SIMD. Each K tile is split into a memory phase
+        // (wait for the tile after next, request a new tile, read this tile's fragments from LDS,
+        // re-bias A) and a matrix phase (the TM x TN MFMAs and nothing else), with an s_barrier after
+        // each. Waves 4-7 run half a tile behind waves 0-3 (one extra barrier up front, one at the
+        // end for the others), so on every SIMD one wave is in its matrix phase while the other is in
+        // its memory phase: the matrix pipe never waits for loads, LDS or VALU work of the same wave.
+        //   visibility: a wave waits for its share of tile t+1 at the start of its memory phase t and
+        //   passes a barrier before any wave reads tile t+1 (memory phase t+1);
+        //   reuse: tile t+STAGES-1 is requested in memory phase t into the slot of tile t-1, whose
+        //   last readers (the late group's memory phase t-1) finished before the barrier just passed.
+        // Every wave executes 2 + 2 * ksteps barriers.
+        static_assert(WM * WN == 8, "ping-pong needs two waves per SIMD");
+        static_assert(STAGES >= 3, "ping-pong needs at least 3 stages");
+        v4i fa[TM], fb[TN];
+        const bool late = wave >= 4;
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));  // tile 0 landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (late) {
+            __builtin_amdgcn_s_barrier();
+        }
+        for (uint32_t t = 0; t < ksteps; ++t) {
+            // ---- memory phase
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * T::kLoads));  // my share of tile t+1 landed
+            asm volatile("" ::: "memory");
+            BG_ISSUE(t + (STAGES - 1), BG_CLAMP(t + (STAGES - 1)), BG_AOFF(BG_CLAMP(t + (STAGES - 1))));
+            {
+                const uint8_t *sA_ = smem + (t % STAGES) * T::kStageBytes;
+                const uint8_t *sB_ = sA_ + T::kAFrags * 1024;
+#pragma unroll
+                for (int y = 0; y < TN; ++y) {
+                    fb[y] = *(const v4i *)(sB_ + (wn * TN + y) * 1024 + lane * 16);
+                }
+#pragma unroll
+                for (int x = 0; x < TM; ++x) {
+                    fa[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + lane * 16);
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): fragments in registers before the matrix phase
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+                fa[x] ^= flip;
+            }
+            __builtin_amdgcn_sched_barrier(0);  // the re-bias belongs to the memory phase
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- matrix phase
+            __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+#pragma unroll
+                for (int y = 0; y < TN; ++y) {
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[x], acc[x][y], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
+        if (!late) {
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches
     } else {
         // Fragment-prefetch schedule: the fragments of tile t+1 are read from LDS into a second
         // register set while the MFMAs of tile t run, so no MFMA ever waits for an LDS read. That
@@ -791,7 +860,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES, bool PIPE = false, bool CONV = false>
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
@@ -902,6 +971,8 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 2, 8, 4, 4, true>(a, st);  // 256 x 128, fragment prefetch
         case 10:
             return launch_dma<2, 2, 4, 4, 4, true>(a, st);  // 128 x 128, fragment prefetch
+        case 11:
+            return launch_dma<2, 4, 8, 4, 4, 2>(a, st);  // 256 x 256, 8 waves, ping-pong memory / matrix phases
         default:
             break;
     }
