@@ -938,7 +938,7 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
         // that 128 x 128 tiles keep more CUs busy; tiny problems go to the general kernel
         const bool k64 = (a.K % 64 == 0);
         if (b256 >= 128 && k64) {
-            tile = 7;
+            tile = 11;  // ping-pong: 12 % faster than the fragment-prefetch loop at 8192^3, level elsewhere
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
             tile = k64 ? 10 : 2;
         }
