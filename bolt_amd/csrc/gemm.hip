@@ -860,6 +860,84 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
+// Skinny kernel for few rows (FullyConnected at small batch: M <= 64 per block, any N, K % 64 == 0).
+// The weight panel is the traffic, so a block owns ONE 16-column panel of B for up to 64 rows of A and
+// its 8 waves split K between them: each wave streams its K range straight from global memory / L2 into
+// registers (B fragment = 1 KiB contiguous in the packed layout, A fragments = 16 rows x 64 bytes), one
+// step ahead of the MFMAs, and the 8 partial accumulators meet in LDS. No barrier inside the K loop.
+__global__ __launch_bounds__(512) void gemm_u8s8_skinny_kernel(GemmArgs a)
+{
+    __shared__ v4i part[7][4][64];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * 16, m0 = blockIdx.y * 64;
+    const uint32_t ksteps = a.K / 64;
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+    // this wave's share of the K steps: a contiguous run
+    const uint32_t per = (ksteps + 7) / 8;
+    const uint32_t s0 = wave * per, s1 = (s0 + per < ksteps) ? s0 + per : ksteps;
+
+    const uint8_t *ap[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        uint32_t row = m0 + x * 16 + i;
+        row = row < a.M ? row : a.M - 1;  // rows past the end are computed and dropped
+        ap[x] = a.A + (size_t)row * a.lda + g * 16;
+    }
+    const int8_t *bp = a.Bp + (size_t)(n0 >> 4) * 16 * a.K + lane * 16;
+
+    v4i acc[4][1];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        acc[x][0] = (v4i){0, 0, 0, 0};
+    }
+    if (s0 < s1) {
+        v4i fb = *(const v4i *)(bp + (size_t)s0 * 1024);
+        v4i fa[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            fa[x] = *(const v4i *)(ap[x] + (size_t)s0 * 64);
+        }
+        for (uint32_t s = s0; s < s1; ++s) {
+            const uint32_t sn = (s + 1 < s1) ? s + 1 : s;  // the last step refetches itself: no branch around the loads
+            const v4i nb = *(const v4i *)(bp + (size_t)sn * 1024);
+            v4i na[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                na[x] = *(const v4i *)(ap[x] + (size_t)sn * 64);
+            }
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                acc[x][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb, fa[x] ^ flip, acc[x][0], 0, 0, 0);
+            }
+            fb = nb;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                fa[x] = na[x];
+            }
+        }
+    }
+    if (wave != 0) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            part[wave - 1][x][lane] = acc[x][0];
+        }
+    }
+    __syncthreads();
+    if (wave != 0) {
+        return;
+    }
+#pragma unroll
+    for (int w = 0; w < 7; ++w) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            acc[x][0] += part[w][x][lane];
+        }
+    }
+    epilogue_panel<1, 1, 4, 1>(a, acc, nullptr, lane, 0u, m0, n0, 0);
+}
+
 template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
@@ -975,6 +1053,15 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 4, 8, 4, 4, 2>(a, st);  // 256 x 256, 8 waves, ping-pong memory / matrix phases
         default:
             break;
+    }
+    if (tile == 0 && g_force_tile < 0 && dma_ok && a.M <= 256) {
+        // few rows: one 16-column weight panel per block, K split over its 8 waves
+        hipLaunchKernelGGL(gemm_u8s8_skinny_kernel, dim3((a.N + 15) / 16, (a.M + 63) / 64), dim3(512), 0, st, a);
+        return hipGetLastError();
+    }
+    if (g_force_tile == 14 && dma_ok) {
+        hipLaunchKernelGGL(gemm_u8s8_skinny_kernel, dim3((a.N + 15) / 16, (a.M + 63) / 64), dim3(512), 0, st, a);
+        return hipGetLastError();
     }
     dim3 grid((a.N + 63) / 64, (a.M + 63) / 64);
     hipLaunchKernelGGL(gemm_u8s8_general_kernel, grid, dim3(256), 0, st, a);
