@@ -4,26 +4,63 @@
 //   border reads 128          (Bolt x86: compute/tensor/src/cpu/x86/int8/avx512/convolution_direct.cpp:2584-2809)
 // = round(bias * s) + sum over taps inside the image of (in_u8 - 128) * w_s8.
 //
-// Three launches:
+// Launches:
 //   1. conv_pad_kernel      u8 NCHWC8 / NCHWC16 activations -> s8 (x - 128), zero-padded border and
 //                           channel tail, channel-innermost [n][Hp][Wp][ICp]. After this the 16
 //                           K-bytes a lane feeds to one MFMA are 16 consecutive channels of one tap:
 //                           one contiguous 16-byte load, no bounds checks, no re-bias in the loop.
 //   2. the pipelined GEMM kernel of gemm.hip in convolution mode (rows = output pixels, K ordered
-//      (kh, kw, c), a [K/16] table gives each 16-channel chunk's offset from the pixel's base).
-//      Epilogue: folded bias, integer ReLU + running max|acc| (int32 out) or dequantise + eltwise +
-//      fp32 ReLU (fp32 out), written in the reference's NCHWC16 / NCHWC8 output order.
-//   3. for u8 output: the tensor-wide dynamic requantisation of quantize.hip.
+//      (kh, kw, c); each lane steps its (kh, kw, 16-channel chunk) position in registers).
+//      Epilogue: folded bias, integer ReLU + running max|acc| (int32 out), dequantise + eltwise +
+//      fp32 ReLU (fp32 out), or the tensor-wide dynamic requantisation to u8 from a maximum found by
+//      a first, store-free pass; written in the reference's NCHWC16 / NCHWC8 output order.
 #include "device_common.h"
 #include "kernels.h"
 #include "layout.h"
 
 namespace bg {
 
-// one thread per 8 output bytes (8 channels of one padded pixel); consecutive threads write
-// consecutive bytes
+// One workgroup per padded image row (n, hp). The row is gathered plane by plane -- consecutive lanes read
+// consecutive pixels of one 8-channel plane, 8 contiguous bytes each -- into LDS in channel-innermost
+// order, re-biased to s8 on the way, and then streamed out linearly with 16-byte stores. Border pixels
+// and the channel tail stay zero.
 __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
     uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t row[];
+    const uint32_t n = blockIdx.x / Hp, hp = blockIdx.x % Hp;
+    const uint32_t row_bytes = Wp * ICp;
+    for (uint32_t o = threadIdx.x * 16; o < row_bytes; o += 256 * 16) {
+        *(v4i *)(row + o) = (v4i){0, 0, 0, 0};
+    }
+    __syncthreads();
+    if (hp >= pt && hp < pt + H) {
+        const uint32_t h = hp - pt, c8n = C / 8;
+        for (uint32_t idx = threadIdx.x; idx < c8n * W; idx += 256) {
+            const uint32_t c8 = idx / W, w = idx % W, c0 = c8 * 8;
+            // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
+            // 8 channels starting at c0 are contiguous for x = 8 and x = 16; a trailing block of an
+            // NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
+            const uint32_t blk = c0 / cx;
+            uint32_t bw = C - blk * cx;
+            bw = bw < cx ? bw : cx;
+            const size_t src = (size_t)n * C * H * W + (size_t)blk * cx * H * W + ((size_t)h * W + w) * bw + c0 % cx;
+            v2i v = *(const v2i *)(in + src);
+            v ^= (v2i){(int)0x80808080, (int)0x80808080};
+            *(v2i *)(row + (size_t)(w + pl) * ICp + c0) = v;
+        }
+    }
+    __syncthreads();
+    int8_t *dst = out + (size_t)blockIdx.x * row_bytes;
+    for (uint32_t o = threadIdx.x * 16; o < row_bytes; o += 256 * 16) {
+        *(v4i *)(dst + o) = *(const v4i *)(row + o);
+    }
+}
+
+// the same without LDS, for rows too wide to stage: one thread per 8 output bytes
+__global__ __launch_bounds__(256) void conv_pad_wide_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C,
+    uint32_t H, uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp,
+    int8_t *__restrict__ out)
 {
     const uint32_t c8n = ICp / 8;
     const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -41,9 +78,6 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict
     const uint32_t c0 = c8 * 8;
     if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W && c0 < C) {
         const uint32_t h = hp - pt, w = wp - pl;
-        // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
-        // 8 channels starting at c0 are contiguous for x = 8 and x = 16; a trailing block of an
-        // NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
         const uint32_t blk = c0 / cx;
         uint32_t bw = C - blk * cx;
         bw = bw < cx ? bw : cx;
@@ -62,8 +96,14 @@ hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H
     if (total == 0) {
         return hipSuccess;
     }
-    hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, in, N, C, H, W, cx, pt,
-        pl, Hp, Wp, ICp, out);
+    const uint32_t row_bytes = Wp * ICp;
+    if (row_bytes <= 65536 && (((uintptr_t)out & 15) == 0)) {
+        hipLaunchKernelGGL(conv_pad_kernel, dim3(N * Hp), dim3(256), row_bytes, st, in, N, C, H, W, cx, pt, pl, Hp, Wp, ICp,
+            out);
+    } else {
+        hipLaunchKernelGGL(conv_pad_wide_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, in, N, C, H, W,
+            cx, pt, pl, Hp, Wp, ICp, out);
+    }
     return hipGetLastError();
 }
 
