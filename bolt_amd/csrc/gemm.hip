@@ -161,6 +161,20 @@ struct GemmTile {
 // operations exactly instead of draining them (s_waitcnt vmcnt(0)) between row blocks, which would
 // serialise every wave on the round trip of its own stores. CIN: 0 = C is not read, 1 = it is,
 // 2 = decided at run time (edge tiles).
+// 16-byte result store. STREAM: a large matrix result is written once and not read again by this
+// kernel; stored normally, every round of tiles leaves 8 MiB of dirty lines per XCD in a 4 MiB L2 and
+// pushes out the A and B panels the next tiles of that XCD were sharing (measured: the K loop after
+// the first round of tiles runs 10-15 % slower). The non-temporal hint keeps the result out of the way.
+template <bool STREAM, typename V>
+__device__ __forceinline__ void store_c16(V *p, V v)
+{
+    if (STREAM) {
+        __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
+    }
+}
+
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
@@ -287,7 +301,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 if (CONV && !a.C) {
                     // abs-max pass only
                 } else if (vec) {
-                    *(v4i *)((int32_t *)a.C + idx) = (v4i){t[0], t[1], t[2], t[3]};
+                    store_c16<false>((v4i *)((int32_t *)a.C + idx), (v4i){t[0], t[1], t[2], t[3]});
                 } else {
                     for (int c = 0; c < 4 && n + c < a.N; ++c) {
                         ((int32_t *)a.C)[idx + c] = t[c];
@@ -329,7 +343,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                     }
                 }
                 if (vec) {
-                    *(v4f *)((float *)a.C + idx) = (v4f){f[0], f[1], f[2], f[3]};
+                    store_c16<false>((v4f *)((float *)a.C + idx), (v4f){f[0], f[1], f[2], f[3]});
                 } else {
                     for (int c = 0; c < 4 && n + c < a.N; ++c) {
                         ((float *)a.C)[idx + c] = f[c];
@@ -348,12 +362,126 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     }
 }
 
+// Full-tile epilogue for 32-bit results of a matrix product, through a wave-private LDS panel.
+// Straight from the accumulators a store instruction covers 16 rows x 64 bytes: sixteen half cache
+// lines, which the memory pipeline takes several times longer to absorb than whole lines (measured:
+// 256 such stores of a CU take 3 us against 1 us for the same bytes as 4 rows x 256 bytes). So each
+// wave passes one 16 x 64 block of int32 accumulators at a time through 4.25 KiB of LDS (row pitch
+// 272 bytes: both the fragment-order writes and the row-order reads are conflict free) and comes out
+// with lane (r = lane / 16, c = lane % 16) holding columns 4c .. 4c+3 of row 4 * it + r: every
+// result store and every C_in load is then 4 rows x 256 contiguous bytes, and the per-column terms
+// shrink to four values per lane. The panel is private to the wave, so there is no barrier: LDS
+// operations of one wave execute in order.
+template <int MODE, int WM, int WN, int TM, int TN, int CIN, bool STREAM>
+__device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
+{
+    static_assert(TN == 4, "a wave's tile row must be 64 columns = 256 bytes of int32");
+    static_assert(MODE == EPI_I32 || MODE == EPI_F32 || MODE == EPI_F32_CH, "32-bit results only");
+    constexpr uint32_t kPitch = 272;
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    uint8_t *pan = smem + wave * (16 * kPitch);
+    uint8_t *wr = pan + i * kPitch + g * 16;  // + 64 * y
+    const uint8_t *rd = pan + g * kPitch + i * 16;  // + 4 * kPitch * it   (here g = row in group, i = column chunk)
+    const uint32_t n = n0 + wn * 64 + i * 4;
+    const uint32_t row0 = m0 + wm * TM * 16 + g;
+
+    float factor = 0.0f, sI = 0.0f;
+    if (MODE == EPI_F32) {
+        factor = epi_factor(a.epi);
+    } else if (MODE == EPI_F32_CH) {
+        sI = *a.epi.scaleI;
+    }
+    uint32_t base[4];
+    float qs[4], bs[4];
+    {
+        const v4i ob = *(const v4i *)(a.ob + n), cp = *(const v4i *)(a.comp + n);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            base[c] = (uint32_t)ob[c] - (uint32_t)cp[c];
+            qs[c] = 1.0f;
+            bs[c] = 0.0f;
+            if (MODE == EPI_F32_CH) {
+                qs[c] = 1.0f / (sI * a.epi.scaleW[n + c]);
+                bs[c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
+            }
+        }
+    }
+    v4i cin[2][4];
+#define BG_LOAD_CIN(xx, buf)                                                                           \
+    if (CIN) {                                                                                         \
+        _Pragma("unroll") for (int it = 0; it < 4; ++it)                                               \
+        {                                                                                              \
+            cin[buf][it] = *(const v4i *)((const int32_t *)a.C + (size_t)(row0 + (xx)*16 + it * 4) * a.N + n); \
+        }                                                                                              \
+    }
+    BG_LOAD_CIN(0, 0);
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+        if (x + 1 < TM) {
+            BG_LOAD_CIN(x + 1, (x + 1) & 1);
+        }
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            *(v4i *)(wr + 64 * y) = acc[x][y];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        v4i t[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            t[it] = *(const v4i *)(rd + 4 * kPitch * it);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const size_t idx = (size_t)(row0 + x * 16 + it * 4) * a.N + n;
+            int v[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                v[c] = (int)((uint32_t)t[it][c] + base[c] + (CIN ? (uint32_t)cin[x & 1][it][c] : 0u));  // int32 wrap
+            }
+            if (MODE == EPI_I32) {
+                store_c16<STREAM>((v4i *)((int32_t *)a.C + idx), (v4i){v[0], v[1], v[2], v[3]});
+            } else {
+                float f[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (MODE == EPI_F32) {
+                        f[c] = (float)v[c] * factor;
+                    } else {
+                        f[c] = (float)v[c] * qs[c];
+                        if (a.epi.bias) {
+                            f[c] = f[c] + bs[c];
+                        }
+                    }
+                }
+                store_c16<STREAM>((v4f *)((float *)a.C + idx), (v4f){f[0], f[1], f[2], f[3]});
+            }
+        }
+    }
+#undef BG_LOAD_CIN
+}
+
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
     const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
     const bool cin = !CONV && a.add_cin && MODE != EPI_U8;
+    if constexpr (!CONV && MODE != EPI_U8 && TN == 4) {
+        // smem: the kernel's LDS, free by now and at least 8 waves x 4352 bytes (the DMA kernels); null otherwise
+        if (full && smem) {
+            if (cin) {
+                epilogue_rows_lds<MODE, WM, WN, TM, TN, 1, false>(a, acc, smem, lane, wave, m0, n0);
+            } else {
+                epilogue_rows_lds<MODE, WM, WN, TM, TN, 0, false>(a, acc, smem, lane, wave, m0, n0);
+            }
+            return;
+        }
+    }
     if (full && !cin) {
         epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0);
     } else if (full && MODE != EPI_U8 && !CONV) {
@@ -508,7 +636,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_tiled_kernel(GemmArgs a
 #undef BG_LOAD_GLOBAL
 #undef BG_STORE_LDS
 
-    epilogue_panel<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+    epilogue_panel<WM, WN, TM, TN>(a, acc, nullptr, lane, wave, m0, n0, T::kLdsBytes);
 }
 
 // Pipelined kernel for K % 64 == 0 (the shapes that matter for throughput).
@@ -857,6 +985,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 #undef BG_CV_OFF
 #undef BG_CV_ADVANCE
     asm volatile("" ::"v"(warm));  // keeps the warming loads alive; the value itself is not used
+    if (!CONV) {
+        // the matrix epilogue stages results through LDS: every wave's tile fetches have landed (each
+        // drained its own above) and every wave has read its last fragments before anyone writes there
+        static_assert(CONV || T::kLdsBytes >= WM * WN * 16 * 272, "LDS too small for the epilogue panels");
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
     epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
