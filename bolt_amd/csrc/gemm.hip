@@ -474,7 +474,13 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
     if constexpr (!CONV && MODE != EPI_U8 && TN == 4) {
         // smem: the kernel's LDS, free by now and at least 8 waves x 4352 bytes (the DMA kernels); null otherwise
         if (full && smem) {
-            if (cin) {
+            if (a.stream_c) {
+                if (cin) {
+                    epilogue_rows_lds<MODE, WM, WN, TM, TN, 1, true>(a, acc, smem, lane, wave, m0, n0);
+                } else {
+                    epilogue_rows_lds<MODE, WM, WN, TM, TN, 0, true>(a, acc, smem, lane, wave, m0, n0);
+                }
+            } else if (cin) {
                 epilogue_rows_lds<MODE, WM, WN, TM, TN, 1, false>(a, acc, smem, lane, wave, m0, n0);
             } else {
                 epilogue_rows_lds<MODE, WM, WN, TM, TN, 0, false>(a, acc, smem, lane, wave, m0, n0);
@@ -1088,7 +1094,11 @@ static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
         attr_set = true;
     }
     const uint32_t tiles = ((a.N + T::kBN - 1) / T::kBN) * ((a.M + T::kBM - 1) / T::kBM);
-    hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), T::kLdsBytes, st, a);
+    GemmArgs b = a;
+    // a result much larger than the L2s (8 x 4 MiB) is written in several rounds of tiles: keep it from
+    // displacing the operand panels (measured at 8192^3: 6 % faster; at 64 MiB and below: level or slower)
+    b.stream_c = !CONV && (uint64_t)a.M * a.N * 4 > ((uint64_t)96 << 20);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), T::kLdsBytes, st, b);
     return hipGetLastError();
 }
 
@@ -1169,20 +1179,8 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_tiled<2, 2, 8, 8>(a, st);  // 256 x 256
         case 2:
             return launch_tiled<2, 2, 4, 4>(a, st);  // 128 x 128
-        case 3:
-            return launch_dma<2, 2, 8, 4, 3>(a, st);  // 256 x 128, 3 stages, 2 blocks / CU
-        case 4:
-            return launch_dma<2, 2, 4, 4, 4>(a, st);  // 128 x 128, 4 stages
-        case 5:
-            return launch_dma<2, 4, 8, 4, 4>(a, st);  // 256 x 256, 8 waves, 4 stages
-        case 6:
-            return launch_dma<2, 2, 8, 4, 4>(a, st);  // 256 x 128, 4 stages
         case 7:
             return launch_dma<2, 4, 8, 4, 4, true>(a, st);  // 256 x 256, 8 waves, fragment prefetch
-        case 8:
-            return launch_dma<2, 2, 8, 8, 4, true>(a, st);  // 256 x 256, 4 waves of 128 x 128
-        case 9:
-            return launch_dma<2, 2, 8, 4, 4, true>(a, st);  // 256 x 128, fragment prefetch
         case 10:
             return launch_dma<2, 2, 4, 4, 4, true>(a, st);  // 128 x 128, fragment prefetch
         case 11:

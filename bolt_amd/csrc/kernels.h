@@ -60,6 +60,7 @@ struct GemmArgs {
     const int32_t *comp; // blob's own compensation vector [N]
     void *C;             // [M][N] row-major
     int add_cin;         // accumulate into the int32 bits already in C
+    int stream_c;        // set by the launcher: write C with the non-temporal hint
     Epilogue epi;
     ConvGeom conv;       // used by launch_conv_u8s8 only
 };

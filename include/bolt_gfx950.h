@@ -36,9 +36,10 @@ EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
 /* Tuning / test knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1-2 the
- * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 3-10 the LDS-DMA kernel
- * variants (need K % 64 == 0); a variant whose shape requirement fails falls back to the general
- * kernel. Every variant returns the same bytes. */
+ * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 7 / 10 / 11 the LDS-DMA
+ * kernels (256x256 fragment-prefetch, 128x128 fragment-prefetch, 256x256 ping-pong; need
+ * K % 64 == 0), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
+ * the general kernel. Every variant returns the same bytes. */
 EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);

@@ -118,7 +118,7 @@ def test_mmm_all_outputs_device(torch_mod, oracle, M, K, N):
     assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 14])
+@pytest.mark.parametrize("tile", [0, 1, 2, 7, 10, 11, 14])
 def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
     """Each GEMM kernel (general, register-staged tiles, LDS-DMA pipelines) is forced in turn on
     shapes with ragged M / N edges, one and many K tiles, and all four epilogues."""
@@ -175,6 +175,31 @@ def test_mmm_full_size_properties(torch_mod, oracle):
     rows = [0, 1, 255, 256, 2047, 4095]
     want = oracle.mmm(A1[rows].cpu().numpy(), Wh, offh, np.zeros((len(rows), N), np.int32), DT_I32)
     assert np.array_equal(C1[rows].cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("cdt,scale", [(DT_I32, None), (DT_F32, [37.25])])
+def test_mmm_large_result_streamed(torch_mod, oracle, cdt, scale):
+    """A result above 96 MiB is written with streaming stores (a different epilogue instantiation):
+    5184 x 5184 x 4 bytes, K = 64 so that the oracle still finishes in seconds; C_in non-zero."""
+    torch = torch_mod
+    M = N = 5184
+    K = 64
+    rng = np.random.default_rng(5184)
+    A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    off = oracle.offsetC(W, True) + rng.integers(-5000, 5000, size=N, dtype=np.int32)
+    Cin = rng.integers(-100000, 100000, size=(M, N), dtype=np.int32)
+    blob, bd, rhs = host.mmm_transform_rhs(torch.from_numpy(W).cuda(), DF_TRANSPOSE, K, N)
+    Cd = torch.from_numpy(Cin.copy()).cuda()
+    if cdt == DT_F32:
+        Cd = Cd.view(torch.float32)
+    say("streamed result", M, K, N, cdt)
+    capi.check(host.matrix_matrix_multiply(torch.from_numpy(A).cuda(), tensor2df(DT_U8_Q, DF_NORMAL, M, K), blob, bd,
+                                           torch.from_numpy(off).cuda().view(torch.uint8), Cd,
+                                           tensor2df(cdt, DF_NORMAL, M, N), scale), "mmm")
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    want = oracle.mmm(A, W, off, Cin.view(np.float32) if cdt == DT_F32 else Cin, cdt, scale=scale)
+    assert np.array_equal(Cd.cpu().numpy().view(np.int32), want.view(np.int32))
 
 
 def test_mmm_u8_epilogue_ties_and_saturation(torch_mod, oracle):
