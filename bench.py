@@ -122,8 +122,12 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         capi.check(L.bolt_gfx950_timer_stop(C.byref(ms)), "timer")
         return ms.value / reps
 
-    # -- int8 GEMM: square sweep + the BERT-base layer shapes (fp32 out = FullyConnected epilogue; int32 out = C += A.B)
+    # -- int8 GEMM: square sweep + the BERT-base layer shapes, through both callers of the kernel:
+    #    matrix_matrix_multiply (C += A.B: the int32 bits already in C are read and added, as the reference
+    #    does, for int32 and fp32 results; u8 results start from zero) and FullyConnected (starts from the
+    #    folded bias, never reads C; this is what a model's layers run)
     if want("gemm"):
+        from bolt_amd.capi import AMD_GFX950_DEVICE, DT_I8, tensor1d
         gemm = []
         for (M, K, N, reps) in ((2048, 2048, 2048, 50), (4096, 4096, 4096, 30), (8192, 8192, 8192, 10), (4096, 768, 768, 50),
                                 (4096, 768, 3072, 50), (4096, 3072, 768, 50)):
@@ -131,14 +135,34 @@ def other_kernels(L, capi, host, torch, dev, only=None):
             W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
             blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
             off = blob[rhs:rhs + 4 * N].clone()
+            bias = torch.randn(N, device=dev, generator=g) * 0.1
             ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
-            for cdt, tdt, sc, nm in ((DT_F32, torch.float32, [37.25], "f32"), (DT_I32, torch.int32, None, "i32_accumulate")):
+            fdesc = tensor2df(DT_I8, DF_NKNxKx, K, N)
+
+            def add(path, nm, t):
+                tops = 2.0 * M * N * K / t / 1e9
+                gemm.append({"M": M, "K": K, "N": N, "path": path, "out": nm, "ms": t, "tops": tops,
+                             "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
+            for cdt, tdt, sc, nm in ((DT_F32, torch.float32, [37.25], "f32"), (DT_I32, torch.int32, None, "i32_accumulate"),
+                                     (DT_U8_Q, torch.uint8, [-1.0, 1e-5], "u8")):
                 Cb = torch.zeros((M, N), dtype=tdt, device=dev)
                 cd = tensor2df(cdt, DF_NORMAL, M, N)
-                t = timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps)
-                tops = 2.0 * M * N * K / t / 1e9
-                gemm.append({"M": M, "K": K, "N": N, "out": nm, "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
-            del A, W, blob, Cb
+                add("matrix_matrix_multiply", nm,
+                    timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps))
+                del Cb
+            for odt, tdt, so0, nm in ((DT_F32, torch.float32, -1.0, "f32"), (DT_U8_Q, torch.uint8, 0.05, "u8_static_scale")):
+                nbytes = host.fully_connected_tmp_bytes(M, K, N, DF_NKNxKx, odt, AMD_GFX950_DEVICE)
+                tmp = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                out = torch.empty((M, N), dtype=tdt, device=dev)
+                so = C.c_float(so0)
+                od = tensor2df(odt, DF_NORMAL, M, N)
+                add("fully_connected", nm,
+                    timed(lambda: capi.check(L.fully_connected_gfx950(ad, host.ptr(A), 30.0, fdesc, host.ptr(blob), 100.0,
+                                                                      tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp),
+                                                                      od, host.ptr(out), C.byref(so), AMD_GFX950_DEVICE),
+                                             "fully_connected"), reps))
+                del tmp, out
+            del A, W, blob
         res["gemm_int8"] = gemm
     # -- C1: FullyConnected M=64 K=1024 N=1024, fp32 out
     if want("fc"):
@@ -147,9 +171,17 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
         blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
         bias = torch.randn(N, device=dev, generator=g) * 0.1
-        t = timed(lambda: host.fully_connected(x, 30.0, blob, DF_NKNxKx, 100.0, bias, M, K, N, DT_F32), 200)
+        from bolt_amd.capi import AMD_GFX950_DEVICE, DT_I8, tensor1d
+        nbytes = host.fully_connected_tmp_bytes(M, K, N, DF_NKNxKx, DT_F32, AMD_GFX950_DEVICE)
+        tmp = torch.empty(nbytes, dtype=torch.uint8, device=dev)     # reused across calls, as an engine's shared tmp is
+        out = torch.empty((M, N), dtype=torch.float32, device=dev)
+        so = C.c_float(-1.0)
+        idesc, fdesc, odesc = tensor2df(DT_U8_Q, DF_NORMAL, M, K), tensor2df(DT_I8, DF_NKNxKx, K, N), tensor2df(DT_F32, DF_NORMAL, M, N)
+        t = timed(lambda: capi.check(L.fully_connected_gfx950(idesc, host.ptr(x), 30.0, fdesc, host.ptr(blob), 100.0,
+                                                              tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp), odesc,
+                                                              host.ptr(out), C.byref(so), AMD_GFX950_DEVICE), "fully_connected"), 200)
         res["fc_c1"] = {"ms": t, "tops": 2.0 * M * N * K / t / 1e9, "algorithmic_bytes": 1380352,
-                        "gbps": 1380352 / t / 1e6, "note": "call-overhead bound: includes tmp/out allocation by the Python wrapper"}
+                        "gbps": 1380352 / t / 1e6, "note": "two launches (bias fold, GEMM) issued from Python through ctypes"}
     # -- C3: int8 3x3 convolution 32x64x56x56 -> 64, ReLU, u8 out with dynamic output scale
     if want("conv"):
         n, ic, ih, iw, oc = 32, 64, 56, 56, 64
