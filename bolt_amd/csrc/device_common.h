@@ -104,6 +104,19 @@ __device__ __forceinline__ float wave_reduce_max(float v)
     return v;
 }
 
+// Load / store for data that a kernel touches exactly once and that is too large to stay cached.
+template <typename V>
+__device__ __forceinline__ V ld_stream(const V *p)
+{
+    return __builtin_nontemporal_load(p);
+}
+
+template <typename V>
+__device__ __forceinline__ void st_stream(V *p, V v)
+{
+    __builtin_nontemporal_store(v, p);
+}
+
 __device__ __forceinline__ float wave_reduce_sum(float v)
 {
 #pragma unroll

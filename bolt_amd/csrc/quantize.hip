@@ -324,12 +324,30 @@ hipError_t launch_u8_to_i8(const uint8_t *x, uint32_t n, int8_t *q, hipStream_t 
 }
 
 // ---- dequantize: avx512/dequantize.cpp:18-101, f = cvt(q) * (1 / s) -----------------------------
-__global__ void dequant_i32_kernel(const int32_t *__restrict__ q, uint32_t n, const float *__restrict__ ds, float s,
-    float *__restrict__ out)
+__global__ __launch_bounds__(256) void dequant_i32_kernel(const int32_t *__restrict__ q, uint32_t n, const float *__restrict__ ds,
+    float s, float *__restrict__ out)
 {
     const float f = 1 / (ds ? *ds : s);
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    uint32_t done = 0;
+    if ((((uintptr_t)q | (uintptr_t)out) & 15) == 0) {
+        const uint32_t n4 = n / 4;
+        const v4i *q4 = (const v4i *)q;
+        v4f *o4 = (v4f *)out;
+        uint32_t i = tid;
+        for (; i + stride < n4; i += 2 * stride) {  // two independent 16-byte loads in flight
+            const v4i a = ld_stream(q4 + i), b = ld_stream(q4 + i + stride);
+            st_stream(o4 + i, (v4f){(float)a.x * f, (float)a.y * f, (float)a.z * f, (float)a.w * f});
+            st_stream(o4 + i + stride, (v4f){(float)b.x * f, (float)b.y * f, (float)b.z * f, (float)b.w * f});
+        }
+        for (; i < n4; i += stride) {
+            const v4i a = ld_stream(q4 + i);
+            o4[i] = (v4f){(float)a.x * f, (float)a.y * f, (float)a.z * f, (float)a.w * f};
+        }
+        done = n4 * 4;
+    }
+    for (uint32_t i = done + tid; i < n; i += stride) {
         out[i] = (float)q[i] * f;
     }
 }
