@@ -1788,7 +1788,10 @@ EE matmul_shape(TensorDesc a, bool tA, TensorDesc b, bool tB, TensorDesc c, Matm
     };
     s->offQA = take(s->elemsA);
     s->offQB = take(s->elemsB);
-    s->offBlob = take((size_t)s->N * 4 + packed_matrix_bytes(s->N, s->K) + 64);
+    // the operand that gets packed per slice: B (N x K) for a matrix result; A (M x K) when B is a single
+    // column (matrix_vector_multiply packs its unpacked matrix into tmp, mvm.cpp:176-182); nothing for M == 1
+    const U32 rowsP = (s->M != 1 && s->N == 1) ? s->M : s->N;
+    s->offBlob = take((size_t)rowsP * 4 + packed_matrix_bytes(rowsP, s->K) + 64);
     s->offScale = take(64);
     s->total = off;
     return SUCCESS;
@@ -1833,12 +1836,11 @@ EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F
     }
     const DataType adt = matrixADesc.dt, bdt = matrixBDesc.dt, cdt = matrixCDesc.dt;
     const bool af32 = (adt == DT_F32 || adt == DT_F32_8Q), bf32 = (bdt == DT_F32 || bdt == DT_F32_8Q);
-    if ((!af32 && adt != DT_U8_Q) || (!bf32 && bdt != DT_I8) || (cdt != DT_F32 && cdt != DT_I32)) {
-        return NOT_SUPPORTED;
-    }
-    if (s.M == 1 || s.N == 1) {
-        // the reference quantises the operands the other way round for a vector result (A -> I8,
-        // B -> U8_Q, matmul.cpp:376-382) and goes through matrix_vector_multiply; not wired up here
+    // A vector result goes through matrix_vector_multiply with the operands quantised the other way
+    // round: A -> I8, B -> U8_Q (matmul.cpp:374-382, :531-548).
+    const bool vec = (s.M == 1 || s.N == 1);
+    const DataType qadt = vec ? DT_I8 : DT_U8_Q, qbdt = vec ? DT_U8_Q : DT_I8;
+    if ((!af32 && adt != qadt) || (!bf32 && bdt != qbdt) || (cdt != DT_F32 && cdt != DT_I32)) {
         return NOT_SUPPORTED;
     }
     if ((!af32 && scaleA <= 0) || (!bf32 && scaleB <= 0)) {
@@ -1881,16 +1883,16 @@ EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F
     // matmul.cpp:401-421): A -> U8_Q, B -> I8.
     if (af32) {
         HIP_TRY(launch_absmax_f32((const float *)dA, (U32)s.elemsA, c.ws, c.stream));
-        HIP_TRY(launch_quantize_f32((const float *)dA, (U32)s.elemsA, dT + s.offQA, 1, c.ws, scaleA, nullptr, 0, sc + 0,
-            c.stream));
+        HIP_TRY(launch_quantize_f32((const float *)dA, (U32)s.elemsA, dT + s.offQA, vec ? 0 : 1, c.ws, scaleA, nullptr, 0,
+            sc + 0, c.stream));
         qA = dT + s.offQA;
     } else {
         HIP_TRY(launch_fill_u32((uint32_t *)(sc + 0), 1, f32_bits(scaleA), c.stream));
     }
     if (bf32) {
         HIP_TRY(launch_absmax_f32((const float *)dB, (U32)s.elemsB, c.ws, c.stream));
-        HIP_TRY(launch_quantize_f32((const float *)dB, (U32)s.elemsB, dT + s.offQB, 0, c.ws, scaleB, nullptr, 0, sc + 1,
-            c.stream));
+        HIP_TRY(launch_quantize_f32((const float *)dB, (U32)s.elemsB, dT + s.offQB, vec ? 1 : 0, c.ws, scaleB, nullptr, 0,
+            sc + 1, c.stream));
         qB = (const int8_t *)(dT + s.offQB);
     } else {
         HIP_TRY(launch_fill_u32((uint32_t *)(sc + 1), 1, f32_bits(scaleB), c.stream));
@@ -1901,7 +1903,42 @@ EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F
     // unpacked right-hand side (mmm.cpp:206-218).
     int8_t *blob = (int8_t *)(dT + s.offBlob);
     int32_t *comp = (int32_t *)((U8 *)blob + packed_matrix_bytes(s.N, s.K));
-    for (U32 ic = 0; ic < s.batch; ++ic) {
+    for (U32 ic = 0; ic < s.batch && vec; ++ic) {
+        const U8 *as = qA + (s.batchA == 1 ? 0 : (size_t)ic * s.M * s.K);
+        const U8 *bs = (const U8 *)qB + (s.batchB == 1 ? 0 : (size_t)ic * s.K * s.N);
+        void *cs = (U8 *)dC + (size_t)ic * s.M * s.N * 4;
+        Epilogue epi;
+        memset(&epi, 0, sizeof(epi));
+        epi.mode = (cdt == DT_F32) ? EPI_F32 : EPI_I32;
+        epi.dfactor = (cdt == DT_F32) ? sc + 2 : nullptr;
+        if (s.M == 1) {
+            // u8 matrix B (stored [K][N], or [N][K] if transposed) times the s8 row vector A (:531-539)
+            HIP_TRY(launch_gemv_u8s8(bs, transposeB ? s.K : 1, transposeB ? 1 : s.N, (const int8_t *)as, s.K, s.N, cs, epi,
+                c.stream));
+        } else {
+            // s8 matrix A (stored [M][K], or [K][M] if transposed) times the u8 column vector B (:540-548);
+            // the matrix is packed into tmp with its compensation in front, the result starts from zero
+            int32_t *vcomp = (int32_t *)blob;
+            int8_t *vmat = (int8_t *)blob + (size_t)s.M * 4;
+            if (ic == 0 || s.batchA != 1) {
+                HIP_TRY(launch_pack_mvm((const int8_t *)as, transposeA ? s.M : 1, transposeA ? 1 : s.K, s.K, s.M, vmat, vcomp,
+                    c.stream));
+            }
+            GemvArgs g;
+            memset(&g, 0, sizeof(g));
+            g.W = vmat;
+            g.ldw = align_up(s.K, 8);
+            g.x = bs;
+            g.K = s.K;
+            g.N = s.M;
+            g.ob = vcomp;
+            g.comp = vcomp;
+            g.y = cs;
+            g.epi = epi;
+            HIP_TRY(launch_gemv_s8u8(g, c.stream));
+        }
+    }
+    for (U32 ic = 0; ic < s.batch && !vec; ++ic) {
         const int8_t *bs = qB + (s.batchB == 1 ? 0 : (size_t)ic * s.K * s.N);
         if (ic == 0 || s.batchB != 1) {
             HIP_TRY(launch_pack_mmm(bs, transposeB ? 1 : s.N, transposeB ? s.K : 1, s.K, s.N, blob, comp, c.stream));

@@ -119,8 +119,10 @@ EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScal
  * through matrix_matrix_multiply with B packed per slice, and C = cvt(acc) * (1 / (scaleA * scaleB))
  * (DT_F32) or the raw accumulators (DT_I32). Leading dimensions of A and B must equal C's or be
  * absent (a 2-D operand is shared by all slices). The bias copy of the reference is not part of the
- * int8 branch's result and is left out. Vector results (M == 1 or N == 1) are NOT_SUPPORTED: the
- * reference swaps the operand types there and uses matrix_vector_multiply. */
+ * int8 branch's result and is left out. For a vector result (M == 1 or N == 1) the reference swaps
+ * the operand types (A -> I8, B -> U8_Q, :374-382) and goes through matrix_vector_multiply per
+ * slice (:531-548): u8 matrix B x s8 row vector A when M == 1, s8 matrix A (packed into tmp) x u8
+ * column vector B otherwise; operands handed over already quantised must then be I8 / U8_Q. */
 EE matmul_infer_forward_tmp_bytes_gfx950(TensorDesc matrixADesc, bool transposeA, TensorDesc matrixBDesc, bool transposeB,
     TensorDesc matrixCDesc, U32 *bytes, Arch arch);
 EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F32 scaleA, TensorDesc matrixBDesc,

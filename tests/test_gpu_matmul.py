@@ -97,7 +97,79 @@ def test_matmul_errors(torch_mod):
     assert L.matmul_infer_forward_tmp_bytes_gfx950(a, False, b, False, c, capi.C.byref(nb), 0) == capi.NOT_SUPPORTED
     assert L.matmul_infer_forward_tmp_bytes_gfx950(a, False, b, False, c, capi.C.byref(nb), capi.AMD_GFX950) == 0
     x = np.zeros(32, np.float32)
-    v = host.tensor_nd(DT_F32, (8, 1))
+    v = host.tensor_nd(DT_U8_Q, (8, 1))   # a vector result wants B as U8_Q (or fp32), not I8
     cv = host.tensor_nd(DT_F32, (4, 1))
-    assert L.matmul_gfx950(a, False, x.ctypes.data, -1.0, v, False, x.ctypes.data, -1.0, 1 << 20, x.ctypes.data, cv,
+    vi = host.tensor_nd(DT_I8, (8, 1))
+    assert L.matmul_gfx950(a, False, x.ctypes.data, -1.0, vi, False, x.ctypes.data, 1.0, 1 << 20, x.ctypes.data, cv,
                            x.ctypes.data, capi.AMD_GFX950) == capi.NOT_SUPPORTED
+
+
+def oracle_matmul_vector(oracle, A, tA, B, tB, cdt):
+    """Vector result: A -> I8, B -> U8_Q, then matrix_vector_multiply per slice (matmul.cpp:374-382, :531-548)."""
+    qa, sa = oracle.quantize_f32(A.reshape(-1), DT_I8)
+    qb, sb = oracle.quantize_f32(B.reshape(-1), DT_U8_Q)
+    A3 = qa.reshape((-1,) + A.shape[-2:])
+    B3 = qb.reshape((-1,) + B.shape[-2:])
+    batch = max(A3.shape[0], B3.shape[0])
+    s = np.float32(sa) * np.float32(sb)
+    M = A.shape[-1] if tA else A.shape[-2]
+    N = B.shape[-2] if tB else B.shape[-1]
+    ydt = np.float32 if cdt == DT_F32 else np.int32
+    sc = [s] if cdt == DT_F32 else None
+    outs = []
+    for i in range(batch):
+        a = A3[i % A3.shape[0]]
+        b = B3[i % B3.shape[0]]
+        if M == 1:
+            # u8 matrix b ([K, N], or [N, K] if tB) times the s8 vector a
+            outs.append(oracle.mvm_u8mat(b, a.reshape(-1), np.zeros(N, ydt), cdt, scale=sc, a_is_KM=not tB))
+        else:
+            # s8 matrix a ([M, K], or [K, M] if tA) times the u8 vector b
+            off = oracle.offsetC(a, not tA)
+            outs.append(oracle.mvm(a, b.reshape(-1), off, np.zeros(M, ydt), cdt, scale=sc, w_is_NK=not tA))
+    return np.stack(outs), sa, sb
+
+
+VECTOR_CASES = [  # (A shape, transposeA, B shape, transposeB): one of M, N is 1
+    ((1, 64), False, (64, 48), False),                       # row vector x matrix
+    ((1, 100), False, (37, 100), True),                      # ... with B stored [N, K]
+    ((2, 3, 1, 64), False, (2, 3, 64, 128), False),          # decode-step attention scores: q [1, d] x K^T
+    ((50, 72), False, (72, 1), False),                       # matrix x column vector
+    ((72, 50), True, (72, 1), False),                        # ... with A stored [K, M]
+    ((4, 130, 96), False, (4, 96, 1), False),
+    ((3, 1, 40), False, (40, 1), False),                     # both: treated as the row-vector case
+    ((2100, 256), False, (256, 1), False),                   # enough rows for the two-rows-per-wave kernel
+]
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+@pytest.mark.parametrize("case", VECTOR_CASES)
+def test_matmul_int8_vector_result(torch_mod, oracle, device_mode, case):
+    torch = torch_mod
+    a_shape, tA, b_shape, tB = case
+    print("matmul vector", device_mode, case, flush=True)
+    rng = np.random.default_rng(sum(a_shape) + 7 * sum(b_shape))
+    A = rng.standard_normal(a_shape).astype(np.float32)
+    B = rng.standard_normal(b_shape).astype(np.float32)
+    M = a_shape[-1] if tA else a_shape[-2]
+    N = b_shape[-2] if tB else b_shape[-1]
+    lead = a_shape[:-2] if len(a_shape) >= len(b_shape) else b_shape[:-2]
+    c_shape = tuple(lead) + (M, N)
+
+    def put(x):
+        return torch.from_numpy(np.ascontiguousarray(x)).cuda() if device_mode else np.ascontiguousarray(x)
+    for cdt in (DT_F32, DT_I32):
+        want, sa, sb = oracle_matmul_vector(oracle, A, tA, B, tB, cdt)
+        got = host.matmul(put(A), DT_F32, a_shape, tA, -1.0, put(B), DT_F32, b_shape, tB, -1.0, c_shape, cdt)
+        if device_mode:
+            capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+            got = got.cpu().numpy()
+        assert np.array_equal(got.reshape(want.shape).view(np.int32), want.reshape(want.shape).view(np.int32)), (case, cdt)
+    qa, sa = oracle.quantize_f32(A.reshape(-1), DT_I8)
+    qb, sb = oracle.quantize_f32(B.reshape(-1), DT_U8_Q)
+    got = host.matmul(put(qa), DT_I8, a_shape, tA, sa, put(qb), DT_U8_Q, b_shape, tB, sb, c_shape, DT_F32)
+    if device_mode:
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        got = got.cpu().numpy()
+    want, _, _ = oracle_matmul_vector(oracle, A, tA, B, tB, DT_F32)
+    assert np.array_equal(got.reshape(want.shape).view(np.int32), want.view(np.int32))
