@@ -307,6 +307,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
         gemm_force_tile(value);
         return SUCCESS;
     }
+    if (strcmp(name, "conv_panel") == 0) {
+        if (value != 0 && value != 2 && value != 4) {
+            return NOT_MATCH;
+        }
+        conv_force_panel(value);
+        return SUCCESS;
+    }
     return NOT_FOUND;
 }
 

@@ -6,9 +6,11 @@
 //
 // Launches:
 //   1. conv_pad_kernel      u8 NCHWC8 / NCHWC16 activations -> s8 (x - 128), zero-padded border and
-//                           channel tail, channel-innermost [n][Hp][Wp][ICp]. After this the 16
-//                           K-bytes a lane feeds to one MFMA are 16 consecutive channels of one tap:
-//                           one contiguous 16-byte load, no bounds checks, no re-bias in the loop.
+//                           channel tail, in planes of 16 channels: [n][ICp/16][Hp][Wp][16]. After this
+//                           the 16 K-bytes a lane feeds to one MFMA are 16 consecutive channels of one
+//                           tap -- one contiguous 16-byte load, no bounds checks, no re-bias in the loop --
+//                           and the 16 lanes that hold consecutive output pixels of a fragment read
+//                           consecutive 16-byte pieces (whole cache lines for unit stride).
 //   2. the pipelined GEMM kernel of gemm.hip in convolution mode (rows = output pixels, K ordered
 //      (kh, kw, c); each lane steps its (kh, kw, 16-channel chunk) position in registers).
 //      Epilogue: folded bias, integer ReLU + running max|acc| (int32 out), dequantise + eltwise +
@@ -20,90 +22,68 @@
 
 namespace bg {
 
-// One workgroup per padded image row (n, hp). The row is gathered plane by plane -- consecutive lanes read
-// consecutive pixels of one 8-channel plane, 8 contiguous bytes each -- into LDS in channel-innermost
-// order, re-biased to s8 on the way, and then streamed out linearly with 16-byte stores. Border pixels
-// and the channel tail stay zero.
+// One wave per row (n, 16-channel plane, hp) of the padded image, one lane per pixel: a lane reads the
+// pixel's 16 (or 8) channels from the NCHWC8 / NCHWC16 input -- consecutive lanes read consecutive
+// pixels, 8 or 16 contiguous bytes each -- re-biases them to s8 and writes 16 contiguous bytes. Border
+// pixels and the channel tail are zero. The row decomposition is wave-uniform (scalar arithmetic).
 __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
     uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t row[];
-    const uint32_t n = blockIdx.x / Hp, hp = blockIdx.x % Hp;
-    const uint32_t row_bytes = Wp * ICp;
-    for (uint32_t o = threadIdx.x * 16; o < row_bytes; o += 256 * 16) {
-        *(v4i *)(row + o) = (v4i){0, 0, 0, 0};
-    }
-    __syncthreads();
-    if (hp >= pt && hp < pt + H) {
-        const uint32_t h = hp - pt, c8n = C / 8;
-        for (uint32_t idx = threadIdx.x; idx < c8n * W; idx += 256) {
-            const uint32_t c8 = idx / W, w = idx % W, c0 = c8 * 8;
-            // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
-            // 8 channels starting at c0 are contiguous for x = 8 and x = 16; a trailing block of an
-            // NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
-            const uint32_t blk = c0 / cx;
-            uint32_t bw = C - blk * cx;
-            bw = bw < cx ? bw : cx;
-            const size_t src = (size_t)n * C * H * W + (size_t)blk * cx * H * W + ((size_t)h * W + w) * bw + c0 % cx;
-            v2i v = *(const v2i *)(in + src);
-            v ^= (v2i){(int)0x80808080, (int)0x80808080};
-            *(v2i *)(row + (size_t)(w + pl) * ICp + c0) = v;
-        }
-    }
-    __syncthreads();
-    int8_t *dst = out + (size_t)blockIdx.x * row_bytes;
-    for (uint32_t o = threadIdx.x * 16; o < row_bytes; o += 256 * 16) {
-        *(v4i *)(dst + o) = *(const v4i *)(row + o);
-    }
-}
-
-// the same without LDS, for rows too wide to stage: one thread per 8 output bytes
-__global__ __launch_bounds__(256) void conv_pad_wide_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C,
-    uint32_t H, uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp,
-    int8_t *__restrict__ out)
-{
-    const uint32_t c8n = ICp / 8;
-    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t total = (uint64_t)N * Hp * Wp * c8n;
-    if (id >= total) {
+    const uint32_t planes = ICp / 16;
+    const uint32_t rows = N * planes * Hp;
+    const uint32_t row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (row >= rows) {
         return;
     }
-    const uint32_t c8 = (uint32_t)(id % c8n);
-    uint64_t p = id / c8n;
-    const uint32_t wp = (uint32_t)(p % Wp);
-    p /= Wp;
-    const uint32_t hp = (uint32_t)(p % Hp);
-    const uint32_t n = (uint32_t)(p / Hp);
-    v2i v = {0, 0};
-    const uint32_t c0 = c8 * 8;
-    if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W && c0 < C) {
-        const uint32_t h = hp - pt, w = wp - pl;
+    const uint32_t hp = row % Hp, c16 = (row / Hp) % planes, n = row / (Hp * planes);
+    const bool inside = hp >= pt && hp < pt + H;
+    const uint32_t h = hp - pt;
+    // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
+    // 8 channels starting at a multiple of 8 are contiguous for x = 8 and x = 16; a trailing block of
+    // an NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
+    size_t src[2];
+    uint32_t bw[2];
+    bool have[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const uint32_t c0 = c16 * 16 + half * 8;
+        have[half] = inside && c0 < C;
         const uint32_t blk = c0 / cx;
-        uint32_t bw = C - blk * cx;
-        bw = bw < cx ? bw : cx;
-        const size_t src = (size_t)n * C * H * W + (size_t)blk * cx * H * W + ((size_t)h * W + w) * bw + c0 % cx;
-        v = *(const v2i *)(in + src);
-        v ^= (v2i){(int)0x80808080, (int)0x80808080};
+        uint32_t w_ = (have[half] ? C - blk * cx : cx);
+        bw[half] = w_ < cx ? w_ : cx;
+        src[half] = (size_t)n * C * H * W + (size_t)blk * cx * H * W + (size_t)h * W * bw[half] + c0 % cx;
     }
-    *(v2i *)(out + id * 8) = v;
+    int8_t *dst = out + (size_t)row * Wp * 16;
+    for (uint32_t wp = threadIdx.x & 63; wp < Wp; wp += 64) {
+        v2i lo = {0, 0}, hi = {0, 0};
+        if (wp >= pl && wp < pl + W) {
+            const uint32_t w = wp - pl;
+            if (have[0]) {
+                lo = *(const v2i *)(in + src[0] + (size_t)w * bw[0]);
+                lo ^= (v2i){(int)0x80808080, (int)0x80808080};
+            }
+            if (have[1]) {
+                hi = *(const v2i *)(in + src[1] + (size_t)w * bw[1]);
+                hi ^= (v2i){(int)0x80808080, (int)0x80808080};
+            }
+        }
+        *(v4i *)(dst + (size_t)wp * 16) = (v4i){lo.x, lo.y, hi.x, hi.y};
+    }
 }
 
 hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
     uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st)
 {
     const uint32_t Hp = H + pt + pb, Wp = W + pl + pr, ICp = align_up(C, 16);
-    const uint64_t total = (uint64_t)N * Hp * Wp * (ICp / 8);
-    if (total == 0) {
+    const uint64_t rows = (uint64_t)N * (ICp / 16) * Hp;
+    if (rows == 0 || Wp == 0) {
         return hipSuccess;
     }
-    const uint32_t row_bytes = Wp * ICp;
-    if (row_bytes <= 65536 && (((uintptr_t)out & 15) == 0)) {
-        hipLaunchKernelGGL(conv_pad_kernel, dim3(N * Hp), dim3(256), row_bytes, st, in, N, C, H, W, cx, pt, pl, Hp, Wp, ICp,
-            out);
-    } else {
-        hipLaunchKernelGGL(conv_pad_wide_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, in, N, C, H, W,
-            cx, pt, pl, Hp, Wp, ICp, out);
+    if (rows > 0xffffffffull) {
+        return hipErrorInvalidValue;
     }
+    hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)((rows + 3) / 4)), dim3(256), 0, st, in, N, C, H, W, cx, pt, pl, Hp,
+        Wp, ICp, out);
     return hipGetLastError();
 }
 

@@ -740,10 +740,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             row = row < a.M ? row : a.M - 1;
             if (CONV) {
                 // implicit GEMM: row = output pixel; its receptive field starts at this offset of the
-                // padded, channel-innermost s8 image; the tap / channel-chunk offset comes per K tile
+                // padded s8 image (planes of 16 channels); the tap / channel-plane offset comes per K tile
                 const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
                 const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
-                off[q] = ((img * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * a.conv.ICp;
+                off[q] = ((img * (a.conv.ICp / 16) * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
             } else {
                 off[q] = row * a.lda + g * 16;
             }
@@ -786,7 +786,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         cv_kw = tap % a.conv.fw;
     }
 #define BG_CV_OFF()                                                                                            \
-    ((cv_kh < a.conv.fh) ? (size_t)((cv_kh * a.conv.dh * a.conv.Wp + cv_kw * a.conv.dw) * a.conv.ICp + cv_c16 * 16) \
+    ((cv_kh < a.conv.fh) ? (size_t)(((cv_c16 * a.conv.Hp + cv_kh * a.conv.dh) * a.conv.Wp + cv_kw * a.conv.dw) * 16) \
                          : (size_t)0)
 #define BG_CV_ADVANCE()                                      \
     {                                                        \
@@ -1002,6 +1002,117 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
 }
 
+// Convolution with few output channels (N <= 64) and a filter panel that fits in LDS (K <= 1024).
+// With one 64-channel panel every wave's pixel rows are its own, so staging A through LDS buys nothing
+// and the shared pipeline pays a barrier per K tile for it. Here the whole packed filter panel is
+// fetched into LDS once per block (K x 64 bytes, fragment order), and after one barrier the four
+// waves run independently: each owns TM x 16 pixels, gathers its A fragments from the padded image
+// straight into registers three K tiles ahead (the compiler tracks those loads), reads the four B
+// fragments of a tile from LDS and issues TM x 4 MFMAs. LDS traffic is a third of the shared
+// pipeline's and there is no barrier inside the K loop.
+template <int TM>
+__global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int P = 3;  // K tiles of A in flight per wave
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t m0 = blockIdx.x * (4 * TM * 16);
+    const uint32_t K = a.K, ksteps = K / 64;
+    const uint32_t nblocks = align_up(a.N, 16) >> 4;
+
+    // the filter panel: fragment (tile t, column block y) at smem + (4 t + y) KiB
+    for (uint32_t f = wave; f < 4 * ksteps; f += 4) {
+        const uint32_t t = f >> 2, y = f & 3;
+        const uint32_t nb = y < nblocks ? y : nblocks - 1;
+        const uint8_t *src = (const uint8_t *)a.Bp + (size_t)nb * 16 * K + (size_t)t * 1024 + lane * 16;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(smem + f * 1024), 16, 0, 0);
+    }
+
+    const uint32_t cpc = a.conv.ICp / 16;  // 16-channel planes of the padded image
+    uint32_t off[TM];
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+        uint32_t row = m0 + (wave * TM + x) * 16 + i;
+        row = row < a.M ? row : a.M - 1;
+        const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
+        const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
+        off[x] = ((img * cpc * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
+    }
+    // this lane's K-group g covers 16-channel chunk 4 * tile + g; its (kh, kw, c16) is stepped in registers
+    uint32_t c16 = g % cpc, kw = (g / cpc) % a.conv.fw, kh = (g / cpc) / a.conv.fw, at = 0;  // at: tile the walk points to
+    auto tap_offset = [&]() -> uint32_t {
+        return (kh < a.conv.fh) ? ((c16 * a.conv.Hp + kh * a.conv.dh) * a.conv.Wp + kw * a.conv.dw) * 16 : 0u;
+    };
+    auto advance = [&]() {
+        if (at + 1 < ksteps) {  // past the last tile the walk stays put: the refetch is never used
+            ++at;
+            c16 += 4;
+#pragma unroll
+            for (int w_ = 0; w_ < 4; ++w_) {
+                const bool wr_ = c16 >= cpc;
+                c16 -= wr_ ? cpc : 0u;
+                kw += wr_ ? 1u : 0u;
+                const bool w2_ = kw >= a.conv.fw;
+                kw = w2_ ? 0u : kw;
+                kh += w2_ ? 1u : 0u;
+            }
+        }
+    };
+
+    v4i fa[P][TM];
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+        const uint32_t o = tap_offset();
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            fa[s][x] = *(const v4i *)(a.A + off[x] + o);
+        }
+        advance();
+    }
+    v4i acc[TM][4];
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < 4; ++y) {
+            acc[x][y] = (v4i){0, 0, 0, 0};
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the panel (and the first A tiles) have landed
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    for (uint32_t t = 0; t < ksteps; t += P) {
+#pragma unroll
+        for (int u = 0; u < P; ++u) {
+            if (t + u < ksteps) {
+                const uint8_t *sB = smem + (size_t)(t + u) * 4096 + lane * 16;
+                v4i fb[4];
+#pragma unroll
+                for (int y = 0; y < 4; ++y) {
+                    fb[y] = *(const v4i *)(sB + y * 1024);
+                }
+#pragma unroll
+                for (int x = 0; x < TM; ++x) {
+#pragma unroll
+                    for (int y = 0; y < 4; ++y) {
+                        acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[u][x], acc[x][y], 0, 0, 0);
+                    }
+                }
+                const uint32_t o = tap_offset();
+#pragma unroll
+                for (int x = 0; x < TM; ++x) {
+                    fa[u][x] = *(const v4i *)(a.A + off[x] + o);
+                }
+                advance();
+            }
+        }
+    }
+    epilogue_panel<4, 1, TM, 4, true>(a, acc, nullptr, lane, wave, m0, 0u, 0);
+}
+
 // Skinny kernel for few rows (FullyConnected at small batch: M <= 64 per block, any N, K % 64 == 0).
 // The weight panel is the traffic, so a block owns ONE 16-column panel of B for up to 64 rows of A and
 // its 8 waves split K between them: each wave streams its K range straight from global memory / L2 into
@@ -1120,11 +1231,41 @@ static hipError_t launch_tiled(const GemmArgs &a, hipStream_t st)
     return hipGetLastError();
 }
 
+static int g_conv_panel = 4;  // test hook: 0 = shared pipeline only, 2 / 4 = pixel blocks per wave of the panel kernel
+
+void conv_force_panel(int v)
+{
+    g_conv_panel = v;
+}
+
 // Implicit-GEMM convolution: same pipeline, A rows are output pixels gathered from the padded image.
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
 {
     if (a.M == 0 || a.N == 0) {
         return hipSuccess;
+    }
+    if (a.N <= 64 && a.K % 64 == 0 && a.K <= 1024 && g_conv_panel) {
+        // one filter panel, small enough to sit in LDS: no barrier in the K loop (see the kernel)
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)conv_u8s8_panel_kernel<2>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+            if (e == hipSuccess) {
+                e = hipFuncSetAttribute((const void *)conv_u8s8_panel_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                    65536);
+            }
+            if (e != hipSuccess) {
+                return e;
+            }
+            attr_set = true;
+        }
+        const uint32_t lds = a.K * 64;
+        if (g_conv_panel == 2) {
+            hipLaunchKernelGGL(conv_u8s8_panel_kernel<2>, dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+        } else {
+            hipLaunchKernelGGL(conv_u8s8_panel_kernel<4>, dim3((a.M + 255) / 256), dim3(256), lds, st, a);
+        }
+        return hipGetLastError();
     }
     if (a.N <= 64) {
         // Few output channels: nowhere near MFMA-bound, the time is load latency, so what matters is

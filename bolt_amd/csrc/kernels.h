@@ -35,7 +35,7 @@ hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const i
 
 // ---- GEMM ---------------------------------------------------------------------------------------
 // Geometry of an implicit-GEMM convolution (GemmArgs::conv), all in elements / bytes of the padded,
-// channel-innermost s8 image [n][Hp][Wp][ICp] that conv_pad produces.
+// s8 image in planes of 16 channels, [n][ICp/16][Hp][Wp][16], that conv_pad produces.
 struct ConvGeom {
     uint32_t OHW, OW;          // output pixels per image, output width
     uint32_t sh, sw;           // strides
@@ -67,6 +67,7 @@ struct GemmArgs {
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
 // A = padded s8 image, M = n * OH * OW output pixels, N = output channels, K = fh * fw * ICp
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
+void conv_force_panel(int v);  // 0: shared-pipeline kernel only; 2 / 4: panel kernel with 32 / 64 pixels per wave
 // tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
 void gemm_force_tile(int tile);
 
