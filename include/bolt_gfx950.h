@@ -39,7 +39,9 @@ const char *bolt_gfx950_last_error(void);
  * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 7 / 10 / 11 the LDS-DMA
  * kernels (256x256 fragment-prefetch, 128x128 fragment-prefetch, 256x256 ping-pong; need
  * K % 64 == 0), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
- * the general kernel. Every variant returns the same bytes. */
+ * the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
+ * K <= 1024 uses: 4 (default) / 2 the filter-panel-in-LDS kernel with 64 / 32 pixels per wave, 0 the
+ * shared-pipeline kernel. Every variant returns the same bytes. */
 EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);

@@ -61,6 +61,30 @@ def test_conv_int8(torch_mod, oracle, co, device_mode, case, relu):
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (case, odt, out_c)
 
 
+@pytest.mark.parametrize("panel", [0, 2, 4])
+def test_conv_int8_every_kernel(torch_mod, oracle, co, panel):
+    """Convolutions with up to 64 output channels and K <= 1024 have three kernels to choose from: the shared
+    LDS pipeline (0) and the filter-panel kernel with 32 (2) or 64 (4) pixels per wave. Each is forced in turn
+    on shapes with ragged pixel counts, channel tails, strides and a 5 x 5 filter."""
+    L = capi.lib()
+    try:
+        capi.check(L.bolt_gfx950_set_option(b"conv_panel", panel), "set_option")
+        for case in [(2, 24, 6, 5, 24, 5, 5, 1, 2), (3, 16, 10, 9, 40, 3, 3, 1, 1), (1, 64, 56, 56, 64, 3, 3, 1, 1),
+                     (2, 8, 9, 7, 8, 3, 3, 2, 1), (5, 32, 13, 13, 64, 1, 1, 1, 0)]:
+            print("conv kernel", panel, case, flush=True)
+            n, ic, ih, iw, oc, fh, fw, stride, pad = case
+            xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, sum(case) + panel)
+            for odt in (DT_U8_Q, DT_F32, DT_I32):
+                d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, True, odt, 16)
+                want, ws = co.conv(d, xq, W, bias, [sI, -1.0, sF])
+                sc = [sI, -1.0, sF]
+                got = run_conv(torch_mod, True, xq, DF_NCHWC8, W, bias, sc, case, True, odt, DF_NCHWC16)
+                assert np.array_equal(np.array(sc, np.float32), ws), (odt, sc, ws)
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (panel, case, odt)
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"conv_panel", 4), "set_option")
+
+
 def test_conv_int8_nchwc16_input_and_eltwise(torch_mod, oracle, co):
     case = (2, 32, 7, 6, 48, 3, 3, 1, 1)
     n, ic, ih, iw, oc, fh, fw, stride, pad = case
