@@ -216,11 +216,114 @@ hipError_t launch_gemv_s8u8(const GemvArgs &a, hipStream_t st)
     return launch_s8u8<1>(a, st);
 }
 
+__device__ __forceinline__ void gemv_u8s8_store(void *y, uint32_t m, int acc, const Epilogue &epi)
+{
+    switch (epi.mode) {
+        case EPI_I32:
+            ((int32_t *)y)[m] = acc;
+            break;
+        case EPI_F32:
+            ((float *)y)[m] = (float)acc * epi_factor(epi);
+            break;
+        case EPI_U8:
+            ((uint8_t *)y)[m] = (uint8_t)epi_u8(acc, epi_factor(epi));
+            break;
+        default:
+            break;
+    }
+}
+
+// Row-major u8 matrix [M][lda], rows and x 16-byte aligned: one wave per row, 16 bytes per lane and
+// step, (a ^ 0x80) as s8 against x with v_dot4; the K tail (K % 16) byte by byte.
+__global__ __launch_bounds__(256) void gemv_u8s8_rows_kernel(const uint8_t *__restrict__ A, uint32_t lda,
+    const int8_t *__restrict__ x, uint32_t K, uint32_t M, void *__restrict__ y, Epilogue epi)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (m >= M) {
+        return;
+    }
+    const uint8_t *row = A + (size_t)m * lda;
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+    int acc = 0;
+    const uint32_t K16 = K & ~15u;
+    for (uint32_t k = lane * 16; k < K16; k += 1024) {
+        v4i a = __builtin_nontemporal_load((const v4i *)(row + k));
+        const v4i xv = *(const v4i *)(x + k);
+        a ^= flip;
+        acc = __builtin_amdgcn_sdot4(a.x, xv.x, acc, false);
+        acc = __builtin_amdgcn_sdot4(a.y, xv.y, acc, false);
+        acc = __builtin_amdgcn_sdot4(a.z, xv.z, acc, false);
+        acc = __builtin_amdgcn_sdot4(a.w, xv.w, acc, false);
+    }
+    if (K16 + lane < K) {
+        acc += ((int)row[K16 + lane] - 128) * (int)x[K16 + lane];
+    }
+    acc = wave_reduce_add(acc);
+    if (lane == 0) {
+        gemv_u8s8_store(y, m, acc, epi);
+    }
+}
+
+// u8 matrix stored [K][ldk] (row k holds all M results' coefficients), 4-byte aligned rows: one lane
+// per 4 consecutive results, a dword per lane and k (256 contiguous bytes per wave), x[k] is wave-uniform.
+// The K range is split over the 4 waves of a block and the partial sums meet in LDS.
+__global__ __launch_bounds__(256) void gemv_u8s8_cols_kernel(const uint8_t *__restrict__ A, uint32_t ldk,
+    const int8_t *__restrict__ x, uint32_t K, uint32_t M, void *__restrict__ y, Epilogue epi)
+{
+    __shared__ int part[4][64][4];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t m = (blockIdx.x * 64 + lane) * 4;
+    int acc[4] = {0, 0, 0, 0};
+    if (m < M) {
+        const uint32_t kper = (K + 3) / 4, k0 = wave * kper, k1 = (k0 + kper < K) ? k0 + kper : K;
+        const bool full = m + 4 <= M;
+        for (uint32_t k = k0; k < k1; ++k) {
+            const uint8_t *p = A + (size_t)k * ldk + m;
+            uint32_t w;
+            if (full) {
+                w = *(const uint32_t *)p;
+            } else {
+                w = 0x80808080u;  // (0x80 - 128) = 0 for the results past M
+                for (uint32_t j = 0; m + j < M; ++j) {
+                    w = (w & ~(0xffu << (8 * j))) | ((uint32_t)p[j] << (8 * j));
+                }
+            }
+            const int xv = x[k];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] += ((int)((w >> (8 * j)) & 0xff) - 128) * xv;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        part[wave][lane][j] = acc[j];
+    }
+    __syncthreads();
+    if (wave == 0 && m < M) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (m + j < M) {
+                gemv_u8s8_store(y, m + j, part[0][lane][j] + part[1][lane][j] + part[2][lane][j] + part[3][lane][j], epi);
+            }
+        }
+    }
+}
+
 hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const int8_t *x, uint32_t K, uint32_t M,
     void *y, const Epilogue &epi, hipStream_t st)
 {
     if (M == 0) {
         return hipSuccess;
+    }
+    if (sk == 1 && K >= 16 && (lda & 15) == 0 && ((((uintptr_t)A | (uintptr_t)x) & 15) == 0)) {
+        hipLaunchKernelGGL(gemv_u8s8_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, A, lda, x, K, M, y, epi);
+        return hipGetLastError();
+    }
+    if (lda == 1 && M >= 4 && (sk & 3) == 0 && (((uintptr_t)A & 3) == 0)) {
+        hipLaunchKernelGGL(gemv_u8s8_cols_kernel, dim3((M + 255) / 256), dim3(256), 0, st, A, sk, x, K, M, y, epi);
+        return hipGetLastError();
     }
     const uint32_t blocks = (M + 3) / 4;
     hipLaunchKernelGGL((gemv_u8s8_kernel<1>), dim3(blocks), dim3(256), 0, st, A, lda, sk, x, K, M, y, epi);

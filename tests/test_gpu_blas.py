@@ -297,7 +297,9 @@ def test_mvm_decode_shape_and_device_pack(torch_mod, oracle):
 @pytest.mark.parametrize("device_mode", [False, True])
 def test_mvm_u8_matrix_s8_vector(torch_mod, oracle, device_mode):
     rng = np.random.default_rng(9)
-    for M, K in itertools.product([1, 3, 4, 5, 8, 9, 17, 40], [1, 15, 16, 17, 63, 64, 65, 300]):
+    # includes shapes that take the vectorised kernels (rows: K % 16 == 0 rows, 16-byte aligned; K-major: M % 4 == 0)
+    for M, K in list(itertools.product([1, 3, 4, 5, 8, 9, 17, 40], [1, 15, 16, 17, 63, 64, 65, 300])) + [
+            (300, 512), (260, 1040), (1028, 96), (2048, 2048), (257, 4096)]:
         A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
         x = rng.integers(-127, 128, size=K, dtype=np.int8)
         yin = rng.integers(-500, 500, size=M, dtype=np.int32)
