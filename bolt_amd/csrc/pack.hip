@@ -57,8 +57,11 @@ template <int MMM>
 static hipError_t launch_pack(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t K, uint32_t N, int8_t *dst,
     int32_t *comp, hipStream_t st)
 {
-    if (N == 0 || K == 0) {
+    if (N == 0) {
         return hipSuccess;
+    }
+    if (K == 0) {
+        return launch_fill_u32((uint32_t *)comp, N, 0, st);  // an empty sum: the compensation is zero
     }
     const uint32_t Kp = align_up(K, 8), N16 = align_up(N, 16);
     const uint64_t threads = (uint64_t)N16 * (Kp / 8);
