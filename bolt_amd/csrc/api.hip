@@ -2111,7 +2111,7 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
 
     HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
     // x -> u8 (dynamic per-tensor scale), one quantisation shared by Q, K and V
-    HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st));
+    HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st, true));
     HIP_TRY(launch_quantize_f32(hidden, T * H, xq, 1, ws0, 0.0f, nullptr, 0, sc + 0, st));
     HIP_TRY(gemm(xq, L.wqkv, 3 * H, H, sc + 0, L.sqkv, L.bqkv, qkv));
     HIP_TRY(launch_attention_f32(qkv, L.batch, L.seq, H, L.heads, cx, ws1, st));

@@ -115,7 +115,8 @@ hipError_t launch_pack_mvm(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t
 
 // ---- quantize family ----------------------------------------------------------------------------
 // Device scratch word layout used by the two-pass kernels: ws[0] = max bits / max int.
-hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st);
+// folds max |x| into the scratch slots ws; clears them first unless the caller just did
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear = false);
 // Caller's scale = *ds_in (device) if given, else s_in. Dynamic when !mode or that scale <= 0:
 // the scale used is max(caller's, 127 / max|x|) with max|x| taken from ws[0]. The scale used is
 // written to *ds_out (device) when non-null.

@@ -92,9 +92,9 @@ __global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict
     ws_block_fold_max(ws, (int)__float_as_uint(m), red);
 }
 
-hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st)
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear)
 {
-    hipError_t e = launch_fill_u32(ws, kWsWords, 0, st);
+    hipError_t e = ws_is_clear ? hipSuccess : launch_fill_u32(ws, kWsWords, 0, st);
     if (e != hipSuccess || n == 0) {
         return e;
     }
