@@ -57,6 +57,9 @@ EE fail(EE code, const char *what, hipError_t he = hipSuccess)
         }                                               \
     } while (0)
 
+// 1-bit convolution: 1 = int8 matrix-core route (default), 0 = vector-ALU xor / popcount route
+int g_bnn_mfma = 1;
+
 EE ensure_init()
 {
     Ctx &c = ctx();
@@ -305,6 +308,10 @@ EE bolt_gfx950_set_option(const char *name, int value)
     }
     if (strcmp(name, "gemm_tile") == 0) {
         gemm_force_tile(value);
+        return SUCCESS;
+    }
+    if (strcmp(name, "bnn_mfma") == 0) {
+        g_bnn_mfma = value != 0;
         return SUCCESS;
     }
     if (strcmp(name, "conv_panel") == 0) {
@@ -1552,6 +1559,19 @@ EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwi
 }
 
 // ---- 1-bit convolution (compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72) ----------------------
+// Transformed-filter blob: [bit-packed filter, fn * fc * fh * fw / 8 bytes rounded up to 256 (the vector-ALU
+// route)][the same filter expanded to int8 in the GEMM's packed right-hand-side layout, K = fh * fw * fc padded
+// to 64 (the matrix-core route)]
+static size_t bnn_blob_bits_bytes(U32 fn, U32 fc, U32 fh, U32 fw)
+{
+    return ((size_t)fn * fc * fh * fw / 8 + 255) / 256 * 256;
+}
+
+static size_t bnn_blob_bytes(U32 fn, U32 fc, U32 fh, U32 fw)
+{
+    return bnn_blob_bits_bytes(fn, fc, fh, fw) + (size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16);
+}
+
 EE convolution_transform_filter_bytes_bnn_gfx950(TensorDesc filterDesc, U32 *bytes, Arch arch)
 {
     if (!IS_GFX950(arch)) {
@@ -1567,7 +1587,11 @@ EE convolution_transform_filter_bytes_bnn_gfx950(TensorDesc filterDesc, U32 *byt
     if (filterDesc.dt != DT_BIN01 && filterDesc.dt != DT_BIN11) {
         return NOT_SUPPORTED;
     }
-    *bytes = fn * fc * fh * fw / 8;  // same size as the reference's DF_NCHWN16C8 blob
+    const size_t b = bnn_blob_bytes(fn, fc, fh, fw);
+    if (b > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)b;
     return SUCCESS;
 }
 
@@ -1598,23 +1622,33 @@ EE convolution_transform_filter_bnn_gfx950(TensorDesc filterDesc, const void *fi
         return e;
     }
     Ctx &c = ctx();
-    const size_t bytes = (size_t)fn * fc * fh * fw / 8;
+    const size_t bytes = (size_t)fn * fc * fh * fw / 8, bits = bnn_blob_bits_bytes(fn, fc, fh, fw),
+                 total = bnn_blob_bytes(fn, fc, fh, fw);
     const int fmt = (filterDesc.df == DF_NCHWN16C8) ? 1 : 0;
+    const int xnor = (filterDesc.dt == DT_BIN11);
     if (arch == AMD_GFX950) {
         Stage st;
-        void *a = st.get(bytes), *b = st.get(bytes);
+        void *a = st.get(bytes);
+        U8 *b = (U8 *)st.get(total);
         if (!a || !b) {
             return fail(ALLOC_FAILED, "device staging");
         }
         HIP_TRY(hipMemcpyAsync(a, filter, bytes, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemsetAsync(b, 0, bits, c.stream));
         HIP_TRY(launch_bnn_pack_filter((const uint8_t *)a, fmt, fn, fc, fh * fw, (uint32_t *)b, c.stream));
-        HIP_TRY(hipMemcpyAsync(filterTransformed, b, bytes, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(launch_bnn_expand_filter((const uint32_t *)b, fn, fc, fh * fw, xnor, (int8_t *)(b + bits), c.stream));
+        HIP_TRY(hipMemcpyAsync(filterTransformed, b, total, hipMemcpyDeviceToHost, c.stream));
         HIP_TRY(hipStreamSynchronize(c.stream));
     } else {
-        if (!aligned4(filterTransformed)) {
-            return fail(NOT_SUPPORTED, "device filterTransformed must be 4-byte aligned");
+        if (((uintptr_t)filterTransformed & 15) != 0) {
+            return fail(NOT_SUPPORTED, "device filterTransformed must be 16-byte aligned");
         }
-        HIP_TRY(launch_bnn_pack_filter((const uint8_t *)filter, fmt, fn, fc, fh * fw, (uint32_t *)filterTransformed, c.stream));
+        U8 *b = (U8 *)filterTransformed;
+        if (bits > bytes / 4 * 4) {  // the padding behind the bits, so that equal filters give equal blobs
+            HIP_TRY(launch_fill_u32((uint32_t *)(b + bytes / 4 * 4), (U32)((bits - bytes / 4 * 4) / 4), 0, c.stream));
+        }
+        HIP_TRY(launch_bnn_pack_filter((const uint8_t *)filter, fmt, fn, fc, fh * fw, (uint32_t *)b, c.stream));
+        HIP_TRY(launch_bnn_expand_filter((const uint32_t *)b, fn, fc, fh * fw, xnor, (int8_t *)(b + bits), c.stream));
     }
     *ftmDesc = filterDesc;
     ftmDesc->df = DF_NCHWN16C8;  // the tag the operator layer checks; the byte order inside is this library's
@@ -1633,7 +1667,11 @@ EE convolution_infer_forward_tmp_bytes_bnn_gfx950(TensorDesc inputDesc, Convolut
     if (get4d(inputDesc, &n, &ic, &ih, &iw) != SUCCESS) {
         return NOT_MATCH;
     }
-    const size_t b = (size_t)n * (ih + p.pad_top + p.pad_bottom) * (iw + p.pad_left + p.pad_right) * (ic / 8) + 32;
+    const size_t Hp = ih + p.pad_top + p.pad_bottom, Wp = iw + p.pad_left + p.pad_right;
+    // vector-ALU route: the bit-packed padded image. Matrix-core route: the image expanded to one byte per value.
+    const size_t bits = (size_t)n * Hp * Wp * (ic / 8) + 32;
+    const size_t img = (size_t)n * Hp * Wp * ic + 32;
+    const size_t b = std::max(bits, img);
     if (b > 0xffffffffull) {
         return NOT_SUPPORTED;
     }
@@ -1696,7 +1734,7 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     Ctx &c = ctx();
     Stage st;
     const size_t inB = (idt == DT_F32) ? (size_t)n * ic * ih * iw * 4 : (size_t)n * ic * ih * iw / 8;
-    const size_t fB = (size_t)oc * ic * fh * fw / 8;
+    const size_t fB = bnn_blob_bytes(oc, ic, fh, fw);
     const size_t outN = (size_t)n * oc * oh * ow;
     const void *dIn = input, *dF = filter, *dS = scale, *dB = bias;
     void *dT = tmp, *dO = output;
@@ -1719,6 +1757,49 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
         return fail(NOT_SUPPORTED, "device tmp / filter must be 4-byte aligned, output 16-byte aligned");
     }
     const int xnor = (fdt == DT_BIN11);
+    if (g_bnn_mfma && (((uintptr_t)dT | (uintptr_t)dF) & 15) == 0) {
+        // matrix-core route: the image expanded to int8, the filter already expanded in the blob, then the
+        // int8 implicit-GEMM convolution with fma(S, scale, bias) (or the raw sums) as its epilogue
+        int8_t *img = (int8_t *)dT;
+        const int8_t *flt = (const int8_t *)dF + bnn_blob_bits_bytes(oc, ic, fh, fw);
+        HIP_TRY(launch_bnn_expand_input(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left, p.pad_right,
+            xnor ? 0.0f : 0.5f, xnor, img, c.stream));
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = (const uint8_t *)img;
+        g.Bp = flt;
+        g.M = n * oh * ow;
+        g.N = oc;
+        g.K = align_up(fh * fw * ic, 64);
+        g.ob = (const int32_t *)flt;  // ob == comp: no offset, the sums are exact as they are
+        g.comp = (const int32_t *)flt;
+        g.C = dO;
+        g.conv.OHW = oh * ow;
+        g.conv.OW = ow;
+        g.conv.sh = p.stride_h;
+        g.conv.sw = p.stride_w;
+        g.conv.Hp = Hp;
+        g.conv.Wp = Wp;
+        g.conv.ICp = ic;
+        g.conv.fh = fh;
+        g.conv.fw = fw;
+        g.conv.dh = 1;
+        g.conv.dw = 1;
+        g.conv.out_c = 8;
+        if (odt == DT_I32) {
+            g.epi.mode = EPI_I32;
+        } else {
+            g.epi.mode = EPI_F32_CH;
+            g.epi.scaleW = (const float *)dS;
+            g.epi.bias = (const float *)dB;
+        }
+        HIP_TRY(launch_conv_u8s8(g, c.stream));
+        if (arch == AMD_GFX950) {
+            HIP_TRY(hipMemcpyAsync(output, dO, outN * 4, hipMemcpyDeviceToHost, c.stream));
+            HIP_TRY(hipStreamSynchronize(c.stream));
+        }
+        return SUCCESS;
+    }
     HIP_TRY(launch_bnn_pack_input(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left, p.pad_right,
         xnor ? 0.0f : 0.5f, (uint32_t *)dT, c.stream));
     BnnArgs a;

@@ -1,5 +1,6 @@
-// 1-bit (XNOR / DoReFa) convolution on the vector ALU: bit-packed +-1 / {0,1} operands, XOR (or AND)
-// and population count, no matrix cores.
+// 1-bit (XNOR / DoReFa) convolution. Two routes: on the vector ALU with bit-packed +-1 / {0,1}
+// operands, XOR (or AND) and population count; and on the int8 matrix cores with the operands
+// expanded to one byte per value (see "matrix-core route" below).
 // (Bolt: compute/tensor/src/cpu/arm/bnn/convolution_xnor_A76.cpp:17-724, convolution_dorefa_A76.cpp,
 //  naive form compute/tensor/src/cpu/general/convolution.cpp:141-178.)
 //   XNOR   (DT_BIN11): bit 1 = +1, bit 0 = -1, padding = bit 0;  S = fh*fw*ic - 2 * popcount(x ^ w)
@@ -120,6 +121,126 @@ hipError_t launch_bnn_pack_filter(const uint8_t *src, int src_fmt, uint32_t OC, 
     }
     hipLaunchKernelGGL(bnn_pack_filter_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, src, src_fmt, OC, IC,
         fhw, dst);
+    return hipGetLastError();
+}
+
+// ---- matrix-core route ----------------------------------------------------------------------------
+// +-1 (XNOR) and {0, 1} (DoReFa) are int8 values too, and the int8 matrix cores are five times faster
+// than the vector ALU's xor + popcount, so the convolution can run as the int8 implicit GEMM of
+// conv.hip / gemm.hip on operands expanded to one byte per value: S = sum a * w directly, the
+// padding border is -1 (XNOR: a zero bit) or 0 (DoReFa). The expanded image (n * Hp * Wp * ic
+// bytes) and the expanded filter live in tmp; the transformed-filter blob stays bit-packed.
+
+// fp32 NCHWC8 (or bit-packed [n][ic/8][h][w] bytes, MSB = first channel of the 8) -> s8 planes of 16
+// channels [n][ic/16][Hp][Wp][16]. One workgroup per (image, plane, chunk of 1024 padded pixels), one
+// thread per pixel.
+template <int FROM_F32>
+__global__ __launch_bounds__(256) void bnn_expand_input_kernel(const void *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
+    uint32_t W, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, float thr, int zero, int8_t *__restrict__ out)
+{
+    const uint32_t planes = C / 16;
+    const uint32_t c16 = blockIdx.x % planes, n = blockIdx.x / planes;
+    const uint32_t npix = Hp * Wp;
+    uint32_t end = (blockIdx.y + 1) * 1024;
+    end = end < npix ? end : npix;
+    const uint32_t lo = (uint32_t)zero & 0xffu;  // the byte a cleared bit expands to: 0xff (-1) or 0
+    const uint32_t border = lo * 0x01010101u;
+    // a set bit becomes 0x01; a cleared bit 0xff or 0x00: byte = bit ? 1 : lo, four channels at a time
+    int8_t *dst = out + (size_t)blockIdx.x * npix * 16;
+    for (uint32_t pix = blockIdx.y * 1024 + threadIdx.x; pix < end; pix += 256) {
+        const uint32_t hp = pix / Wp, wp = pix % Wp;
+        uint32_t o[4] = {border, border, border, border};
+        if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W) {
+            const size_t hw = (size_t)(hp - pt) * W + (wp - pl);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const uint32_t c8 = c16 * 2 + half;
+                const size_t p = ((size_t)n * (C / 8) + c8) * H * W + hw;
+                uint32_t bits = 0;  // bit 7 - k = channel k of the 8
+                if (FROM_F32) {
+                    const v4f f0 = *(const v4f *)((const float *)in + p * 8), f1 = *(const v4f *)((const float *)in + p * 8 + 4);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        bits |= (f0[k] >= thr) ? (1u << (7 - k)) : 0u;  // common/uni/include/data_type.h:213-221
+                        bits |= (f1[k] >= thr) ? (1u << (3 - k)) : 0u;
+                    }
+                } else {
+                    bits = ((const uint8_t *)in)[p];
+                }
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    uint32_t w4 = 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        w4 |= (((bits >> (7 - (4 * q + k))) & 1u) ? 1u : lo) << (8 * k);
+                    }
+                    o[half * 2 + q] = w4;
+                }
+            }
+        }
+        *(v4i *)(dst + (size_t)pix * 16) = (v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+    }
+}
+
+hipError_t launch_bnn_expand_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, float thr, int xnor, int8_t *out, hipStream_t st)
+{
+    const uint32_t Hp = H + pt + pb, Wp = W + pl + pr;
+    const uint64_t np = (uint64_t)N * (C / 16), npix = (uint64_t)Hp * Wp;
+    if (np == 0 || npix == 0) {
+        return hipSuccess;
+    }
+    if (np > 0x7fffffffull || npix > 0x3fffffffull || (npix + 1023) / 1024 > 65535) {
+        return hipErrorInvalidValue;
+    }
+    const dim3 grid((uint32_t)np, (uint32_t)((npix + 1023) / 1024));
+    const int zero = xnor ? -1 : 0;
+    if (from_f32) {
+        hipLaunchKernelGGL((bnn_expand_input_kernel<1>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, zero, out);
+    } else {
+        hipLaunchKernelGGL((bnn_expand_input_kernel<0>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, zero, out);
+    }
+    return hipGetLastError();
+}
+
+// Transformed filter ([oc/32][tap][ic/32][32] dwords of bits) -> the int8 GEMM's packed right-hand side over
+// K = (tap, c), K padded to a multiple of 64 with zeros, N = oc. One thread per 16 output bytes
+// (16 consecutive channels of one tap for one output channel).
+__global__ __launch_bounds__(256) void bnn_expand_filter_kernel(const uint32_t *__restrict__ src, uint32_t OC, uint32_t IC,
+    uint32_t fhw, uint32_t Kp, int zero, int8_t *__restrict__ dst)
+{
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t kb_n = Kp / 16;
+    if (id >= (uint64_t)OC * kb_n) {
+        return;
+    }
+    const uint32_t kb = (uint32_t)(id % kb_n), n = (uint32_t)(id / kb_n);
+    const uint32_t k0 = kb * 16;
+    uint32_t o[4] = {0, 0, 0, 0};
+    if (k0 < fhw * IC) {
+        const uint32_t tap = k0 / IC, c0 = k0 % IC, cw = IC / 32;
+        const uint32_t word = src[(((size_t)(n / 32) * fhw + tap) * cw + c0 / 32) * 32 + n % 32];
+        const uint32_t lo = (uint32_t)zero & 0xffu;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const uint32_t c = (c0 % 32) + q;                       // channel within the dword
+            const uint32_t bit = (word >> (8 * (c / 8) + 7 - (c % 8))) & 1u;
+            o[q / 4] |= (bit ? 1u : lo) << (8 * (q & 3));
+        }
+    }
+    *(v4i *)(dst + mmm_packed_offset(n, k0, Kp)) = (v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+}
+
+hipError_t launch_bnn_expand_filter(const uint32_t *src, uint32_t OC, uint32_t IC, uint32_t fhw, int xnor, int8_t *dst,
+    hipStream_t st)
+{
+    const uint32_t Kp = align_up(fhw * IC, 64);
+    const uint64_t total = (uint64_t)OC * (Kp / 16);
+    if (total == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(bnn_expand_filter_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, src, OC, IC, fhw, Kp,
+        xnor ? -1 : 0, dst);
     return hipGetLastError();
 }
 

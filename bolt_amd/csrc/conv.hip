@@ -22,22 +22,18 @@
 
 namespace bg {
 
-// One wave per row (n, 16-channel plane, hp) of the padded image, one lane per pixel: a lane reads the
-// pixel's 16 (or 8) channels from the NCHWC8 / NCHWC16 input -- consecutive lanes read consecutive
-// pixels, 8 or 16 contiguous bytes each -- re-biases them to s8 and writes 16 contiguous bytes. Border
-// pixels and the channel tail are zero. The row decomposition is wave-uniform (scalar arithmetic).
+// One workgroup per (image, 16-channel plane, chunk of 1024 padded pixels), one thread per pixel: a thread
+// reads the pixel's 16 (or 8) channels from the NCHWC8 / NCHWC16 input -- consecutive threads read
+// consecutive pixels, 8 or 16 contiguous bytes each -- re-biases them to s8 and writes 16 contiguous
+// bytes. Border pixels and the channel tail are zero.
 __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
     uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out)
 {
     const uint32_t planes = ICp / 16;
-    const uint32_t rows = N * planes * Hp;
-    const uint32_t row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (row >= rows) {
-        return;
-    }
-    const uint32_t hp = row % Hp, c16 = (row / Hp) % planes, n = row / (Hp * planes);
-    const bool inside = hp >= pt && hp < pt + H;
-    const uint32_t h = hp - pt;
+    const uint32_t c16 = blockIdx.x % planes, n = blockIdx.x / planes;
+    const uint32_t npix = Hp * Wp;
+    uint32_t end = (blockIdx.y + 1) * 1024;
+    end = end < npix ? end : npix;
     // NCHWCx element (n, c, h, w): (((n * C/x + c/x) * H + h) * W + w) * x + c % x. C % 8 == 0, so the
     // 8 channels starting at a multiple of 8 are contiguous for x = 8 and x = 16; a trailing block of
     // an NCHWC16 tensor with C % 16 == 8 is 8 wide (transform_functions_int8.h:208-222).
@@ -47,27 +43,28 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         const uint32_t c0 = c16 * 16 + half * 8;
-        have[half] = inside && c0 < C;
+        have[half] = c0 < C;
         const uint32_t blk = c0 / cx;
         uint32_t w_ = (have[half] ? C - blk * cx : cx);
         bw[half] = w_ < cx ? w_ : cx;
-        src[half] = (size_t)n * C * H * W + (size_t)blk * cx * H * W + (size_t)h * W * bw[half] + c0 % cx;
+        src[half] = (size_t)n * C * H * W + (size_t)blk * cx * H * W + c0 % cx;
     }
-    int8_t *dst = out + (size_t)row * Wp * 16;
-    for (uint32_t wp = threadIdx.x & 63; wp < Wp; wp += 64) {
+    int8_t *dst = out + (size_t)blockIdx.x * npix * 16;
+    for (uint32_t pix = blockIdx.y * 1024 + threadIdx.x; pix < end; pix += 256) {
+        const uint32_t hp = pix / Wp, wp = pix % Wp;
         v2i lo = {0, 0}, hi = {0, 0};
-        if (wp >= pl && wp < pl + W) {
-            const uint32_t w = wp - pl;
+        if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W) {
+            const size_t p = (size_t)(hp - pt) * W + (wp - pl);
             if (have[0]) {
-                lo = *(const v2i *)(in + src[0] + (size_t)w * bw[0]);
+                lo = *(const v2i *)(in + src[0] + p * bw[0]);
                 lo ^= (v2i){(int)0x80808080, (int)0x80808080};
             }
             if (have[1]) {
-                hi = *(const v2i *)(in + src[1] + (size_t)w * bw[1]);
+                hi = *(const v2i *)(in + src[1] + p * bw[1]);
                 hi ^= (v2i){(int)0x80808080, (int)0x80808080};
             }
         }
-        *(v4i *)(dst + (size_t)wp * 16) = (v4i){lo.x, lo.y, hi.x, hi.y};
+        *(v4i *)(dst + (size_t)pix * 16) = (v4i){lo.x, lo.y, hi.x, hi.y};
     }
 }
 
@@ -75,15 +72,15 @@ hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H
     uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st)
 {
     const uint32_t Hp = H + pt + pb, Wp = W + pl + pr, ICp = align_up(C, 16);
-    const uint64_t rows = (uint64_t)N * (ICp / 16) * Hp;
-    if (rows == 0 || Wp == 0) {
+    const uint64_t np = (uint64_t)N * (ICp / 16), npix = (uint64_t)Hp * Wp;
+    if (np == 0 || npix == 0) {
         return hipSuccess;
     }
-    if (rows > 0xffffffffull) {
+    if (np > 0x7fffffffull || npix > 0x3fffffffull || (npix + 1023) / 1024 > 65535) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)((rows + 3) / 4)), dim3(256), 0, st, in, N, C, H, W, cx, pt, pl, Hp,
-        Wp, ICp, out);
+    hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)np, (uint32_t)((npix + 1023) / 1024)), dim3(256), 0, st, in, N, C, H, W,
+        cx, pt, pl, Hp, Wp, ICp, out);
     return hipGetLastError();
 }
 

@@ -197,7 +197,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     } else if (MODE == EPI_F32 || MODE == EPI_U8) {
         factor = epi_factor(a.epi);
     } else if (MODE == EPI_F32_CH) {
-        sI = *a.epi.scaleI;
+        sI = CONV ? 1.0f : *a.epi.scaleI;
     }
 
     uint32_t base[TN][4];
@@ -213,9 +213,15 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             qs[y][c] = 1.0f;
             bs[y][c] = 0.0f;
             if (MODE == EPI_F32_CH && ok) {
-                const float s = sI * a.epi.scaleW[n + c];
-                qs[y][c] = 1.0f / s;
-                bs[y][c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
+                if (CONV) {
+                    // 1-bit convolution on the matrix cores: fma(S, scale[oc], bias[oc]), scale used as it is
+                    qs[y][c] = a.epi.scaleW[n + c];
+                    bs[y][c] = a.epi.bias[n + c];
+                } else {
+                    const float s = sI * a.epi.scaleW[n + c];
+                    qs[y][c] = 1.0f / s;
+                    bs[y][c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
+                }
             }
         }
         cblk_off[y] = 0;
@@ -335,6 +341,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                                 f[c] = 0.0f;
                             }
                         }
+                    } else if (CONV) {
+                        f[c] = __builtin_fmaf((float)t[c], qs[y][c], bs[y][c]);  // vfmaq in the reference's 1-bit kernels
                     } else {
                         f[c] = (float)t[c] * qs[y][c];
                         if (a.epi.bias) {
@@ -507,6 +515,8 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
             epilogue_mode<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else if (a.epi.mode == EPI_U8) {
             epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+        } else if (a.epi.mode == EPI_F32_CH) {
+            epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else {
             epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         }
@@ -776,7 +786,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 // a table in memory would put a vector load, and with it a wait on every tile fetch in flight,
 // into each step. Chunks past the last tap (K padded to 64) read the pixel base; their weights are 0.
 #define BG_AOFF(tile) ((size_t)(tile)*64)
-    static_assert(!CONV || PIPE == 1, "the convolution walk is wired into the fragment-prefetch loop");
+    static_assert(!CONV || PIPE == 1 || PIPE == 2, "the convolution walk is wired into the fragment-prefetch and ping-pong loops");
     uint32_t cv_c16 = 0, cv_kw = 0, cv_kh = 0;
     const uint32_t cv_cpc = CONV ? a.conv.ICp / 16 : 1;
     if (CONV) {
@@ -858,6 +868,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         static_assert(STAGES >= 3, "ping-pong needs at least 3 stages");
         v4i fa[TM], fb[TN];
         const bool late = wave >= 4;
+        size_t pp_aoff = CONV ? BG_CV_OFF() : 0;  // convolution: offset of the next tile to request (the walk is one ahead)
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));  // tile 0 landed
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -869,7 +880,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             // ---- memory phase
             __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * T::kLoads));  // my share of tile t+1 landed
             asm volatile("" ::: "memory");
-            BG_ISSUE(t + (STAGES - 1), BG_CLAMP(t + (STAGES - 1)), BG_AOFF(BG_CLAMP(t + (STAGES - 1))));
+            BG_ISSUE(t + (STAGES - 1), BG_CLAMP(t + (STAGES - 1)), (CONV ? pp_aoff : BG_AOFF(BG_CLAMP(t + (STAGES - 1)))));
+            if (CONV) {
+                if (t + STAGES < ksteps) {
+                    BG_CV_ADVANCE();
+                }
+                pp_aoff = BG_CV_OFF();
+            }
             {
                 const uint8_t *sA_ = smem + (t % STAGES) * T::kStageBytes;
                 const uint8_t *sB_ = sA_ + T::kAFrags * 1024;
@@ -883,9 +900,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): fragments in registers before the matrix phase
+            if (!CONV) {  // a convolution's image is already s8
 #pragma unroll
-            for (int x = 0; x < TM; ++x) {
-                fa[x] ^= flip;
+                for (int x = 0; x < TM; ++x) {
+                    fa[x] ^= flip;
+                }
             }
             __builtin_amdgcn_sched_barrier(0);  // the re-bias belongs to the memory phase
             asm volatile("" ::: "memory");
@@ -1277,6 +1296,9 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<4, 1, 2, 4, 4, true, true>(a, st);
         }
         return launch_dma<4, 1, 4, 4, 4, true, true>(a, st);
+    }
+    if (a.N >= 256 && (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256) >= 128) {
+        return launch_dma<2, 4, 8, 4, 4, 2, true>(a, st);     // 256 pixels x 256 channels, ping-pong K loop
     }
     return launch_dma<2, 2, 8, 4, 4, true, true>(a, st);      // 256 pixels x 128 channels
 }

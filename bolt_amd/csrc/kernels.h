@@ -95,6 +95,11 @@ hipError_t launch_bnn_pack_input(const void *in, int from_f32, uint32_t N, uint3
 hipError_t launch_bnn_pack_filter(const uint8_t *src, int src_fmt, uint32_t OC, uint32_t IC, uint32_t fhw, uint32_t *dst,
     hipStream_t st);
 hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st);
+// matrix-core route: operands expanded to int8 (+1 / -1 or 1 / 0), image in planes of 16 channels like conv_pad's
+hipError_t launch_bnn_expand_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
+    uint32_t pb, uint32_t pl, uint32_t pr, float thr, int xnor, int8_t *out, hipStream_t st);
+hipError_t launch_bnn_expand_filter(const uint32_t *src, uint32_t OC, uint32_t IC, uint32_t fhw, int xnor, int8_t *dst,
+    hipStream_t st);
 
 // ---- fp32 neighbours of the int8 GEMMs in an encoder layer (encoder.hip) --------------------------
 // Each takes an optional `ws` (kWsWords scratch words, zeroed by the caller) into which max|out| is folded.

@@ -67,11 +67,21 @@ SHAPES = [
 ]
 
 
+@pytest.fixture(params=[1, 0], ids=["matrix_cores", "vector_alu"])
+def route(request):
+    """Both routes of the 1-bit convolution: int8 matrix cores on expanded operands (default) and
+    xor / popcount on the vector ALU."""
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", request.param), "set_option")
+    yield request.param
+    capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", 1), "set_option")
+
+
 @pytest.mark.parametrize("device_mode", [False, True])
 @pytest.mark.parametrize("xnor", [True, False])
 @pytest.mark.parametrize("shape", SHAPES)
-def test_bnn_conv(torch_mod, co, device_mode, xnor, shape):
-    print("bnn", device_mode, xnor, shape, flush=True)
+def test_bnn_conv(torch_mod, co, route, device_mode, xnor, shape):
+    print("bnn", route, device_mode, xnor, shape, flush=True)
     torch = torch_mod
     n, ic, ih, iw, oc, fh, fw, stride, pad = shape
     fdt = DT_BIN11 if xnor else DT_BIN01
@@ -103,7 +113,8 @@ def test_bnn_errors(torch_mod):
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(fd, capi.C.byref(b), 0) == capi.NOT_SUPPORTED
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(fd, None, capi.AMD_GFX950) == capi.NULL_POINTER
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(fd, capi.C.byref(b), capi.AMD_GFX950) == 0
-    assert b.value == 32 * 32 * 9 // 8
+    # the bit-packed filter (the reference's size, rounded up to 256) + its int8 expansion (K = 288 -> 320, N = 32)
+    assert b.value == (32 * 32 * 9 // 8 + 255) // 256 * 256 + 320 * 32
     bad = capi.tensor4df(capi.DT_I8, DF_NCHW, 32, 32, 3, 3)
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(bad, capi.C.byref(b), capi.AMD_GFX950) == capi.NOT_SUPPORTED
     w = np.zeros(48 * 32 * 9 // 8, np.uint8)
@@ -114,7 +125,7 @@ def test_bnn_errors(torch_mod):
                                                        capi.AMD_GFX950) == capi.NOT_SUPPORTED
 
 
-def test_bnn_config5_single_image(torch_mod, co):
+def test_bnn_config5_single_image(torch_mod, co, route):
     shape = (1, 256, 28, 28, 256, 3, 3, 1, 1)
     n, ic, ih, iw, oc, fh, fw, stride, pad = shape
     x, w, scale, bias = make_case(shape, True, 55)
@@ -129,7 +140,7 @@ def test_bnn_config5_single_image(torch_mod, co):
     assert np.array_equal(got.view(np.int32), want_f.view(np.int32))
 
 
-def test_bnn_config5_full_batch_properties(torch_mod, co):
+def test_bnn_config5_full_batch_properties(torch_mod, co, route):
     """Batch 64 at the full shape: (1) image 9 of the batch equals the same image run alone and the
     oracle; (2) flipping every activation bit negates every XNOR sum whose window has no padding, and
     the sum of a window over an all-(+1) filter equals 2 * popcount(window) - taps * ic; (3) every sum
