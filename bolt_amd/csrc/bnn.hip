@@ -169,16 +169,16 @@ __global__ __launch_bounds__(256) void bnn_expand_input_kernel(const void *__res
                 }
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
-                    uint32_t w4 = 0;
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        w4 |= (((bits >> (7 - (4 * q + k))) & 1u) ? 1u : lo) << (8 * k);
-                    }
-                    o[half * 2 + q] = w4;
+                    // nibble (channels 4q .. 4q+3, first channel in bit 3) -> one byte per channel: copy the
+                    // nibble into every byte, keep bit 3 - k in byte k, turn "non-zero" into 1
+                    const uint32_t nib = (bits >> (4 - 4 * q)) & 0xfu;
+                    uint32_t t = (nib * 0x01010101u) & 0x01020408u;
+                    t = ((t + 0x7f7f7f7fu) >> 7) & 0x01010101u;
+                    o[half * 2 + q] = t | ((t ^ 0x01010101u) * lo);  // set bit -> 1, cleared bit -> lo (0xff or 0)
                 }
             }
         }
-        *(v4i *)(dst + (size_t)pix * 16) = (v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+        __builtin_nontemporal_store((v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]}, (v4i *)(dst + (size_t)pix * 16));
     }
 }
 
