@@ -205,13 +205,19 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         wb = torch.randint(0, 256, (oc * ic * 9 // 8,), dtype=torch.uint8, device=dev, generator=g)
         bblob, bftm = host_conv.bnn_transform_filter(wb, DT_BIN11, DF_NCHWN16C8, oc, ic, 3, 3)
         bs, bb = torch.rand(oc, device=dev, generator=g) + 0.5, torch.randn(oc, device=dev, generator=g) * 0.1
-        btmp = torch.empty(8 << 20, dtype=torch.uint8, device=dev)
+        btmp = torch.empty(host_conv.bnn_tmp_bytes(DT_BIN11, n, ic, ih, iw, oc, 3, 3, 1, 1, xb), dtype=torch.uint8, device=dev)
         bout = torch.empty(n * oc * ih * iw, dtype=torch.float32, device=dev)
-        t = timed(lambda: host_conv.convolution_bnn(xb, DT_BIN11, n, ic, ih, iw, bblob, bftm, oc, 3, 3, 1, 1, bs, bb, DT_F32,
-                                                    tmp=btmp, out=bout), 20)
         macs = float(n) * ih * iw * oc * ic * 9
-        res["bnn_c5_xnor"] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
-                              "gbps": 53061632 / t / 1e6}
+        # default route: operands expanded to int8, int8 matrix cores; the other: xor + popcount on the vector ALU
+        for route, key in ((1, "bnn_c5_xnor"), (0, "bnn_c5_xnor_vector_alu")):
+            capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", route), "set_option")
+            t = timed(lambda: host_conv.convolution_bnn(xb, DT_BIN11, n, ic, ih, iw, bblob, bftm, oc, 3, 3, 1, 1, bs, bb,
+                                                        DT_F32, tmp=btmp, out=bout), 20)
+            res[key] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
+                        "gbps": 53061632 / t / 1e6}
+        capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", 1), "set_option")
+        res["bnn_c5_xnor"]["int8_tops"] = 2 * macs / res["bnn_c5_xnor"]["ms"] / 1e9
+        res["bnn_c5_xnor"]["frac_mfma_peak"] = res["bnn_c5_xnor"]["int8_tops"] / MFMA_PEAK_TOPS
     # -- C4: BERT-base int8 encoder layer, batch 32 x seq 128 (4096 tokens), one C call per layer
     if want("encoder"):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))

@@ -47,6 +47,8 @@ def convolution(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias,
                                                            arch), "conv_tmp_bytes")
     if tmp is None:
         tmp = _empty_like_mode(x, b.value)
+    elif (tmp.numel() if _is_torch(tmp) else tmp.nbytes) < b.value:
+        raise ValueError("tmp holds %d bytes, the convolution needs %d" % (tmp.numel() if _is_torch(tmp) else tmp.nbytes, b.value))
     count = n * oc * oh * ow
     if out is not None:
         pass
@@ -81,6 +83,15 @@ def bnn_transform_filter(filt_bits, fdt, fdf, oc, ic, fh, fw):
     return blob, ftm
 
 
+def bnn_tmp_bytes(idt, n, ic, ih, iw, oc, fh, fw, stride, pad, like):
+    """Bytes of tmp convolution_bnn needs for this shape (`like` selects host or device pointers)."""
+    b = C.c_uint32(0)
+    check(lib().convolution_infer_forward_tmp_bytes_bnn_gfx950(tensor4df(idt, DF_NCHWC8, n, ic, ih, iw),
+                                                               conv_param_spec(oc, fh, fw, stride, pad), C.byref(b),
+                                                               arch_of(like)), "bnn_tmp_bytes")
+    return b.value
+
+
 def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, scale, bias, odt=DT_F32, tmp=None,
                     out=None):
     """x: fp32 NCHWC8 activations (idt = DT_F32) or packed bits (idt = the filter's type); scale / bias fp32 [oc].
@@ -94,6 +105,8 @@ def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, s
     check(lib().convolution_infer_forward_tmp_bytes_bnn_gfx950(idesc, p, C.byref(b), arch), "bnn_tmp_bytes")
     if tmp is None:
         tmp = _empty_like_mode(x, b.value)
+    elif (tmp.numel() if _is_torch(tmp) else tmp.nbytes) < b.value:
+        raise ValueError("tmp holds %d bytes, the convolution needs %d" % (tmp.numel() if _is_torch(tmp) else tmp.nbytes, b.value))
     count = n * oc * oh * ow
     if out is not None:
         pass
