@@ -208,16 +208,17 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         btmp = torch.empty(host_conv.bnn_tmp_bytes(DT_BIN11, n, ic, ih, iw, oc, 3, 3, 1, 1, xb), dtype=torch.uint8, device=dev)
         bout = torch.empty(n * oc * ih * iw, dtype=torch.float32, device=dev)
         macs = float(n) * ih * iw * oc * ic * 9
-        # default route: operands expanded to int8, int8 matrix cores; the other: xor + popcount on the vector ALU
-        for route, key in ((1, "bnn_c5_xnor"), (0, "bnn_c5_xnor_vector_alu")):
+        # default route: operands expanded to E2M1 pairs, fp4 matrix cores; then int8 matrix cores; then xor + popcount
+        # on the vector ALU
+        for route, key in ((2, "bnn_c5_xnor"), (1, "bnn_c5_xnor_int8_matrix_cores"), (0, "bnn_c5_xnor_vector_alu")):
             capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", route), "set_option")
             t = timed(lambda: host_conv.convolution_bnn(xb, DT_BIN11, n, ic, ih, iw, bblob, bftm, oc, 3, 3, 1, 1, bs, bb,
                                                         DT_F32, tmp=btmp, out=bout), 20)
             res[key] = {"ms": t, "binary_tops": 2 * macs / t / 1e9, "algorithmic_bytes": 53061632,
                         "gbps": 53061632 / t / 1e6}
-        capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", 1), "set_option")
-        res["bnn_c5_xnor"]["int8_tops"] = 2 * macs / res["bnn_c5_xnor"]["ms"] / 1e9
-        res["bnn_c5_xnor"]["frac_mfma_peak"] = res["bnn_c5_xnor"]["int8_tops"] / MFMA_PEAK_TOPS
+        capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", 2), "set_option")
+        res["bnn_c5_xnor"]["frac_fp4_mfma_peak"] = res["bnn_c5_xnor"]["binary_tops"] / 10100.0
+        res["bnn_c5_xnor_int8_matrix_cores"]["frac_mfma_peak"] = res["bnn_c5_xnor_int8_matrix_cores"]["binary_tops"] / MFMA_PEAK_TOPS
     # -- C4: BERT-base int8 encoder layer, batch 32 x seq 128 (4096 tokens), one C call per layer
     if want("encoder"):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))

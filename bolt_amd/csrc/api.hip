@@ -57,8 +57,9 @@ EE fail(EE code, const char *what, hipError_t he = hipSuccess)
         }                                               \
     } while (0)
 
-// 1-bit convolution: 1 = int8 matrix-core route (default), 0 = vector-ALU xor / popcount route
-int g_bnn_mfma = 1;
+// 1-bit convolution: 2 = matrix cores with E2M1 operands where the shape has that kernel, else int8 (default);
+// 1 = matrix cores with int8 operands; 0 = vector-ALU xor / popcount route
+int g_bnn_mfma = 2;
 
 EE ensure_init()
 {
@@ -311,7 +312,10 @@ EE bolt_gfx950_set_option(const char *name, int value)
         return SUCCESS;
     }
     if (strcmp(name, "bnn_mfma") == 0) {
-        g_bnn_mfma = value != 0;
+        if (value < 0 || value > 2) {
+            return NOT_MATCH;
+        }
+        g_bnn_mfma = value;
         return SUCCESS;
     }
     if (strcmp(name, "conv_panel") == 0) {
@@ -1567,9 +1571,16 @@ static size_t bnn_blob_bits_bytes(U32 fn, U32 fc, U32 fh, U32 fw)
     return ((size_t)fn * fc * fh * fw / 8 + 255) / 256 * 256;
 }
 
+static size_t bnn_blob_i8_bytes(U32 fn, U32 fc, U32 fh, U32 fw)
+{
+    return ((size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16) + 255) / 256 * 256;
+}
+
+// ... followed by the filter as E2M1 pairs (K bytes = fh * fw * fc / 2 padded to 64) for the fp4 form of that route
 static size_t bnn_blob_bytes(U32 fn, U32 fc, U32 fh, U32 fw)
 {
-    return bnn_blob_bits_bytes(fn, fc, fh, fw) + (size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16);
+    return bnn_blob_bits_bytes(fn, fc, fh, fw) + bnn_blob_i8_bytes(fn, fc, fh, fw) +
+        (size_t)align_up(fh * fw * fc / 2, 64) * align_up(fn, 16);
 }
 
 EE convolution_transform_filter_bytes_bnn_gfx950(TensorDesc filterDesc, U32 *bytes, Arch arch)
@@ -1637,6 +1648,10 @@ EE convolution_transform_filter_bnn_gfx950(TensorDesc filterDesc, const void *fi
         HIP_TRY(hipMemsetAsync(b, 0, bits, c.stream));
         HIP_TRY(launch_bnn_pack_filter((const uint8_t *)a, fmt, fn, fc, fh * fw, (uint32_t *)b, c.stream));
         HIP_TRY(launch_bnn_expand_filter((const uint32_t *)b, fn, fc, fh * fw, xnor, (int8_t *)(b + bits), c.stream));
+        HIP_TRY(hipMemsetAsync(b + bits + (size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16), 0,
+            bnn_blob_i8_bytes(fn, fc, fh, fw) - (size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16), c.stream));
+        HIP_TRY(launch_bnn_expand_filter_fp4((const uint32_t *)b, fn, fc, fh * fw, xnor,
+            b + bits + bnn_blob_i8_bytes(fn, fc, fh, fw), c.stream));
         HIP_TRY(hipMemcpyAsync(filterTransformed, b, total, hipMemcpyDeviceToHost, c.stream));
         HIP_TRY(hipStreamSynchronize(c.stream));
     } else {
@@ -1649,6 +1664,11 @@ EE convolution_transform_filter_bnn_gfx950(TensorDesc filterDesc, const void *fi
         }
         HIP_TRY(launch_bnn_pack_filter((const uint8_t *)filter, fmt, fn, fc, fh * fw, (uint32_t *)b, c.stream));
         HIP_TRY(launch_bnn_expand_filter((const uint32_t *)b, fn, fc, fh * fw, xnor, (int8_t *)(b + bits), c.stream));
+        const size_t i8 = (size_t)align_up(fh * fw * fc, 64) * align_up(fn, 16), i8p = bnn_blob_i8_bytes(fn, fc, fh, fw);
+        if (i8p > i8) {
+            HIP_TRY(launch_fill_u32((uint32_t *)(b + bits + i8), (U32)((i8p - i8) / 4), 0, c.stream));
+        }
+        HIP_TRY(launch_bnn_expand_filter_fp4((const uint32_t *)b, fn, fc, fh * fw, xnor, b + bits + i8p, c.stream));
     }
     *ftmDesc = filterDesc;
     ftmDesc->df = DF_NCHWN16C8;  // the tag the operator layer checks; the byte order inside is this library's
@@ -1758,19 +1778,26 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     }
     const int xnor = (fdt == DT_BIN11);
     if (g_bnn_mfma && (((uintptr_t)dT | (uintptr_t)dF) & 15) == 0) {
-        // matrix-core route: the image expanded to int8, the filter already expanded in the blob, then the
-        // int8 implicit-GEMM convolution with fma(S, scale, bias) (or the raw sums) as its epilogue
+        // matrix-core route: the image expanded to int8 (or E2M1 pairs), the filter already expanded in the blob,
+        // then the implicit-GEMM convolution with fma(S, scale, bias) (or the raw sums) as its epilogue
+        const bool fp4 = g_bnn_mfma == 2 && conv_fp4_ok(n * oh * ow, oc);
         int8_t *img = (int8_t *)dT;
-        const int8_t *flt = (const int8_t *)dF + bnn_blob_bits_bytes(oc, ic, fh, fw);
-        HIP_TRY(launch_bnn_expand_input(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left, p.pad_right,
-            xnor ? 0.0f : 0.5f, xnor, img, c.stream));
+        const int8_t *flt = (const int8_t *)dF + bnn_blob_bits_bytes(oc, ic, fh, fw) + (fp4 ? bnn_blob_i8_bytes(oc, ic, fh, fw) : 0);
+        if (fp4) {
+            HIP_TRY(launch_bnn_expand_input_fp4(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left,
+                p.pad_right, xnor ? 0.0f : 0.5f, xnor, (uint8_t *)img, c.stream));
+        } else {
+            HIP_TRY(launch_bnn_expand_input(dIn, idt == DT_F32, n, ic, ih, iw, p.pad_top, p.pad_bottom, p.pad_left,
+                p.pad_right, xnor ? 0.0f : 0.5f, xnor, img, c.stream));
+        }
         GemmArgs g;
         memset(&g, 0, sizeof(g));
         g.A = (const uint8_t *)img;
         g.Bp = flt;
         g.M = n * oh * ow;
         g.N = oc;
-        g.K = align_up(fh * fw * ic, 64);
+        g.K = fp4 ? align_up(fh * fw * ic / 2, 64) : align_up(fh * fw * ic, 64);  // in operand bytes
+        g.fp4 = fp4 ? 1 : 0;
         g.ob = (const int32_t *)flt;  // ob == comp: no offset, the sums are exact as they are
         g.comp = (const int32_t *)flt;
         g.C = dO;
@@ -1780,7 +1807,7 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
         g.conv.sw = p.stride_w;
         g.conv.Hp = Hp;
         g.conv.Wp = Wp;
-        g.conv.ICp = ic;
+        g.conv.ICp = fp4 ? ic / 2 : ic;  // bytes per pixel
         g.conv.fh = fh;
         g.conv.fw = fw;
         g.conv.dh = 1;

@@ -244,6 +244,127 @@ hipError_t launch_bnn_expand_filter(const uint32_t *src, uint32_t OC, uint32_t I
     return hipGetLastError();
 }
 
+// ---- fp4 variant of the matrix-core route -----------------------------------------------------------
+// +1, -1 and 0 are E2M1 values (0x2, 0xA, 0x0): two channels per byte, 32 channels per 16-byte chunk, and
+// v_mfma_scale_f32_16x16x128_f8f6f4 multiplies twice as many of them per instruction as the int8 form.
+// Channel c of a 32-channel group sits in byte c / 2, low nibble first; image and filter use the same order,
+// which is all a dot product needs.
+
+// 8 bits (bit 7 - k = channel k) -> 8 nibbles of a dword (nibble k = channel k): set bit -> 0x2, cleared -> lo4
+__device__ __forceinline__ uint32_t bnn_bits_to_fp4(uint32_t bits, uint32_t lo4)
+{
+    uint32_t out = 0;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const uint32_t nib = (bits >> (4 - 4 * q)) & 0xfu;       // channels 4q .. 4q+3, first channel in bit 3
+        uint32_t t = (nib * 0x1111u) & 0x1248u;                  // nibble j keeps bit 3 - j
+        t = ((t + 0x7777u) >> 3) & 0x1111u;                      // non-zero -> 1
+        const uint32_t v = (t << 1) | ((t ^ 0x1111u) * lo4);     // 1 -> 0x2, 0 -> lo4
+        out |= v << (16 * q);
+    }
+    return out;
+}
+
+// fp32 NCHWC8 or bit-packed input -> fp4 planes of 32 channels [n][ic/32][Hp][Wp][16 bytes]
+template <int FROM_F32>
+__global__ __launch_bounds__(256) void bnn_expand_input_fp4_kernel(const void *__restrict__ in, uint32_t N, uint32_t C,
+    uint32_t H, uint32_t W, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, float thr, uint32_t lo4,
+    uint8_t *__restrict__ out)
+{
+    const uint32_t planes = C / 32;
+    const uint32_t c32 = blockIdx.x % planes, n = blockIdx.x / planes;
+    const uint32_t npix = Hp * Wp;
+    uint32_t end = (blockIdx.y + 1) * 1024;
+    end = end < npix ? end : npix;
+    const uint32_t border = lo4 * 0x11111111u;
+    uint8_t *dst = out + (size_t)blockIdx.x * npix * 16;
+    for (uint32_t pix = blockIdx.y * 1024 + threadIdx.x; pix < end; pix += 256) {
+        const uint32_t hp = pix / Wp, wp = pix % Wp;
+        uint32_t o[4] = {border, border, border, border};
+        if (hp >= pt && hp < pt + H && wp >= pl && wp < pl + W) {
+            const size_t hw = (size_t)(hp - pt) * W + (wp - pl);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const uint32_t c8 = c32 * 4 + b;
+                const size_t p = ((size_t)n * (C / 8) + c8) * H * W + hw;
+                uint32_t bits = 0;  // bit 7 - k = channel k of the 8
+                if (FROM_F32) {
+                    const v4f f0 = *(const v4f *)((const float *)in + p * 8), f1 = *(const v4f *)((const float *)in + p * 8 + 4);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        bits |= (f0[k] >= thr) ? (1u << (7 - k)) : 0u;  // common/uni/include/data_type.h:213-221
+                        bits |= (f1[k] >= thr) ? (1u << (3 - k)) : 0u;
+                    }
+                } else {
+                    bits = ((const uint8_t *)in)[p];
+                }
+                o[b] = bnn_bits_to_fp4(bits, lo4);
+            }
+        }
+        __builtin_nontemporal_store((v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]}, (v4i *)(dst + (size_t)pix * 16));
+    }
+}
+
+hipError_t launch_bnn_expand_input_fp4(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+    uint32_t pt, uint32_t pb, uint32_t pl, uint32_t pr, float thr, int xnor, uint8_t *out, hipStream_t st)
+{
+    const uint32_t Hp = H + pt + pb, Wp = W + pl + pr;
+    const uint64_t np = (uint64_t)N * (C / 32), npix = (uint64_t)Hp * Wp;
+    if (np == 0 || npix == 0) {
+        return hipSuccess;
+    }
+    if (np > 0x7fffffffull || npix > 0x3fffffffull || (npix + 1023) / 1024 > 65535) {
+        return hipErrorInvalidValue;
+    }
+    const dim3 grid((uint32_t)np, (uint32_t)((npix + 1023) / 1024));
+    const uint32_t lo4 = xnor ? 0xAu : 0x0u;
+    if (from_f32) {
+        hipLaunchKernelGGL((bnn_expand_input_fp4_kernel<1>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, lo4,
+            out);
+    } else {
+        hipLaunchKernelGGL((bnn_expand_input_fp4_kernel<0>), grid, dim3(256), 0, st, in, N, C, H, W, pt, pl, Hp, Wp, thr, lo4,
+            out);
+    }
+    return hipGetLastError();
+}
+
+// Transformed filter bits -> fp4 pairs in the GEMM's packed right-hand-side layout over K bytes = (tap, c / 2),
+// padded to a multiple of 64 bytes with zeros. One thread per source dword (32 channels = 16 bytes).
+__global__ __launch_bounds__(256) void bnn_expand_filter_fp4_kernel(const uint32_t *__restrict__ src, uint32_t OC, uint32_t IC,
+    uint32_t fhw, uint32_t Kp, uint32_t lo4, uint8_t *__restrict__ dst)
+{
+    const uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t kb_n = Kp / 16;
+    if (id >= (uint64_t)OC * kb_n) {
+        return;
+    }
+    const uint32_t kb = (uint32_t)(id % kb_n), n = (uint32_t)(id / kb_n);
+    const uint32_t cw = IC / 32;
+    uint32_t o[4] = {0, 0, 0, 0};
+    if (kb < fhw * cw) {
+        const uint32_t tap = kb / cw, j = kb % cw;
+        const uint32_t word = src[(((size_t)(n / 32) * fhw + tap) * cw + j) * 32 + n % 32];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            o[b] = bnn_bits_to_fp4((word >> (8 * b)) & 0xffu, lo4);
+        }
+    }
+    *(v4i *)(dst + mmm_packed_offset(n, kb * 16, Kp)) = (v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+}
+
+hipError_t launch_bnn_expand_filter_fp4(const uint32_t *src, uint32_t OC, uint32_t IC, uint32_t fhw, int xnor, uint8_t *dst,
+    hipStream_t st)
+{
+    const uint32_t Kp = align_up(fhw * IC / 2, 64);
+    const uint64_t total = (uint64_t)OC * (Kp / 16);
+    if (total == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(bnn_expand_filter_fp4_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, src, OC, IC, fhw,
+        Kp, xnor ? 0xAu : 0x0u, dst);
+    return hipGetLastError();
+}
+
 // One wave: 64 output pixels (lane = pixel) x 32 output channels.
 template <int XNOR>
 __global__ __launch_bounds__(256) void bnn_conv_kernel(BnnArgs a)

@@ -689,7 +689,10 @@ __device__ __forceinline__ constexpr int vmcnt_imm(int n)
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false>
+// FP4 (1-bit convolution only): the operand bytes hold two E2M1 values each (+1 = 0x2, -1 = 0xA, 0 = 0x0) and the
+// products are formed by v_mfma_scale_f32_16x16x128_f8f6f4 -- twice the K per instruction at the same rate, fp32
+// accumulation that is exact for these integers; the accumulators are converted to int32 before the epilogue.
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false, bool FP4 = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
@@ -917,7 +920,16 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
             for (int x = 0; x < TM; ++x) {
 #pragma unroll
                 for (int y = 0; y < TN; ++y) {
-                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[x], acc[x][y], 0, 0, 0);
+                    if constexpr (FP4) {
+                        const v8i b8 = {fb[y].x, fb[y].y, fb[y].z, fb[y].w, 0, 0, 0, 0};
+                        const v8i a8 = {fa[x].x, fa[x].y, fa[x].z, fa[x].w, 0, 0, 0, 0};
+                        const v4f c = __builtin_bit_cast(v4f, acc[x][y]);
+                        // cbsz = blgp = 4: both operands E2M1; block scales 2^0 (E8M0 127)
+                        acc[x][y] = __builtin_bit_cast(v4i,
+                            __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b8, a8, c, 4, 4, 0, 127, 0, 127));
+                    } else {
+                        acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[x], acc[x][y], 0, 0, 0);
+                    }
                 }
             }
             __builtin_amdgcn_s_setprio(0);
@@ -1010,6 +1022,17 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 #undef BG_CV_OFF
 #undef BG_CV_ADVANCE
     asm volatile("" ::"v"(warm));  // keeps the warming loads alive; the value itself is not used
+    if constexpr (FP4) {
+        static_assert(!FP4 || PIPE == 2, "the fp4 product is wired into the ping-pong loop");
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                const v4f c = __builtin_bit_cast(v4f, acc[x][y]);
+                acc[x][y] = (v4i){(int)c.x, (int)c.y, (int)c.z, (int)c.w};  // exact: sums of +-1 and 0/1 products
+            }
+        }
+    }
     if (!CONV) {
         // the matrix epilogue stages results through LDS: every wave's tile fetches have landed (each
         // drained its own above) and every wave has read its last fragments before anyone writes there
@@ -1210,12 +1233,12 @@ __global__ __launch_bounds__(512) void gemm_u8s8_skinny_kernel(GemmArgs a)
     epilogue_panel<1, 1, 4, 1>(a, acc, nullptr, lane, 0u, m0, n0, 0);
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false>
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false, bool FP4 = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     static bool attr_set = false;
-    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV>;
+    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV, FP4>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
         if (e != hipSuccess) {
@@ -1257,6 +1280,12 @@ void conv_force_panel(int v)
     g_conv_panel = v;
 }
 
+// the fp4 product exists in the 256 x 256 ping-pong instantiation only: take it where that kernel is the choice anyway
+bool conv_fp4_ok(uint32_t M, uint32_t N)
+{
+    return N >= 256 && (uint64_t)((M + 255) / 256) * ((N + 255) / 256) >= 128;
+}
+
 // Implicit-GEMM convolution: same pipeline, A rows are output pixels gathered from the padded image.
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
 {
@@ -1296,6 +1325,12 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<4, 1, 2, 4, 4, true, true>(a, st);
         }
         return launch_dma<4, 1, 4, 4, 4, true, true>(a, st);
+    }
+    if (a.fp4) {
+        if (!conv_fp4_ok(a.M, a.N)) {
+            return hipErrorInvalidValue;
+        }
+        return launch_dma<2, 4, 8, 4, 4, 2, true, true>(a, st);
     }
     if (a.N >= 256 && (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256) >= 128) {
         return launch_dma<2, 4, 8, 4, 4, 2, true>(a, st);     // 256 pixels x 256 channels, ping-pong K loop

@@ -61,12 +61,14 @@ struct GemmArgs {
     void *C;             // [M][N] row-major
     int add_cin;         // accumulate into the int32 bits already in C
     int stream_c;        // set by the launcher: write C with the non-temporal hint
+    int fp4;             // convolution only: operand bytes are pairs of E2M1 values (1-bit convolution), K counts bytes
     Epilogue epi;
     ConvGeom conv;       // used by launch_conv_u8s8 only
 };
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
 // A = padded s8 image, M = n * OH * OW output pixels, N = output channels, K = fh * fw * ICp
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
+bool conv_fp4_ok(uint32_t M, uint32_t N);  // whether launch_conv_u8s8 has an fp4 kernel for this shape
 void conv_force_panel(int v);  // 0: shared-pipeline kernel only; 2 / 4: panel kernel with 32 / 64 pixels per wave
 // tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
 void gemm_force_tile(int tile);
@@ -99,6 +101,11 @@ hipError_t launch_bnn_conv(const BnnArgs &a, int xnor, hipStream_t st);
 hipError_t launch_bnn_expand_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
     uint32_t pb, uint32_t pl, uint32_t pr, float thr, int xnor, int8_t *out, hipStream_t st);
 hipError_t launch_bnn_expand_filter(const uint32_t *src, uint32_t OC, uint32_t IC, uint32_t fhw, int xnor, int8_t *dst,
+    hipStream_t st);
+// the same with two E2M1 values per byte: image in planes of 32 channels [n][ic/32][Hp][Wp][16], K counted in bytes
+hipError_t launch_bnn_expand_input_fp4(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+    uint32_t pt, uint32_t pb, uint32_t pl, uint32_t pr, float thr, int xnor, uint8_t *out, hipStream_t st);
+hipError_t launch_bnn_expand_filter_fp4(const uint32_t *src, uint32_t OC, uint32_t IC, uint32_t fhw, int xnor, uint8_t *dst,
     hipStream_t st);
 
 // ---- fp32 neighbours of the int8 GEMMs in an encoder layer (encoder.hip) --------------------------

@@ -41,9 +41,11 @@ const char *bolt_gfx950_last_error(void);
  * K % 64 == 0), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
  * the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
  * K <= 1024 uses: 4 (default) / 2 the filter-panel-in-LDS kernel with 64 / 32 pixels per wave, 0 the
- * shared-pipeline kernel. "bnn_mfma": 1 (default) the 1-bit convolution runs on the int8 matrix cores
- * with its operands expanded to one byte per value, 0 on the vector ALU (xor + popcount). Every
- * variant returns the same bytes. */
+ * shared-pipeline kernel. "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
+ * with its operands expanded to E2M1 pairs (v_mfma_scale_f32_16x16x128_f8f6f4) where the shape has
+ * that kernel (256+ output channels, 128+ tiles of 256 pixels) and as 1 otherwise; 1 on the int8
+ * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount). Every variant
+ * returns the same bytes. */
 EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);
@@ -168,8 +170,8 @@ EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwi
  *            DF_NCHW bit string or the reference's DF_NCHWN16C8 bytes -> blob tagged DF_NCHWN16C8
  *            of the size convolution_transform_filter_bytes_bnn_gfx950 returns: the bit-packed filter
  *            (oc*ic*fh*fw/8 bytes, the reference's size, rounded up to 256; byte order this library's)
- *            followed by the same filter as int8 values in the int8 GEMM's packed layout, which is
- *            what the matrix-core route multiplies with.
+ *            followed by the same filter as int8 values and as E2M1 pairs in the GEMM's packed
+ *            layout, which is what the matrix-core routes multiply with.
  *   input  : DF_NCHWC8, DT_F32 (binarised on the fly: x >= 0 for BIN11, x >= 0.5 for BIN01, the
  *            thresholds of the reference's fp16 packing) or already packed bits of the filter's type,
  *            [n][ic/8][ih][iw] bytes, MSB = first channel of each 8.

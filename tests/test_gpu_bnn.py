@@ -67,10 +67,11 @@ SHAPES = [
 ]
 
 
-@pytest.fixture(params=[1, 0], ids=["matrix_cores", "vector_alu"])
+@pytest.fixture(params=[2, 1, 0], ids=["matrix_cores_fp4", "matrix_cores_int8", "vector_alu"])
 def route(request):
-    """Both routes of the 1-bit convolution: int8 matrix cores on expanded operands (default) and
-    xor / popcount on the vector ALU."""
+    """Every route of the 1-bit convolution: matrix cores on operands expanded to E2M1 pairs (default where
+    the shape has that kernel, as configs[4] does; otherwise it is the int8 form), matrix cores on int8
+    operands, and xor / popcount on the vector ALU."""
     L = capi.lib()
     capi.check(L.bolt_gfx950_set_option(b"bnn_mfma", request.param), "set_option")
     yield request.param
@@ -114,7 +115,8 @@ def test_bnn_errors(torch_mod):
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(fd, None, capi.AMD_GFX950) == capi.NULL_POINTER
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(fd, capi.C.byref(b), capi.AMD_GFX950) == 0
     # the bit-packed filter (the reference's size, rounded up to 256) + its int8 expansion (K = 288 -> 320, N = 32)
-    assert b.value == (32 * 32 * 9 // 8 + 255) // 256 * 256 + 320 * 32
+    # + its E2M1 expansion (K bytes = 144 -> 192)
+    assert b.value == (32 * 32 * 9 // 8 + 255) // 256 * 256 + 320 * 32 + 192 * 32
     bad = capi.tensor4df(capi.DT_I8, DF_NCHW, 32, 32, 3, 3)
     assert lib.convolution_transform_filter_bytes_bnn_gfx950(bad, capi.C.byref(b), capi.AMD_GFX950) == capi.NOT_SUPPORTED
     w = np.zeros(48 * 32 * 9 // 8, np.uint8)
