@@ -127,6 +127,32 @@ def test_bnn_errors(torch_mod):
                                                        capi.AMD_GFX950) == capi.NOT_SUPPORTED
 
 
+@pytest.mark.parametrize("xnor", [True, False])
+def test_bnn_many_pixels_every_route(torch_mod, co, route, xnor):
+    """44 x 28 x 28 pixels x 256 channels is 135 tiles of 256 pixels: enough for the E2M1 kernel to be
+    chosen, which the small shapes above never reach. Whole result against the oracle, fp32 and sums,
+    XNOR and DoReFa, fp32 and bit-packed input."""
+    torch = torch_mod
+    shape = (44, 32, 28, 28, 256, 3, 3, 1, 1)
+    n, ic, ih, iw, oc, fh, fw, stride, pad = shape
+    print("bnn many pixels", route, xnor, shape, flush=True)
+    fdt = DT_BIN11 if xnor else DT_BIN01
+    x, w, scale, bias = make_case(shape, xnor, 5 + int(xnor))
+    d = co.bnn_desc(n, ic, ih, iw, oc, fh, fw, stride, pad, xnor)
+    x8 = to_nchwc(x, 8)
+    bits = co.bnn_pack_input(d, x8)
+    wb = bnn_pack_filter_nchwn16c8(w, xnor)
+    want_s, want_f = co.bnn_conv(d, bits, wb, scale, bias)
+    blob, ftm = host_conv.bnn_transform_filter(put(torch, True, wb), fdt, DF_NCHWN16C8, oc, ic, fh, fw)
+    sc, bs = put(torch, True, scale), put(torch, True, bias)
+    got_f = get(True, host_conv.convolution_bnn(put(torch, True, x8.reshape(-1)), DT_F32, n, ic, ih, iw, blob, ftm, oc,
+                                                fh, fw, stride, pad, sc, bs, DT_F32))
+    assert np.array_equal(got_f.view(np.int32), want_f.view(np.int32))
+    got_s = get(True, host_conv.convolution_bnn(put(torch, True, bits), fdt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride,
+                                                pad, sc, bs, DT_I32))
+    assert np.array_equal(got_s, want_s)
+
+
 def test_bnn_config5_single_image(torch_mod, co, route):
     shape = (1, 256, 28, 28, 256, 3, 3, 1, 1)
     n, ic, ih, iw, oc, fh, fw, stride, pad = shape
