@@ -112,15 +112,22 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         return only is None or only == name
 
     def timed(fn, reps, warm=3):
+        """Milliseconds per call: `reps` calls in up to five equal batches, each batch between HIP events on the
+        library stream; the median batch is reported, so that one stall of the box does not set the figure."""
         for _ in range(warm):
             fn()
         capi.check(L.bolt_gfx950_synchronize(), "sync")
-        ms = C.c_float(0)
-        capi.check(L.bolt_gfx950_timer_start(), "timer")
-        for _ in range(reps):
-            fn()
-        capi.check(L.bolt_gfx950_timer_stop(C.byref(ms)), "timer")
-        return ms.value / reps
+        batches = 5 if reps >= 10 else 1
+        per = max(1, reps // batches)
+        out = []
+        for _ in range(batches):
+            ms = C.c_float(0)
+            capi.check(L.bolt_gfx950_timer_start(), "timer")
+            for _ in range(per):
+                fn()
+            capi.check(L.bolt_gfx950_timer_stop(C.byref(ms)), "timer")
+            out.append(ms.value / per)
+        return sorted(out)[len(out) // 2]
 
     # -- int8 GEMM: square sweep + the BERT-base layer shapes, through both callers of the kernel:
     #    matrix_matrix_multiply (C += A.B: the int32 bits already in C are read and added, as the reference
