@@ -188,7 +188,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                                                               tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp), odesc,
                                                               host.ptr(out), C.byref(so), AMD_GFX950_DEVICE), "fully_connected"), 200)
         res["fc_c1"] = {"ms": t, "tops": 2.0 * M * N * K / t / 1e9, "algorithmic_bytes": 1380352,
-                        "gbps": 1380352 / t / 1e6, "note": "two launches (bias fold, GEMM) issued from Python through ctypes"}
+                        "gbps": 1380352 / t / 1e6, "note": "one launch (bias fold inside the GEMM kernel) issued from Python through ctypes"}
     # -- C3: int8 3x3 convolution 32x64x56x56 -> 64, ReLU, u8 out with dynamic output scale
     if want("conv"):
         n, ic, ih, iw, oc = 32, 64, 56, 56, 64

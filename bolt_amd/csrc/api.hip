@@ -207,6 +207,7 @@ EE mmm_device(U32 M, U32 N, U32 K, DataFormat adf, const void *A, DataFormat bdf
         scale = nullptr;  // mmm.cpp:222-224
     }
     GemmArgs g;
+    memset(&g, 0, sizeof(g));  // every field a kernel may look at, including the ones this caller does not use
     g.A = (const uint8_t *)A;
     g.transA = (adf == DF_TRANSPOSE);
     g.lda = g.transA ? M : K;
@@ -1108,9 +1109,13 @@ static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataForm
     }
     const U32 mat = packed_matrix_bytes(N, K);
     const bool packed = (fdf == DF_NKNxKx || fdf == DF_NKN32K4);
-    // :404-406 -- the compensation vector sits behind the packed matrix; native formats have none
-    HIP_TRY(launch_bias_offsetC((const float *)bias, N, packed ? (const int32_t *)((const U8 *)filter + mat) : nullptr,
-        nullptr, scaleO, (int32_t *)t, c.stream));
+    // :404-406 -- round(bias * scaleO) is added to the compensation vector behind the packed matrix; the kernels do
+    // that fold themselves for the columns they own (same arithmetic as quantize_bias_offsetC), so there is no
+    // separate launch and nothing is parked in tmp
+    if (!packed) {
+        return fail(NOT_SUPPORTED, "FullyConnected expects a pre-packed filter (transform_filter)");
+    }
+    const int32_t *fcomp = (const int32_t *)((const U8 *)filter + mat);
     // the reference zeroes the result (:458) and the product accumulates into it; starting the
     // accumulation from zero without reading the buffer is the same result
     EE e;
@@ -1125,8 +1130,10 @@ static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataForm
         g.x = (const uint8_t *)input;
         g.K = K;
         g.N = N;
-        g.ob = (const int32_t *)t;
-        g.comp = (const int32_t *)((const U8 *)filter + mat);
+        g.ob = fcomp;
+        g.comp = fcomp;
+        g.fold_bias = (const float *)bias;
+        g.fold_scale = scaleO;
         g.y = dst;
         g.epi = epi_from_scale(cdt == DT_I32 ? nullptr : scale);
         HIP_TRY(launch_gemv_s8u8(g, c.stream));
@@ -1142,8 +1149,10 @@ static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataForm
         g.M = M;
         g.N = N;
         g.K = K;
-        g.ob = (const int32_t *)t;
-        g.comp = (const int32_t *)((const U8 *)filter + mat);
+        g.ob = fcomp;
+        g.comp = fcomp;
+        g.fold_bias = (const float *)bias;
+        g.fold_scale = scaleO;
         g.C = dst;
         g.epi = epi_from_scale(cdt == DT_I32 ? nullptr : scale);
         HIP_TRY(launch_gemm_u8s8(g, c.stream));
@@ -1340,7 +1349,8 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // filter blob = [offsetC oc*4][packed matrix] (convolution_transform.cpp:36-44 keeps the vector in front)
     const int32_t *offC = (const int32_t *)filter;
     const int8_t *mat = (const int8_t *)filter + (size_t)s.oc * 4;
-    HIP_TRY(launch_bias_offsetC((const float *)bias, s.oc, offC, nullptr, scaleO, (int32_t *)(t + offOff), c.stream));
+    // offsetC + round(bias * scaleO) (convolution_direct.cpp:2687-2700) is formed inside the kernel for the columns
+    // it owns: no separate launch
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.A = (const uint8_t *)t;
@@ -1348,8 +1358,10 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     g.M = s.n * s.oh * s.ow;
     g.N = s.oc;
     g.K = s.Kp;
-    g.ob = (const int32_t *)(t + offOff);
+    g.ob = offC;
     g.comp = offC;
+    g.fold_bias = (const float *)bias;
+    g.fold_scale = scaleO;
     g.conv.OHW = s.oh * s.ow;
     g.conv.OW = s.ow;
     g.conv.sh = s.sh;

@@ -45,12 +45,12 @@ enum EpiMode : int {
 };
 
 struct Epilogue {
-    int mode;
-    float factor;            // EPI_F32 / EPI_U8 when dfactor == nullptr
-    const float *dfactor;    // optional device scalar: EPI_F32 uses 1.0f / *dfactor, EPI_U8 uses *dfactor
-    const float *scaleI;     // EPI_F32_CH: device scalar input scale
-    const float *scaleW;     // EPI_F32_CH: device per-channel weight scales [N]
-    const float *bias;       // EPI_F32_CH: optional device fp32 bias [N]
+    int mode = 0;
+    float factor = 0;            // EPI_F32 / EPI_U8 when dfactor == nullptr
+    const float *dfactor = nullptr;    // optional device scalar: EPI_F32 uses 1.0f / *dfactor, EPI_U8 uses *dfactor
+    const float *scaleI = nullptr;     // EPI_F32_CH: device scalar input scale
+    const float *scaleW = nullptr;     // EPI_F32_CH: device per-channel weight scales [N]
+    const float *bias = nullptr;       // EPI_F32_CH: optional device fp32 bias [N]
 };
 
 __device__ __forceinline__ float epi_factor(const Epilogue &e)
@@ -116,6 +116,22 @@ template <typename V>
 __device__ __forceinline__ void st_stream(V *p, V v)
 {
     __builtin_nontemporal_store(v, p);
+}
+
+// Offset a product's column n starts from, less the compensation of the u8 -> s8 re-bias: ob[n] - comp[n], or --
+// when the caller hands over the fp32 bias instead of a folded vector -- the fold done here exactly as the
+// stand-alone kernel does it (round(bias * scale) + offsetC in double, converted to int32;
+// avx512/quantize.cpp:236-269), so that no separate launch is needed for it.
+__device__ __forceinline__ uint32_t column_base(const int32_t *ob, const int32_t *comp, const float *fold_bias,
+    float fold_scale, uint32_t n)
+{
+    const int32_t c = comp[n];
+    if (fold_bias) {
+        const float p = fold_bias[n] * fold_scale;
+        const int32_t o = (int32_t)(round((double)p) + (double)c);
+        return (uint32_t)o - (uint32_t)c;
+    }
+    return (uint32_t)ob[n] - (uint32_t)c;
 }
 
 __device__ __forceinline__ float wave_reduce_sum(float v)

@@ -26,7 +26,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v4i &acc, ui
     if (n >= a.N) {
         return;
     }
-    const uint32_t base = (uint32_t)a.ob[n] - (uint32_t)a.comp[n];
+    const uint32_t base = column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n);
     float factor = 0.0f, sI = 0.0f, sW = 0.0f;
     if (a.epi.mode == EPI_F32 || a.epi.mode == EPI_U8) {
         factor = epi_factor(a.epi);
@@ -209,7 +209,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const bool ok = FULL || (n + c < a.N);
-            base[y][c] = ok ? (uint32_t)a.ob[n + c] - (uint32_t)a.comp[n + c] : 0u;
+            base[y][c] = ok ? column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c) : 0u;
             qs[y][c] = 1.0f;
             bs[y][c] = 0.0f;
             if (MODE == EPI_F32_CH && ok) {
@@ -404,10 +404,9 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
     uint32_t base[4];
     float qs[4], bs[4];
     {
-        const v4i ob = *(const v4i *)(a.ob + n), cp = *(const v4i *)(a.comp + n);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            base[c] = (uint32_t)ob[c] - (uint32_t)cp[c];
+            base[c] = column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c);
             qs[c] = 1.0f;
             bs[c] = 0.0f;
             if (MODE == EPI_F32_CH) {
@@ -726,7 +725,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     {
         const uint32_t n = n0 + wn * TN * 16 + lane;
         if (lane < TN * 16 && n < a.N) {
-            warm = a.ob[n] ^ a.comp[n];
+            warm = (a.fold_bias ? __float_as_int(a.fold_bias[n]) : a.ob[n]) ^ a.comp[n];
         }
     }
 

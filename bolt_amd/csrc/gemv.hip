@@ -26,7 +26,7 @@ template <int ROWS, int XV>
 __global__ __launch_bounds__(256) void gemv_s8u8_kernel(const int8_t *__restrict__ W, uint32_t ldw,
     const uint8_t *__restrict__ x, uint32_t K, uint32_t N, const int32_t *__restrict__ ob,
     const int32_t *__restrict__ comp, void *__restrict__ y, uint32_t tail0, int add_yin, Epilogue epi,
-    GemvBatch bt)
+    GemvBatch bt, const float *__restrict__ fold_bias, float fold_scale)
 {
     // strided batch of independent products: slice b uses weight blob b % wcopies, its own
     // activation vector, result vector and (per-channel epilogue) input scale
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void gemv_s8u8_kernel(const int8_t *__restrict
     if (lane < ROWS && n < N) {
         const bool tail = (n >= tail0);
         // int32 two's-complement wrap, as vpdpbusd / vpaddd
-        uint32_t a = (uint32_t)mine + (uint32_t)ob[n] - (uint32_t)comp[n];
+        uint32_t a = (uint32_t)mine + column_base(ob, comp, fold_bias, fold_scale, n);
         if (add_yin && !tail && epi.mode != EPI_U8) {
             a += (uint32_t)((const int32_t *)y)[n];
         }
@@ -193,10 +193,10 @@ static hipError_t launch_s8u8(const GemvArgs &a, hipStream_t st)
     const bool xv = (((uintptr_t)a.x | (uintptr_t)a.batch.xstride) & 3) == 0;
     if (xv) {
         hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 1>), grid, dim3(256), 0, st, a.W, a.ldw, a.x, a.K, a.N, a.ob,
-            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch);
+            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch, a.fold_bias, a.fold_scale);
     } else {
         hipLaunchKernelGGL((gemv_s8u8_kernel<ROWS, 0>), grid, dim3(256), 0, st, a.W, a.ldw, a.x, a.K, a.N, a.ob,
-            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch);
+            a.comp, a.y, tail0, a.add_yin, a.epi, a.batch, a.fold_bias, a.fold_scale);
     }
     return hipGetLastError();
 }

@@ -7,25 +7,30 @@
 
 namespace bg {
 
+// Every field of the argument structs below has a default (null / 0): a caller that leaves one out hands the
+// kernel a harmless value, never an indeterminate pointer.
+
 // ---- GEMV ---------------------------------------------------------------------------------------
 struct GemvBatch {
-    uint32_t count;      // number of independent products in the launch (0 / 1: a single one)
-    uint32_t wcopies;    // slice b reads the weight blob b % wcopies (0: one blob)
-    size_t wstride;      // bytes between consecutive weight blobs
-    uint32_t xstride;    // bytes between activation vectors
-    uint32_t ystride;    // bytes between result vectors
-    int ob_in_blob;      // ob points into the blob and moves with it
+    uint32_t count = 0;      // number of independent products in the launch (0 / 1: a single one)
+    uint32_t wcopies = 0;    // slice b reads the weight blob b % wcopies (0: one blob)
+    size_t wstride = 0;      // bytes between consecutive weight blobs
+    uint32_t xstride = 0;    // bytes between activation vectors
+    uint32_t ystride = 0;    // bytes between result vectors
+    int ob_in_blob = 0;      // ob points into the blob and moves with it
 };
 
 struct GemvArgs {
-    const int8_t *W;     // packed weight: row-major [ALIGN(N,16)][ldw], rows zero-padded
-    uint32_t ldw;        // ALIGN(K, 8)
-    const uint8_t *x;    // [K]
-    uint32_t K, N;
-    const int32_t *ob;   // caller's offsetC (+ folded bias) [N]
-    const int32_t *comp; // -128 * sum_k W[n][k], stored behind the packed matrix [N]
-    void *y;
-    int add_yin;         // accumulate into the int32 bits already in y
+    const int8_t *W = nullptr;     // packed weight: row-major [ALIGN(N,16)][ldw], rows zero-padded
+    uint32_t ldw = 0;        // ALIGN(K, 8)
+    const uint8_t *x = nullptr;    // [K]
+    uint32_t K = 0, N = 0;
+    const int32_t *ob = nullptr;   // caller's offsetC (+ folded bias) [N]
+    const int32_t *comp = nullptr; // -128 * sum_k W[n][k], stored behind the packed matrix [N]
+    const float *fold_bias = nullptr;  // if set, ob is not read: the offset is (int32)(round(fold_bias[n] * fold_scale) + comp[n])
+    float fold_scale = 0;
+    void *y = nullptr;
+    int add_yin = 0;         // accumulate into the int32 bits already in y
     Epilogue epi;
     GemvBatch batch;
 };
@@ -37,31 +42,33 @@ hipError_t launch_gemv_u8s8(const uint8_t *A, uint32_t lda, uint32_t sk, const i
 // Geometry of an implicit-GEMM convolution (GemmArgs::conv), all in elements / bytes of the padded,
 // s8 image in planes of 16 channels, [n][ICp/16][Hp][Wp][16], that conv_pad produces.
 struct ConvGeom {
-    uint32_t OHW, OW;          // output pixels per image, output width
-    uint32_t sh, sw;           // strides
-    uint32_t Hp, Wp, ICp;      // padded image height / width, channels rounded up to 16
-    uint32_t fh, fw, dh, dw;   // filter taps and dilation: K runs over (kh, kw, c) in 16-channel chunks
-    uint32_t out_c;            // channel block of the output layout: 16 (NCHWC16) or 8 (NCHWC8)
-    int relu;
-    const float *eltwise;      // optional fp32 tensor added before the ReLU (fp32 output only)
-    uint32_t *absmax;          // scratch slots: int32 mode folds max |acc| into them (C may then be null:
+    uint32_t OHW = 0, OW = 0;          // output pixels per image, output width
+    uint32_t sh = 0, sw = 0;           // strides
+    uint32_t Hp = 0, Wp = 0, ICp = 0;      // padded image height / width, channels rounded up to 16
+    uint32_t fh = 0, fw = 0, dh = 0, dw = 0;   // filter taps and dilation: K runs over (kh, kw, c) in 16-channel chunks
+    uint32_t out_c = 0;            // channel block of the output layout: 16 (NCHWC16) or 8 (NCHWC8)
+    int relu = 0;
+    const float *eltwise = nullptr;      // optional fp32 tensor added before the ReLU (fp32 output only)
+    uint32_t *absmax = nullptr;          // scratch slots: int32 mode folds max |acc| into them (C may then be null:
                                // nothing is stored); u8 mode reads them for the tensor-wide dynamic scale
-    float scaleO;              // u8 mode: scale of the accumulators (input scale * filter scale)
-    float *dscale_out;         // u8 mode: device word that receives the resulting output scale
+    float scaleO = 0;              // u8 mode: scale of the accumulators (input scale * filter scale)
+    float *dscale_out = nullptr;         // u8 mode: device word that receives the resulting output scale
 };
 
 struct GemmArgs {
-    const uint8_t *A;    // u8 activations
-    uint32_t lda;        // bytes between consecutive m (transA = 0) or consecutive k (transA = 1)
-    int transA;          // 1: A stored [K][M]
-    const int8_t *Bp;    // packed right-hand side (fragment layout, see pack.hip)
-    uint32_t M, N, K;
-    const int32_t *ob;   // caller's offsetC (+ folded bias) [N]
-    const int32_t *comp; // blob's own compensation vector [N]
-    void *C;             // [M][N] row-major
-    int add_cin;         // accumulate into the int32 bits already in C
-    int stream_c;        // set by the launcher: write C with the non-temporal hint
-    int fp4;             // convolution only: operand bytes are pairs of E2M1 values (1-bit convolution), K counts bytes
+    const uint8_t *A = nullptr;    // u8 activations
+    uint32_t lda = 0;        // bytes between consecutive m (transA = 0) or consecutive k (transA = 1)
+    int transA = 0;          // 1: A stored [K][M]
+    const int8_t *Bp = nullptr;    // packed right-hand side (fragment layout, see pack.hip)
+    uint32_t M = 0, N = 0, K = 0;
+    const int32_t *ob = nullptr;   // caller's offsetC (+ folded bias) [N]
+    const int32_t *comp = nullptr; // blob's own compensation vector [N]
+    const float *fold_bias = nullptr;  // if set, ob is not read: the offset is (int32)(round(fold_bias[n] * fold_scale) + comp[n])
+    float fold_scale = 0;
+    void *C = nullptr;             // [M][N] row-major
+    int add_cin = 0;         // accumulate into the int32 bits already in C
+    int stream_c = 0;        // set by the launcher: write C with the non-temporal hint
+    int fp4 = 0;             // convolution only: operand bytes are pairs of E2M1 values (1-bit convolution), K counts bytes
     Epilogue epi;
     ConvGeom conv;       // used by launch_conv_u8s8 only
 };
@@ -83,13 +90,13 @@ hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, 
 
 // ---- 1-bit convolution (bnn.hip) ----------------------------------------------------------------
 struct BnnArgs {
-    const uint32_t *x;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded
-    const uint32_t *w;     // [OC/32][fh*fw][IC/32][32] dwords
-    uint32_t M;            // n * OH * OW output pixels
-    uint32_t OHW, OW, sh, sw, Hp, Wp, IC, OC, fh, fw;
-    int32_t *sums;         // optional int32 sums, NCHWC8
-    float *out;            // optional fma(S, scale[oc], bias[oc]), NCHWC8
-    const float *scale, *bias;
+    const uint32_t *x = nullptr;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded
+    const uint32_t *w = nullptr;     // [OC/32][fh*fw][IC/32][32] dwords
+    uint32_t M = 0;            // n * OH * OW output pixels
+    uint32_t OHW = 0, OW = 0, sh = 0, sw = 0, Hp = 0, Wp = 0, IC = 0, OC = 0, fh = 0, fw = 0;
+    int32_t *sums = nullptr;         // optional int32 sums, NCHWC8
+    float *out = nullptr;            // optional fma(S, scale[oc], bias[oc]), NCHWC8
+    const float *scale = nullptr, *bias = nullptr;
 };
 hipError_t launch_bnn_pack_input(const void *in, int from_f32, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t pt,
     uint32_t pb, uint32_t pl, uint32_t pr, float thr, uint32_t *out, hipStream_t st);
