@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--only", choices=["gemm", "fc", "conv", "bnn", "encoder", "quantize"],
+    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize"],
                     help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
@@ -148,8 +148,8 @@ def other_kernels(L, capi, host, torch, dev, only=None):
 
             def add(path, nm, t):
                 tops = 2.0 * M * N * K / t / 1e9
-                gemm.append({"M": M, "K": K, "N": N, "path": path, "out": nm, "ms": t, "tops": tops,
-                             "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
+                gemm.append({"M": M, "K": K, "N": N, "path": path, "out": nm, "operands": "uniform u8 x uniform s8",
+                             "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
             for cdt, tdt, sc, nm in ((DT_F32, torch.float32, [37.25], "f32"), (DT_I32, torch.int32, None, "i32_accumulate"),
                                      (DT_U8_Q, torch.uint8, [-1.0, 1e-5], "u8")):
                 Cb = torch.zeros((M, N), dtype=tdt, device=dev)
@@ -171,6 +171,51 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                 del tmp, out
             del A, W, blob
         res["gemm_int8"] = gemm
+    if want("gemm_data"):
+        from bolt_amd.capi import AMD_GFX950_DEVICE, DT_I8, tensor1d
+        # -- the same kernel against what the device sustains: the clock it holds depends on how many operand
+        #    bits toggle, so 8192^3 is also timed on operands as a network produces them and on constant ones,
+        #    next to a register-resident MFMA loop with random and with all-zero operands
+        M = K = N = 8192
+
+        def quantised(x, per_row, lo, hi, zero_point):
+            s = 127.0 / (x.abs().amax(dim=1, keepdim=True) if per_row else x.abs().max())
+            return (torch.round(x * s) + zero_point).clamp(lo, hi)
+        dists = (("uniform u8 x uniform s8",
+                  lambda: torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g),
+                  lambda: torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)),
+                 ("u8 of relu(N(0,1)), per-tensor scale x s8 of N(0,0.02), per-channel scale",
+                  lambda: quantised(torch.relu(torch.randn((M, K), device=dev, generator=g)), False, 1, 255, 128).to(torch.uint8),
+                  lambda: quantised(torch.randn((N, K), device=dev, generator=g) * 0.02, True, -127, 127, 0).to(torch.int8)),
+                 ("constant: u8 128 x s8 0",
+                  lambda: torch.full((M, K), 128, dtype=torch.uint8, device=dev),
+                  lambda: torch.zeros((N, K), dtype=torch.int8, device=dev)))
+        by_data = []
+        for name, fa, fw in dists:
+            A, W = fa(), fw()
+            blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            bias = torch.randn(N, device=dev, generator=g) * 0.1
+            nbytes = host.fully_connected_tmp_bytes(M, K, N, DF_NKNxKx, DT_U8_Q, AMD_GFX950_DEVICE)
+            tmp = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            out = torch.empty((M, N), dtype=torch.uint8, device=dev)
+            so = C.c_float(0.05)
+            t = timed(lambda: capi.check(L.fully_connected_gfx950(
+                tensor2df(DT_U8_Q, DF_NORMAL, M, K), host.ptr(A), 30.0, tensor2df(DT_I8, DF_NKNxKx, K, N), host.ptr(blob), 100.0,
+                tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp), tensor2df(DT_U8_Q, DF_NORMAL, M, N), host.ptr(out),
+                C.byref(so), AMD_GFX950_DEVICE), "fully_connected"), 20, warm=30)  # long warm-up: the clock settles over ~10 ms
+            tops = 2.0 * M * N * K / t / 1e9
+            by_data.append({"M": M, "K": K, "N": N, "path": "fully_connected", "out": "u8_static_scale", "operands": name,
+                            "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
+            del A, W, blob, tmp, out
+        rate = {}
+        for key, zero in (("random_operands_tops", 0), ("zero_operands_tops", 1)):
+            v = C.c_float(0)
+            capi.check(L.bolt_gfx950_mfma_int8_rate(zero, C.byref(v)), "mfma_int8_rate")
+            rate[key] = v.value
+        rate["note"] = ("v_mfma_i32_16x16x64_i8 back to back from registers, 8 waves per CU, no memory traffic: the device "
+                        "lowers its clock when the operand bits are random")
+        res["gemm_int8_8192_by_operand_data"] = by_data
+        res["mfma_int8_sustained"] = rate
     # -- C1: FullyConnected M=64 K=1024 N=1024, fp32 out
     if want("fc"):
         M, K, N = 64, 1024, 1024

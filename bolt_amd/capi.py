@@ -100,6 +100,7 @@ class BoltEncoderLayerInt8(C.Structure):
 
 SIGNATURES = {
     "bolt_gfx950_init": (C.c_int, []),
+    "bolt_gfx950_mfma_int8_rate": (C.c_int, [C.c_int, C.POINTER(C.c_float)]),
     "bolt_gfx950_set_stream": (C.c_int, [_vp]),
     "bolt_gfx950_synchronize": (C.c_int, []),
     "bolt_gfx950_last_error": (C.c_char_p, []),

@@ -397,6 +397,53 @@ EE bolt_gfx950_timer_stop(float *ms)
     return SUCCESS;
 }
 
+EE bolt_gfx950_mfma_int8_rate(int zero_operands, float *tops)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!tops) {
+        return fail(NULL_POINTER, "mfma_int8_rate: tops is null");
+    }
+    Ctx &c = ctx();
+    int dev = 0, cus = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const uint32_t blocks = (uint32_t)cus;
+    const uint32_t iters = 8000;  // 2 waves per SIMD x 8000 x 32 x 16 cycles: a few milliseconds
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    float best = 0.0f;
+    hipError_t err = launch_mfma_i8_rate(blocks, iters / 8, zero_operands, nullptr, c.stream);  // warm-up
+    for (int r = 0; r < 3 && err == hipSuccess; ++r) {
+        float ms = 0.0f;
+        err = hipEventRecord(e0, c.stream);
+        if (err == hipSuccess) {
+            err = launch_mfma_i8_rate(blocks, iters, zero_operands, nullptr, c.stream);
+        }
+        if (err == hipSuccess) {
+            err = hipEventRecord(e1, c.stream);
+        }
+        if (err == hipSuccess) {
+            err = hipEventSynchronize(e1);
+        }
+        if (err == hipSuccess) {
+            err = hipEventElapsedTime(&ms, e0, e1);
+        }
+        if (err == hipSuccess && (best == 0.0f || ms < best)) {
+            best = ms;
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    HIP_TRY(err);
+    const double ops = (double)blocks * 8.0 * (double)iters * 32.0 * (2.0 * 16 * 16 * 64);
+    *tops = (float)(ops / ((double)best * 1e-3) / 1e12);
+    return SUCCESS;
+}
+
 // ---- GEMM ----------------------------------------------------------------------------------------
 DataFormat matrix_matrix_multiply_rhs_format_gfx950(DataType dt)
 {

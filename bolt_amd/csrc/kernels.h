@@ -156,6 +156,8 @@ hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *off
     float scaleB, int32_t *out, hipStream_t st);
 hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float rescale, int8_t *out, hipStream_t st);
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
+// probe.hip: register-resident int8 MFMA loop, blocks x 8 waves x iters x 32 instructions
+hipError_t launch_mfma_i8_rate(uint32_t blocks, uint32_t iters, int zero, int *sink, hipStream_t st);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]
 
 }  // namespace bg

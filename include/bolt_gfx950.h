@@ -54,6 +54,11 @@ EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes);
 /* Event pair on the library stream; stop returns the elapsed milliseconds after waiting. */
 EE bolt_gfx950_timer_start(void);
 EE bolt_gfx950_timer_stop(float *ms);
+/* Measurement aid with no counterpart in the reference: the rate (TOP/s) that the int8 matrix cores of
+ * this device sustain on v_mfma_i32_16x16x64_i8 issued back to back from registers by 8 waves on every
+ * CU, with random operand bits (zero_operands = 0: the device lowers its clock under that load) or with
+ * all-zero operands (1). Takes a few milliseconds. The GEMM figures are read against these two. */
+EE bolt_gfx950_mfma_int8_rate(int zero_operands, float *tops);
 
 /* ---- blas_enhance: int8 GEMM --------------------------------------------------------- */
 /* compute/blas_enhance/include/blas_enhance.h:36-37  matrix_matrix_multiply_tmp_bytes */
