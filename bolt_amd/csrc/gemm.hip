@@ -738,6 +738,141 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
         }
     }
 
+    if constexpr (PIPE == 3) {
+        // Ping-pong schedule as PIPE == 2, with A requested in whole 128-byte lines. A request of 16 rows x 64
+        // bytes (one MFMA fragment, what the other loops issue) touches 16 half lines and the L1 / L2 path
+        // delivers such requests 2.5 times slower than 1 KB made of 8 whole lines (measured in isolation:
+        // 1 040 against 410 cycles per 16 KB and CU), which is more than the MFMAs of a K tile take. Here a
+        // request covers 8 rows x 128 bytes = the K bytes of two consecutive tiles, so A travels in pairs of
+        // tiles: three slots of 256 rows x 128 bytes (tile pair p in slot p % 3, requested four tiles ahead
+        // at the even tile) next to the four B slots of 16 KB (tile t in slot t % 4, requested three ahead).
+        // Inside a slot the 16 rows x 128 bytes of row block r sit at r * 2 KB; lane (8 * row + pos) of a
+        // request fetches 16-byte chunk pos ^ sw of its row, sw = (row16 >> 1) & 7 with row16 the row inside
+        // the 16-row block, so that the fragment read of K half h (lane (i, g) reads chunk 4 h + g of row i:
+        // 16 consecutive lanes = 16 rows) spreads over all 64 banks.
+        static_assert(PIPE != 3 || (!CONV && !FP4 && WM * WN == 8 && STAGES == 5 && T::kAFrags == 16 && T::kBFrags == 16),
+            "the whole-line loop is written for 256 x 256 matrix tiles in 160 KB of LDS");
+        constexpr uint32_t kASlot = T::kAFrags * 2048, kBBase = 3 * kASlot, kBSlot = T::kBFrags * 1024;
+        constexpr int kQA2 = 2 * T::kAFrags / T::kWaves;  // requests per wave and tile pair
+        constexpr int kQB = T::kBFrags / T::kWaves;       // requests per wave and tile
+        static_assert(kBBase + 4 * kBSlot == (uint32_t)T::kLdsBytes, "LDS layout");
+        uint32_t offA[kQA2], offB[kQB];
+#pragma unroll
+        for (int q = 0; q < kQA2; ++q) {
+            const uint32_t b = wave + q * T::kWaves;  // block of 8 rows
+            uint32_t row = m0 + b * 8 + (lane >> 3);
+            row = row < a.M ? row : a.M - 1;
+            const uint32_t row16 = (b & 1) * 8 + (lane >> 3);
+            offA[q] = row * a.lda + (((lane & 7) ^ ((row16 >> 1) & 7)) * 16);
+        }
+#pragma unroll
+        for (int q = 0; q < kQB; ++q) {
+            uint32_t nb = (n0 >> 4) + (wave + q * T::kWaves);
+            nb = nb < nblocks ? nb : nblocks - 1;
+            offB[q] = nb * 16 * K + lane * 16;
+        }
+        const uint32_t ksteps = K / 64, kpairs = ksteps / 2;  // the launcher checks K % 128 == 0
+        const uint32_t rdA = (i >> 3) * 1024 + ((i & 7) * 8 + (g ^ ((i >> 1) & 7))) * 16;
+#define BG3_ISSUE_A(aslot, pair, QLO, QHI)                                                                        \
+    {                                                                                                             \
+        const uint8_t *base_ = a.A + (size_t)((pair) < kpairs ? (pair) : kpairs - 1) * 128;                       \
+        _Pragma("unroll") for (int q = (QLO); q < (QHI); ++q)                                                     \
+        {                                                                                                         \
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_ + offA[q]),                                           \
+                (lptr_t)(smem + (aslot)*kASlot + (wave + q * T::kWaves) * 1024), 16, 0, 0);                       \
+        }                                                                                                         \
+    }
+#define BG3_ISSUE_B(tile)                                                                                         \
+    {                                                                                                             \
+        const uint8_t *base_ = (const uint8_t *)a.Bp + (size_t)((tile) < ksteps ? (tile) : ksteps - 1) * 1024;    \
+        _Pragma("unroll") for (int q = 0; q < kQB; ++q)                                                           \
+        {                                                                                                         \
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_ + offB[q]),                                           \
+                (lptr_t)(smem + kBBase + ((tile)&3) * kBSlot + (wave + q * T::kWaves) * 1024), 16, 0, 0);         \
+        }                                                                                                         \
+    }
+        // Every tile requests its B three tiles ahead; the even tile t then also requests the A pair t / 2 + 2
+        // (tiles t+4, t+5). Order: A0 B0 B1 A1 B2 | tile 0: B3 A2 | tile 1: B4 | tile 2: B5 A3 | tile 3: B6 | ...
+        BG3_ISSUE_A(0u, 0u, 0, kQA2);
+        BG3_ISSUE_B(0u);
+        BG3_ISSUE_B(1u);
+        BG3_ISSUE_A(1u, 1u, 0, kQA2);
+        BG3_ISSUE_B(2u);
+        v4i fa[TM], fb[TN];
+        const bool late = wave >= 4;
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kQA2 + 2 * kQB));  // tile 0 landed: B1, A1, B2 may be outstanding
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (late) {
+            __builtin_amdgcn_s_barrier();
+        }
+        // What must have landed at the start of memory phase t is this wave's share of tile t+1. Even t (HALF 0):
+        // the pair of tile t+1 is the one being read, B(t+1) is the youngest request needed, and behind it are a
+        // pair and B(t+2). Odd t (HALF 1): tile t+1 opens the pair requested three tiles ago, which precedes
+        // B(t+1) in the order; behind B(t+1) are B(t+2) and the pair requested at tile t-1. Either way kQA2 + kQB
+        // requests may still be outstanding.
+#define BG3_STEP(HALF)                                                                                            \
+    {                                                                                                             \
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kQA2 + kQB));                                                        \
+        asm volatile("" ::: "memory");                                                                            \
+        BG3_ISSUE_B(t + 3);                                                                                       \
+        if (!(HALF)) {                                                                                            \
+            BG3_ISSUE_A(aslot_req, t / 2 + 2, 0, kQA2);                                                           \
+        }                                                                                                         \
+        {                                                                                                         \
+            const uint8_t *sA_ = smem + aslot * kASlot + (rdA ^ ((HALF)*64));                                     \
+            const uint8_t *sB_ = smem + kBBase + (t & 3) * kBSlot;                                                \
+            _Pragma("unroll") for (int y = 0; y < TN; ++y)                                                        \
+            {                                                                                                     \
+                fb[y] = *(const v4i *)(sB_ + (wn * TN + y) * 1024 + lane * 16);                                   \
+            }                                                                                                     \
+            _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                        \
+            {                                                                                                     \
+                fa[x] = *(const v4i *)(sA_ + (wm * TM + x) * 2048);                                               \
+            }                                                                                                     \
+        }                                                                                                         \
+        __builtin_amdgcn_s_waitcnt(0xc07f);                                                                       \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                            \
+        {                                                                                                         \
+            fa[x] ^= flip;                                                                                        \
+        }                                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_s_barrier();                                                                             \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        __builtin_amdgcn_s_setprio(1);                                                                            \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                            \
+        {                                                                                                         \
+            _Pragma("unroll") for (int y = 0; y < TN; ++y)                                                        \
+            {                                                                                                     \
+                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[x], acc[x][y], 0, 0, 0);              \
+            }                                                                                                     \
+        }                                                                                                         \
+        __builtin_amdgcn_s_setprio(0);                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_s_barrier();                                                                             \
+        asm volatile("" ::: "memory");                                                                            \
+    }
+        uint32_t aslot = 0, aslot_req = 2;  // slot of the pair being read / of the pair requested at the even tile
+        for (uint32_t t = 0; t < ksteps; t += 2) {
+            BG3_STEP(0);
+            ++t;
+            BG3_STEP(1);
+            --t;
+            aslot = aslot == 2 ? 0 : aslot + 1;
+            aslot_req = aslot_req == 2 ? 0 : aslot_req + 1;
+        }
+        if (!late) {
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches
+#undef BG3_STEP
+#undef BG3_ISSUE_A
+#undef BG3_ISSUE_B
+    } else {
     // This wave's fragments per K tile: kQA A fragments (16 rows x 64 K-bytes), then B fragments.
     // Addresses are split into a wave-uniform 64-bit base that advances with the tile (scalar
     // registers, scalar ALU) and a 32-bit per-lane offset that never changes, so the loop issues
@@ -1020,6 +1155,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 #undef BG_AOFF
 #undef BG_CV_OFF
 #undef BG_CV_ADVANCE
+    }  // PIPE != 3
     asm volatile("" ::"v"(warm));  // keeps the warming loads alive; the value itself is not used
     if constexpr (FP4) {
         static_assert(!FP4 || PIPE == 2, "the fp4 product is wired into the ping-pong loop");
@@ -1272,6 +1408,20 @@ static hipError_t launch_tiled(const GemmArgs &a, hipStream_t st)
     return hipGetLastError();
 }
 
+// whether a block may use 160 KB of LDS on the current device (asked once)
+static bool lds_160k()
+{
+    static int have = -1;
+    if (have < 0) {
+        int dev = 0, bytes = 0;
+        have = (hipGetDevice(&dev) == hipSuccess &&
+                   hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && bytes >= 160 * 1024)
+            ? 1
+            : 0;
+    }
+    return have == 1;
+}
+
 static int g_conv_panel = 4;  // test hook: 0 = shared pipeline only, 2 / 4 = pixel blocks per wave of the panel kernel
 
 void conv_force_panel(int v)
@@ -1359,7 +1509,9 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
         // that 128 x 128 tiles keep more CUs busy; tiny problems go to the general kernel
         const bool k64 = (a.K % 64 == 0);
         if (b256 >= 128 && k64) {
-            tile = 11;  // ping-pong: 12 % faster than the fragment-prefetch loop at 8192^3, level elsewhere
+            // ping-pong: 12 % faster than the fragment-prefetch loop at 8192^3, level elsewhere; with A requested in
+            // whole lines another 4 % at 8192^3 and level at 4096^3 (needs K % 128 == 0 and 160 KB of LDS)
+            tile = (a.K % 128 == 0) ? 12 : 11;
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
             tile = k64 ? 10 : 2;
         }
@@ -1370,6 +1522,9 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     const bool dma_ok = tiled_ok && (a.K % 64 == 0);
     if (tile >= 3 && !dma_ok) {
         tile = tiled_ok ? 2 : 0;
+    }
+    if (tile == 12 && (a.K % 128 != 0 || !lds_160k())) {
+        tile = 11;
     }
     switch (tile) {
         case 1:
@@ -1382,6 +1537,8 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 2, 4, 4, 4, true>(a, st);  // 128 x 128, fragment prefetch
         case 11:
             return launch_dma<2, 4, 8, 4, 4, 2>(a, st);  // 256 x 256, 8 waves, ping-pong memory / matrix phases
+        case 12:
+            return launch_dma<2, 4, 8, 4, 5, 3>(a, st);  // the same with A requested in whole 128-byte lines (160 KB of LDS)
         default:
             break;
     }

@@ -38,7 +38,8 @@ const char *bolt_gfx950_last_error(void);
 /* Tuning / test knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1-2 the
  * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 7 / 10 / 11 the LDS-DMA
  * kernels (256x256 fragment-prefetch, 128x128 fragment-prefetch, 256x256 ping-pong; need
- * K % 64 == 0), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
+ * K % 64 == 0), 12 the 256x256 ping-pong kernel that requests A in whole 128-byte lines (needs
+ * K % 128 == 0, else it runs as 11), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
  * the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
  * K <= 1024 uses: 4 (default) / 2 the filter-panel-in-LDS kernel with 64 / 32 pixels per wave, 0 the
  * shared-pipeline kernel. "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
