@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <chrono>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -22,6 +23,10 @@ struct Ctx {
     bool ready = false;
     hipStream_t stream = nullptr;
     uint32_t *ws = nullptr;  // device scratch words for the two-pass reductions
+    // One pinned host word that kernels write a freshly computed scale into (the interfaces that return a
+    // scale through a host pointer read it after the stream has drained: no copy command in between), and
+    // the address the device uses for it.
+    float *hscale = nullptr, *hscale_dev = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     struct Buf {
@@ -77,7 +82,45 @@ EE ensure_init()
     if (e != hipSuccess) {
         return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
     }
+    e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
+    if (e == hipSuccess) {
+        e = hipHostGetDevicePointer((void **)&c.hscale_dev, c.hscale, 0);
+    }
+    if (e != hipSuccess) {
+        return fail(ALLOC_FAILED, "hipHostMalloc(scale word)", e);
+    }
     c.ready = true;
+    return SUCCESS;
+}
+
+// A scale that a kernel computes and the interface returns through a host pointer: the host arms the pinned
+// word with a pattern no scale can have, the kernel's first thread stores the scale there, and the host
+// takes it as soon as it shows up -- the rest of the call stays ordered on the stream like every other
+// device-pointer call, and no copy command or stream drain sits between two calls. If the word has not
+// changed after 2 ms the stream is drained instead (a launch that produced nothing must not hang the caller).
+constexpr uint32_t kScaleUnset = 0xffffffffu;
+
+void arm_scale(Ctx &c)
+{
+    *(volatile uint32_t *)c.hscale = kScaleUnset;
+}
+
+EE take_scale(Ctx &c, float *dst)
+{
+    volatile uint32_t *w = (volatile uint32_t *)c.hscale;
+    const auto t0 = std::chrono::steady_clock::now();
+    uint32_t spins = 0;
+    while (*w == kScaleUnset) {
+        if ((++spins & 0x3ff) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) {
+            HIP_TRY(hipStreamSynchronize(c.stream));
+            break;
+        }
+    }
+    const uint32_t bits = *w;
+    if (bits == kScaleUnset) {
+        return fail(UNKNOWN, "the kernel did not produce a scale");
+    }
+    memcpy(dst, &bits, 4);
     return SUCCESS;
 }
 
@@ -894,8 +937,9 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     } else if (!aligned4(data) && ddt != DT_U8_Q) {
         return fail(NOT_SUPPORTED, "device data must be 4-byte aligned");
     }
-    float *dscale = (float *)(c.ws + kWsWords);
+    float *dscale = c.hscale_dev;
     bool read_back = false;
+    arm_scale(c);
     if (f32in) {
         const bool dynamic = (!mode || *scale <= 0);
         if (dynamic) {
@@ -920,8 +964,13 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     }
     if (read_back) {
         // the scale is a host value in this interface: the call completes before returning it
-        HIP_TRY(hipMemcpyAsync(scale, dscale, 4, hipMemcpyDeviceToHost, c.stream));
-        HIP_TRY(hipStreamSynchronize(c.stream));
+        if (arch == AMD_GFX950) {
+            HIP_TRY(hipStreamSynchronize(c.stream));  // host-pointer mode: the copy of the result must have landed
+        }
+        EE te = take_scale(c, scale);
+        if (te != SUCCESS) {
+            return te;
+        }
     } else if (arch == AMD_GFX950) {
         HIP_TRY(hipStreamSynchronize(c.stream));
     }
@@ -1206,11 +1255,14 @@ static EE fc_device(U32 M, U32 K, U32 N, const void *input, F32 scaleI, DataForm
     }
     e = SUCCESS;
     if (cdt != odt) {  // :477-486 -- dynamic requantisation of the int32 result
-        float *dscale = (float *)(c.ws + kWsWords);
+        arm_scale(c);
         HIP_TRY(launch_absmax_i32((const int32_t *)dst, M * N, c.ws, c.stream));
-        HIP_TRY(launch_requant_i32((const int32_t *)dst, M * N, output, 1, c.ws, *outputScale, scaleO, dscale, c.stream));
-        HIP_TRY(hipMemcpyAsync(outputScale, dscale, 4, hipMemcpyDeviceToHost, c.stream));
-        HIP_TRY(hipStreamSynchronize(c.stream));  // the output scale is a host value in this interface
+        HIP_TRY(launch_requant_i32((const int32_t *)dst, M * N, output, 1, c.ws, *outputScale, scaleO, c.hscale_dev,
+            c.stream));
+        EE te = take_scale(c, outputScale);  // the output scale is a host value in this interface
+        if (te != SUCCESS) {
+            return te;
+        }
     } else if (odt == DT_F32 || odt == DT_I32) {
         *outputScale = scaleO;
     }
@@ -1445,17 +1497,15 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // written and read back) never exists, which is worth more than the repeated matrix work.
     g.C = nullptr;
     g.conv.absmax = c.ws;
-    float *dscale = (float *)(c.ws + kWsWords);
     HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
     HIP_TRY(launch_conv_u8s8(g, c.stream));
     g.C = output;
     g.epi.mode = EPI_U8;
     g.conv.scaleO = scaleO;
-    g.conv.dscale_out = dscale;
+    g.conv.dscale_out = c.hscale_dev;  // the new output scale goes straight into pinned host memory
+    arm_scale(c);
     HIP_TRY(launch_conv_u8s8(g, c.stream));
-    HIP_TRY(hipMemcpyAsync(&scale[1], dscale, 4, hipMemcpyDeviceToHost, c.stream));
-    HIP_TRY(hipStreamSynchronize(c.stream));
-    return SUCCESS;
+    return take_scale(c, &scale[1]);
 }
 
 }  // namespace

@@ -10,7 +10,10 @@
  *                      GPU, runs, copies results back and returns when they are in place.
  *   AMD_GFX950_DEVICE  all data pointers (matrices, vectors, tmp, results) are DEVICE pointers,
  *                      4-byte aligned; work is enqueued on the library stream and the call
- *                      returns without waiting. TensorDesc and `scale` arguments stay on the host.
+ *                      returns without waiting. TensorDesc and `scale` arguments stay on the host:
+ *                      a call that computes a scale and returns it through such a pointer (dynamic
+ *                      quantisation, u8 results with a dynamic output scale) returns as soon as that
+ *                      scale has reached the host; its tensors follow in stream order.
  * Errors come back as Bolt's EE codes; nothing here calls exit().
  */
 #ifndef BOLT_GFX950_H
