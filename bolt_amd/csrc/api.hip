@@ -65,6 +65,9 @@ EE fail(EE code, const char *what, hipError_t he = hipSuccess)
 // 1-bit convolution: 2 = matrix cores with E2M1 operands where the shape has that kernel, else int8 (default);
 // 1 = matrix cores with int8 operands; 0 = vector-ALU xor / popcount route
 int g_bnn_mfma = 2;
+// int8 convolution through the filter-panel kernel: gather from the caller's tensor in place for int32 / fp32 results
+// (1, default) or for every result type (2); 0 = always re-lay the input as a padded s8 image first
+int g_conv_direct = 1;
 
 EE ensure_init()
 {
@@ -360,6 +363,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         g_bnn_mfma = value;
+        return SUCCESS;
+    }
+    if (strcmp(name, "conv_direct") == 0) {
+        if (value < 0 || value > 2) {
+            return NOT_MATCH;
+        }
+        g_conv_direct = value;
         return SUCCESS;
     }
     if (strcmp(name, "conv_panel") == 0) {
@@ -1443,8 +1453,17 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     conv_tmp_layout(s, &offOff);
     U8 *t = (U8 *)tmp;
     const F32 scaleO = scale[0] * scale[2];  // convolution_direct.cpp:2687
-    HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
-        s.pr, (int8_t *)t, c.stream));
+    // The filter-panel kernel (few output channels, short K) gathers from the caller's tensor itself when the channel
+    // count is a multiple of 16; every other shape first re-lays the input as a zero-padded s8 image in tmp. The
+    // in-place gather costs the kernel about as much as half a padding pass (bounds tests, and two 8-byte loads per
+    // fragment from NCHWC8), so by default (1) it is taken where the convolution runs once -- int32 and fp32
+    // results -- and not for u8 results, whose two passes share one padded image; 2 takes it always.
+    const bool direct = g_conv_direct && (g_conv_direct == 2 || odt != DT_U8_Q) && conv_panel_ok(s.oc, s.Kp) &&
+        s.ic % 16 == 0 && (((uintptr_t)input) & 15) == 0;
+    if (!direct) {
+        HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
+            s.pr, (int8_t *)t, c.stream));
+    }
     // filter blob = [offsetC oc*4][packed matrix] (convolution_transform.cpp:36-44 keeps the vector in front)
     const int32_t *offC = (const int32_t *)filter;
     const int8_t *mat = (const int8_t *)filter + (size_t)s.oc * 4;
@@ -1452,7 +1471,15 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // it owns: no separate launch
     GemmArgs g;
     memset(&g, 0, sizeof(g));
-    g.A = (const uint8_t *)t;
+    g.A = direct ? (const uint8_t *)input : (const uint8_t *)t;
+    if (direct) {
+        g.conv.in_c = idf == DF_NCHWC16 ? 16 : 8;
+        g.conv.H = s.ih;
+        g.conv.W = s.iw;
+        g.conv.IC = s.ic;
+        g.conv.pt = s.pt;
+        g.conv.pl = s.pl;
+    }
     g.Bp = mat;
     g.M = s.n * s.oh * s.ow;
     g.N = s.oc;

@@ -1187,7 +1187,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 // straight into registers three K tiles ahead (the compiler tracks those loads), reads the four B
 // fragments of a tile from LDS and issues TM x 4 MFMAs. LDS traffic is a third of the shared
 // pipeline's and there is no barrier inside the K loop.
-template <int TM>
+//
+// DIRECT: A is the caller's u8 tensor (NCHWC8 or NCHWC16) instead of the padded s8 image, so no padding pass runs
+// before the kernel. A lane's 16 channels of a tap are one 16-byte load (NCHWC16) or two 8-byte loads from
+// neighbouring channel blocks (NCHWC8); taps that fall outside the image, and the chunks that pad K to 64, read a
+// constant block of 0x80 instead, and every fragment is re-biased (^ 0x80) before use, which turns those into the
+// zeros the padded image holds.
+__device__ const uint8_t kConvPad128[16] = {128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128};
+
+template <int TM, bool DIRECT>
 __global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -1207,20 +1215,48 @@ __global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(smem + f * 1024), 16, 0, 0);
     }
 
-    const uint32_t cpc = a.conv.ICp / 16;  // 16-channel planes of the padded image
-    uint32_t off[TM];
+    const uint32_t cpc = a.conv.ICp / 16;  // 16-channel planes of the image
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+    uint32_t off[TM];   // padded image: byte offset of the pixel's receptive field; DIRECT: of pixel (iy0, ix0), may be "negative"
+    int32_t iy0[TM], ix0[TM];  // DIRECT: input row / column of tap (0, 0)
+    const uint32_t ic_bytes = DIRECT ? a.conv.in_c : 16;  // bytes per pixel inside a channel block
 #pragma unroll
     for (int x = 0; x < TM; ++x) {
         uint32_t row = m0 + (wave * TM + x) * 16 + i;
         row = row < a.M ? row : a.M - 1;
         const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
         const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
-        off[x] = ((img * cpc * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
+        if (DIRECT) {
+            iy0[x] = (int32_t)(oy * a.conv.sh) - (int32_t)a.conv.pt;
+            ix0[x] = (int32_t)(ox * a.conv.sw) - (int32_t)a.conv.pl;
+            off[x] = img * a.conv.IC * a.conv.H * a.conv.W +
+                (uint32_t)(iy0[x] * (int32_t)a.conv.W + ix0[x]) * ic_bytes;  // wraps for border pixels; used only when in range
+        } else {
+            off[x] = ((img * cpc * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
+        }
     }
     // this lane's K-group g covers 16-channel chunk 4 * tile + g; its (kh, kw, c16) is stepped in registers
     uint32_t c16 = g % cpc, kw = (g / cpc) % a.conv.fw, kh = (g / cpc) / a.conv.fw, at = 0;  // at: tile the walk points to
     auto tap_offset = [&]() -> uint32_t {
+        if (DIRECT) {  // channel block(s) of chunk c16, then the tap's row / column inside the plane
+            return ((16 / ic_bytes) * c16 * a.conv.H * a.conv.W + kh * a.conv.dh * a.conv.W + kw * a.conv.dw) * ic_bytes;
+        }
         return (kh < a.conv.fh) ? ((c16 * a.conv.Hp + kh * a.conv.dh) * a.conv.Wp + kw * a.conv.dw) * 16 : 0u;
+    };
+    // one fragment: the lane's 16 channels of pixel x at the current tap
+    auto gather = [&](int x, uint32_t o) -> v4i {
+        if (!DIRECT) {
+            return *(const v4i *)(a.A + off[x] + o);
+        }
+        const uint32_t iy = (uint32_t)(iy0[x] + (int32_t)(kh * a.conv.dh)), ix = (uint32_t)(ix0[x] + (int32_t)(kw * a.conv.dw));
+        const bool ok = kh < a.conv.fh && iy < a.conv.H && ix < a.conv.W;
+        const uint8_t *p = ok ? a.A + (uint32_t)(off[x] + o) : kConvPad128;
+        if (a.conv.in_c == 16) {
+            return *(const v4i *)p;
+        }
+        const uint8_t *p2 = ok ? p + a.conv.H * a.conv.W * 8 : kConvPad128;  // the next block of 8 channels
+        const v2i lo = *(const v2i *)p, hi = *(const v2i *)p2;
+        return (v4i){lo.x, lo.y, hi.x, hi.y};
     };
     auto advance = [&]() {
         if (at + 1 < ksteps) {  // past the last tile the walk stays put: the refetch is never used
@@ -1244,7 +1280,7 @@ __global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
         const uint32_t o = tap_offset();
 #pragma unroll
         for (int x = 0; x < TM; ++x) {
-            fa[s][x] = *(const v4i *)(a.A + off[x] + o);
+            fa[s][x] = gather(x, o);
         }
         advance();
     }
@@ -1273,15 +1309,16 @@ __global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
                 }
 #pragma unroll
                 for (int x = 0; x < TM; ++x) {
+                    const v4i fx = DIRECT ? (fa[u][x] ^ flip) : fa[u][x];
 #pragma unroll
                     for (int y = 0; y < 4; ++y) {
-                        acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fa[u][x], acc[x][y], 0, 0, 0);
+                        acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fx, acc[x][y], 0, 0, 0);
                     }
                 }
                 const uint32_t o = tap_offset();
 #pragma unroll
                 for (int x = 0; x < TM; ++x) {
-                    fa[u][x] = *(const v4i *)(a.A + off[x] + o);
+                    fa[u][x] = gather(x, o);
                 }
                 advance();
             }
@@ -1435,34 +1472,48 @@ bool conv_fp4_ok(uint32_t M, uint32_t N)
     return N >= 256 && (uint64_t)((M + 255) / 256) * ((N + 255) / 256) >= 128;
 }
 
+bool conv_panel_ok(uint32_t N, uint32_t K)
+{
+    return N <= 64 && K % 64 == 0 && K <= 1024 && g_conv_panel != 0;
+}
+
 // Implicit-GEMM convolution: same pipeline, A rows are output pixels gathered from the padded image.
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
 {
     if (a.M == 0 || a.N == 0) {
         return hipSuccess;
     }
-    if (a.N <= 64 && a.K % 64 == 0 && a.K <= 1024 && g_conv_panel) {
+    if (conv_panel_ok(a.N, a.K)) {
         // one filter panel, small enough to sit in LDS: no barrier in the K loop (see the kernel)
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void *)conv_u8s8_panel_kernel<2>,
-                hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-            if (e == hipSuccess) {
-                e = hipFuncSetAttribute((const void *)conv_u8s8_panel_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                    65536);
-            }
-            if (e != hipSuccess) {
-                return e;
+            const void *kerns[4] = {(const void *)conv_u8s8_panel_kernel<2, false>, (const void *)conv_u8s8_panel_kernel<4, false>,
+                (const void *)conv_u8s8_panel_kernel<2, true>, (const void *)conv_u8s8_panel_kernel<4, true>};
+            for (const void *k : kerns) {
+                hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+                if (e != hipSuccess) {
+                    return e;
+                }
             }
             attr_set = true;
         }
         const uint32_t lds = a.K * 64;
+        const bool direct = a.conv.in_c != 0;
         if (g_conv_panel == 2) {
-            hipLaunchKernelGGL(conv_u8s8_panel_kernel<2>, dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+            if (direct) {
+                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, true>), dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+            } else {
+                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, false>), dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+            }
+        } else if (direct) {
+            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, true>), dim3((a.M + 255) / 256), dim3(256), lds, st, a);
         } else {
-            hipLaunchKernelGGL(conv_u8s8_panel_kernel<4>, dim3((a.M + 255) / 256), dim3(256), lds, st, a);
+            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, false>), dim3((a.M + 255) / 256), dim3(256), lds, st, a);
         }
         return hipGetLastError();
+    }
+    if (a.conv.in_c != 0) {
+        return hipErrorInvalidValue;  // only the filter-panel kernel gathers from the caller's tensor
     }
     if (a.N <= 64) {
         // Few output channels: nowhere near MFMA-bound, the time is load latency, so what matters is

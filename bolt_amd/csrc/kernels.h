@@ -47,6 +47,10 @@ struct ConvGeom {
     uint32_t Hp = 0, Wp = 0, ICp = 0;      // padded image height / width, channels rounded up to 16
     uint32_t fh = 0, fw = 0, dh = 0, dw = 0;   // filter taps and dilation: K runs over (kh, kw, c) in 16-channel chunks
     uint32_t out_c = 0;            // channel block of the output layout: 16 (NCHWC16) or 8 (NCHWC8)
+    // in_c = 0: A is the padded s8 image in planes of 16 channels (conv_pad's output). in_c = 8 / 16: A is the
+    // caller's u8 tensor itself (NCHWC8 / NCHWC16, IC % 16 == 0), gathered in place by the filter-panel kernel:
+    // H x W pixels per plane, pt / pl rows / columns of padding above / left of it
+    uint32_t in_c = 0, H = 0, W = 0, IC = 0, pt = 0, pl = 0;
     int relu = 0;
     const float *eltwise = nullptr;      // optional fp32 tensor added before the ReLU (fp32 output only)
     uint32_t *absmax = nullptr;          // scratch slots: int32 mode folds max |acc| into them (C may then be null:
@@ -75,7 +79,9 @@ struct GemmArgs {
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
 // A = padded s8 image, M = n * OH * OW output pixels, N = output channels, K = fh * fw * ICp
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
-bool conv_fp4_ok(uint32_t M, uint32_t N);  // whether launch_conv_u8s8 has an fp4 kernel for this shape
+bool conv_fp4_ok(uint32_t M, uint32_t N);
+// whether launch_conv_u8s8 would run the filter-panel kernel for this shape (the one that can gather from the caller's tensor)
+bool conv_panel_ok(uint32_t N, uint32_t K);  // whether launch_conv_u8s8 has an fp4 kernel for this shape
 void conv_force_panel(int v);  // 0: shared-pipeline kernel only; 2 / 4: panel kernel with 32 / 64 pixels per wave
 // tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
 void gemm_force_tile(int tile);

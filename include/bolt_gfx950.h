@@ -45,7 +45,10 @@ const char *bolt_gfx950_last_error(void);
  * K % 128 == 0, else it runs as 11), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
  * the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
  * K <= 1024 uses: 4 (default) / 2 the filter-panel-in-LDS kernel with 64 / 32 pixels per wave, 0 the
- * shared-pipeline kernel. "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
+ * shared-pipeline kernel. "conv_direct": whether that filter-panel kernel gathers from the caller's
+ * u8 tensor in place when the channel count is a multiple of 16: 1 (default) for int32 and fp32
+ * results, 2 for u8 results as well, 0 never (the input is first re-laid as a padded s8 image).
+ * "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
  * with its operands expanded to E2M1 pairs (v_mfma_scale_f32_16x16x128_f8f6f4) where the shape has
  * that kernel (256+ output channels, 128+ tiles of 256 pixels) and as 1 otherwise; 1 on the int8
  * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount). Every variant

@@ -61,17 +61,21 @@ def test_conv_int8(torch_mod, oracle, co, device_mode, case, relu):
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (case, odt, out_c)
 
 
-@pytest.mark.parametrize("panel", [0, 2, 4])
-def test_conv_int8_every_kernel(torch_mod, oracle, co, panel):
+@pytest.mark.parametrize("panel,direct", [(0, 0), (2, 0), (2, 2), (4, 0), (4, 2)])
+def test_conv_int8_every_kernel(torch_mod, oracle, co, panel, direct):
     """Convolutions with up to 64 output channels and K <= 1024 have three kernels to choose from: the shared
-    LDS pipeline (0) and the filter-panel kernel with 32 (2) or 64 (4) pixels per wave. Each is forced in turn
-    on shapes with ragged pixel counts, channel tails, strides and a 5 x 5 filter."""
+    LDS pipeline (0) and the filter-panel kernel with 32 (2) or 64 (4) pixels per wave; the filter-panel kernel
+    either reads the padded s8 image (direct = 0) or, when the channel count is a multiple of 16, gathers from
+    the caller's u8 tensor in place (direct = 2: for every result type). Each is forced in turn on shapes with ragged pixel counts,
+    channel tails, strides, a 5 x 5 filter, no padding, and a K that is padded up to 64."""
     L = capi.lib()
     try:
         capi.check(L.bolt_gfx950_set_option(b"conv_panel", panel), "set_option")
+        capi.check(L.bolt_gfx950_set_option(b"conv_direct", direct), "set_option")
         for case in [(2, 24, 6, 5, 24, 5, 5, 1, 2), (3, 16, 10, 9, 40, 3, 3, 1, 1), (1, 64, 56, 56, 64, 3, 3, 1, 1),
-                     (2, 8, 9, 7, 8, 3, 3, 2, 1), (5, 32, 13, 13, 64, 1, 1, 1, 0)]:
-            print("conv kernel", panel, case, flush=True)
+                     (2, 8, 9, 7, 8, 3, 3, 2, 1), (5, 32, 13, 13, 64, 1, 1, 1, 0), (2, 16, 9, 7, 24, 3, 3, 2, 1),
+                     (2, 32, 6, 5, 24, 5, 5, 1, 2), (1, 16, 5, 4, 8, 3, 3, 1, 0), (3, 48, 7, 11, 40, 3, 3, 1, 1)]:
+            print("conv kernel", panel, direct, case, flush=True)
             n, ic, ih, iw, oc, fh, fw, stride, pad = case
             xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, sum(case) + panel)
             for odt in (DT_U8_Q, DT_F32, DT_I32):
@@ -83,9 +87,11 @@ def test_conv_int8_every_kernel(torch_mod, oracle, co, panel):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (panel, case, odt)
     finally:
         capi.check(L.bolt_gfx950_set_option(b"conv_panel", 4), "set_option")
+        capi.check(L.bolt_gfx950_set_option(b"conv_direct", 1), "set_option")
 
 
-def test_conv_int8_nchwc16_input_and_eltwise(torch_mod, oracle, co):
+@pytest.mark.parametrize("direct", [2, 0])
+def test_conv_int8_nchwc16_input_and_eltwise(torch_mod, oracle, co, direct):
     case = (2, 32, 7, 6, 48, 3, 3, 1, 1)
     n, ic, ih, iw, oc, fh, fw, stride, pad = case
     xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, 9)
@@ -95,9 +101,14 @@ def test_conv_int8_nchwc16_input_and_eltwise(torch_mod, oracle, co):
     # same activations handed over as NCHWC16
     x_nchw = xq.reshape(n, ic // 8, ih, iw, 8).transpose(0, 1, 4, 2, 3).reshape(n, ic, ih, iw)
     x16 = to_nchwc(x_nchw, 16)
-    for mode in (False, True):
-        got = run_conv(torch_mod, mode, x16, DF_NCHWC16, W, bias, [sI, -1.0, sF], case, True, DT_F32, eltwise=elt)
-        assert np.array_equal(got.view(np.int32), want.view(np.int32))
+    L = capi.lib()
+    try:
+        capi.check(L.bolt_gfx950_set_option(b"conv_direct", direct), "set_option")
+        for mode in (False, True):
+            got = run_conv(torch_mod, mode, x16, DF_NCHWC16, W, bias, [sI, -1.0, sF], case, True, DT_F32, eltwise=elt)
+            assert np.array_equal(got.view(np.int32), want.view(np.int32))
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"conv_direct", 1), "set_option")
 
 
 def test_conv_config3_single_image(torch_mod, oracle, co):
