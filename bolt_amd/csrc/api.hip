@@ -1462,7 +1462,7 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
         s.ic % 16 == 0 && (((uintptr_t)input) & 15) == 0;
     if (!direct) {
         HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
-            s.pr, (int8_t *)t, c.stream));
+            s.pr, (int8_t *)t, c.stream, odt == DT_U8_Q ? c.ws : nullptr));  // u8 results: also clears the max slots
     }
     // filter blob = [offsetC oc*4][packed matrix] (convolution_transform.cpp:36-44 keeps the vector in front)
     const int32_t *offC = (const int32_t *)filter;
@@ -1524,7 +1524,9 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // written and read back) never exists, which is worth more than the repeated matrix work.
     g.C = nullptr;
     g.conv.absmax = c.ws;
-    HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
+    if (direct) {  // otherwise the padding kernel has cleared the slots
+        HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
+    }
     HIP_TRY(launch_conv_u8s8(g, c.stream));
     g.C = output;
     g.epi.mode = EPI_U8;

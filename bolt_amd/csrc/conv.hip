@@ -27,8 +27,13 @@ namespace bg {
 // consecutive pixels, 8 or 16 contiguous bytes each -- re-biases them to s8 and writes 16 contiguous
 // bytes. Border pixels and the channel tail are zero.
 __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict__ in, uint32_t N, uint32_t C, uint32_t H,
-    uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out)
+    uint32_t W, uint32_t cx, uint32_t pt, uint32_t pl, uint32_t Hp, uint32_t Wp, uint32_t ICp, int8_t *__restrict__ out,
+    uint32_t *__restrict__ clear_ws)
 {
+    // optional: zero the scratch slots that the convolution after this kernel folds max|acc| into (saves a launch)
+    if (clear_ws && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < kWsSlots) {
+        clear_ws[threadIdx.x * kWsStride] = 0;
+    }
     const uint32_t planes = ICp / 16;
     const uint32_t c16 = blockIdx.x % planes, n = blockIdx.x / planes;
     const uint32_t npix = Hp * Wp;
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const uint8_t *__restrict
 }
 
 hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
-    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st)
+    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st, uint32_t *clear_ws)
 {
     const uint32_t Hp = H + pt + pb, Wp = W + pl + pr, ICp = align_up(C, 16);
     const uint64_t np = (uint64_t)N * (ICp / 16), npix = (uint64_t)Hp * Wp;
@@ -80,7 +85,7 @@ hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H
         return hipErrorInvalidValue;
     }
     hipLaunchKernelGGL(conv_pad_kernel, dim3((uint32_t)np, (uint32_t)((npix + 1023) / 1024)), dim3(256), 0, st, in, N, C, H, W,
-        cx, pt, pl, Hp, Wp, ICp, out);
+        cx, pt, pl, Hp, Wp, ICp, out, clear_ws);
     return hipGetLastError();
 }
 

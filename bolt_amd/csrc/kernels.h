@@ -89,7 +89,7 @@ void gemm_force_tile(int tile);
 // ---- convolution helpers (conv.hip) -------------------------------------------------------------
 // u8 NCHWC8 (cx = 8) / NCHWC16 (cx = 16) -> s8 (x - 128), zero padded, [n][H+pt+pb][W+pl+pr][ALIGN(C,16)]
 hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H, uint32_t W, uint32_t cx, uint32_t pt,
-    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st);
+    uint32_t pb, uint32_t pl, uint32_t pr, int8_t *out, hipStream_t st, uint32_t *clear_ws = nullptr);
 // s8 NCHW filter -> offsetC[OC] and the fragment-layout matrix over K = (kh, kw, c)
 hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, uint32_t fh, uint32_t fw, int32_t *offsetC,
     int8_t *dst, hipStream_t st);
