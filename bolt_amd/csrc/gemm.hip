@@ -667,6 +667,24 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_tiled_kernel(GemmArgs a
 // Rows / column blocks past the matrix edge load a clamped (valid) address; what they produce is
 // never stored. Workgroup ids are re-mapped so that each XCD (ids are dealt round-robin over the 8
 // XCDs) works on one contiguous band of output tiles and re-uses its A rows / B columns in its L2.
+// u8 convolution, second pass: the tensor-wide output scale follows from the maximum the first pass left in the
+// scratch slots, and the host is waiting for it. The first wave of the first workgroup publishes it before any
+// other work and clears the pointer in this workgroup's copy of the arguments, so that the epilogue (which needs
+// the same factor for its own arithmetic) does not store it a second time.
+__device__ __forceinline__ void conv_publish_scale(GemmArgs &a, uint32_t wave)
+{
+    if (a.epi.mode == EPI_U8 && a.conv.dscale_out) {
+        if (blockIdx.x == 0 && wave == 0) {
+            const int mx = ws_read_max(a.conv.absmax);
+            const float factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
+            if ((threadIdx.x & 63) == 0) {
+                *a.conv.dscale_out = a.conv.scaleO * factor;
+            }
+        }
+        a.conv.dscale_out = nullptr;
+    }
+}
+
 template <int WM, int WN, int TM, int TN, int STAGES>
 struct GemmDma {
     static constexpr int kBM = WM * TM * 16;
@@ -700,6 +718,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it scalar
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
+    if (CONV) {
+        conv_publish_scale(a, wave);
+    }
 
     // XCD-aware tile order: hardware deals linear workgroup ids round-robin to the 8 XCDs; give XCD x
     // the x-th contiguous eighth of the tile sequence, and walk that sequence in bands of 8 M-tiles.
@@ -1206,6 +1227,7 @@ __global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
     const uint32_t m0 = blockIdx.x * (4 * TM * 16);
     const uint32_t K = a.K, ksteps = K / 64;
     const uint32_t nblocks = align_up(a.N, 16) >> 4;
+    conv_publish_scale(a, wave);
 
     // the filter panel: fragment (tile t, column block y) at smem + (4 t + y) KiB
     for (uint32_t f = wave; f < 4 * ksteps; f += 4) {
