@@ -68,7 +68,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v4i &acc, ui
 // General kernel: any M, N, K, either A orientation, no alignment assumptions. One wave owns a
 // 16 x 64 strip of C (four MFMA tiles sharing the A fragment); operands go straight from global
 // memory / L2 to registers.
-__global__ __launch_bounds__(256) void gemm_u8s8_general_kernel(GemmArgs a)
+__global__ __launch_bounds__(256, 2) void gemm_u8s8_general_kernel(GemmArgs a)
 {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t i = lane & 15, g = lane >> 4;
@@ -538,7 +538,7 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
 }
 
 template <int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_tiled_kernel(GemmArgs a)
+__global__ __launch_bounds__(WM *WN * 64, (TM * TN >= 64) ? 1 : 2) void gemm_u8s8_tiled_kernel(GemmArgs a)
 {
     using T = GemmTile<WM, WN, TM, TN>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -710,7 +710,9 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 // products are formed by v_mfma_scale_f32_16x16x128_f8f6f4 -- twice the K per instruction at the same rate, fp32
 // accumulation that is exact for these integers; the accumulators are converted to int32 before the epilogue.
 template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false, bool FP4 = false>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
+// Two waves per SIMD are asked for also where a workgroup has four waves: with a budget of 512 registers per lane
+// the compiler keeps the accumulators in AGPRs and spends dozens of v_accvgpr moves per K tile on shuffling them.
+__global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -1217,7 +1219,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_u8s8_dma_kernel(GemmArgs a)
 __device__ const uint8_t kConvPad128[16] = {128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128};
 
 template <int TM, bool DIRECT>
-__global__ __launch_bounds__(256) void conv_u8s8_panel_kernel(GemmArgs a)
+__global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int P = 3;  // K tiles of A in flight per wave
