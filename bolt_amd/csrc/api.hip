@@ -2366,8 +2366,9 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st));
     HIP_TRY(launch_quantize_f32(h1, T * H, xq, 1, ws2, 0.0f, nullptr, 0, sc + 2, st));
     HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
-    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st));
-    HIP_TRY(launch_quantize_f32(f, T * F, xq, 1, ws3, 0.0f, nullptr, 0, sc + 3, st));
+    // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads
+    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st, false));
+    HIP_TRY(launch_quantize_f32(f, T * F, xq, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 1));
     HIP_TRY(gemm(xq, L.w2, H, F, sc + 3, L.s2, L.b2, o));
     HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st));
     return SUCCESS;

@@ -153,6 +153,15 @@ __device__ __forceinline__ int wave_reduce_max_i(int v)
     return v;
 }
 
+// tanh-form GELU: x * 0.5 * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3))), with tanh(u/2) written as 1 - 2 / (1 + e^u)
+__device__ __forceinline__ float gelu_tanh(float x)
+{
+    const float c0 = 1.5957691216057308f;  // 2 * sqrt(2 / pi)
+    const float u = (c0 * x) * __builtin_fmaf(0.044715f, x * x, 1.0f);
+    const float e = __expf(u);
+    return (2.0f - 2.0f / (1.0f + e)) * (0.5f * x);
+}
+
 // ---- tensor-wide max through device scratch words --------------------------------------------------
 // Atomics from many workgroups to ONE address serialise at the memory side (the eight XCDs' L2s
 // are not coherent with each other), ~10 ns apiece. The running max is therefore spread over

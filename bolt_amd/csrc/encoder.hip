@@ -267,15 +267,10 @@ hipError_t launch_add_layernorm(const float *a, const float *b, const float *gam
     return hipGetLastError();
 }
 
-// ---- GELU (in place) ----------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_tanh(float x)
-{
-    const float c0 = 1.5957691216057308f;  // 2 * sqrt(2 / pi)
-    const float u = (c0 * x) * __builtin_fmaf(0.044715f, x * x, 1.0f);
-    const float e = __expf(u);
-    return (2.0f - 2.0f / (1.0f + e)) * (0.5f * x);
-}
-
+// ---- GELU (in place, or only its max|.|) ----------------------------------------------------------------
+// STORE = false leaves x as it is and only folds max|gelu(x)| into ws: the quantiser that follows applies the
+// same gelu_tanh to what it reads, so the activated tensor is never written.
+template <bool STORE>
 __global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, uint32_t n4, uint32_t *ws)
 {
     __shared__ int red[4];
@@ -289,7 +284,9 @@ __global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, ui
         v.y = gelu_tanh(v.y);
         v.z = gelu_tanh(v.z);
         v.w = gelu_tanh(v.w);
-        x4[i] = v;
+        if (STORE) {
+            x4[i] = v;
+        }
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
     }
     if (ws) {
@@ -297,7 +294,7 @@ __global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, ui
     }
 }
 
-hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st)
+hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store)
 {
     if (n == 0) {
         return hipSuccess;
@@ -308,7 +305,11 @@ hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st)
     const uint32_t n4 = (uint32_t)(n / 4);
     uint32_t blocks = (n4 + 255) / 256;
     blocks = blocks > 4096 ? 4096 : blocks;
-    hipLaunchKernelGGL(gelu_f32_kernel, dim3(blocks), dim3(256), 0, st, x, n4, ws);
+    if (store) {
+        hipLaunchKernelGGL(gelu_f32_kernel<true>, dim3(blocks), dim3(256), 0, st, x, n4, ws);
+    } else {
+        hipLaunchKernelGGL(gelu_f32_kernel<false>, dim3(blocks), dim3(256), 0, st, x, n4, ws);
+    }
     return hipGetLastError();
 }
 

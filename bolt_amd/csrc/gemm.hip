@@ -538,7 +538,7 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
 }
 
 template <int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(WM *WN * 64, (TM * TN >= 64) ? 1 : 2) void gemm_u8s8_tiled_kernel(GemmArgs a)
+__global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_tiled_kernel(GemmArgs a)
 {
     using T = GemmTile<WM, WN, TM, TN>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -1602,8 +1602,6 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
         tile = 11;
     }
     switch (tile) {
-        case 1:
-            return launch_tiled<2, 2, 8, 8>(a, st);  // 256 x 256
         case 2:
             return launch_tiled<2, 2, 4, 4>(a, st);  // 128 x 128
         case 7:

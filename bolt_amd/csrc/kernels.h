@@ -129,7 +129,8 @@ hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, ui
 // out = LayerNorm(a + b) (b may be null); H % 4 == 0, H <= 2048
 hipError_t launch_add_layernorm(const float *a, const float *b, const float *gamma, const float *beta, uint32_t rows,
     uint32_t H, float *out, uint32_t *ws, hipStream_t st);
-hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st);
+// store = false: x is left untouched, only max|gelu(x)| is folded into ws (pair it with launch_quantize_f32(..., gelu = 1))
+hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store = true);
 
 // ---- weight pack --------------------------------------------------------------------------------
 // src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].
@@ -146,7 +147,7 @@ hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream
 // the scale used is max(caller's, 127 / max|x|) with max|x| taken from ws[0]. The scale used is
 // written to *ds_out (device) when non-null.
 hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
-    const float *ds_in, int mode, float *ds_out, hipStream_t st);
+    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu = 0);
 hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st);
 // s0 = output scale (< 0: dynamic from ws[0]), s1 = scale of the int32 data; the resulting output
 // scale is written to *ds_out (device) when non-null.

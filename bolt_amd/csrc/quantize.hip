@@ -197,7 +197,8 @@ __device__ __forceinline__ float resolve_scale(float s_in, int mode, const uint3
     return s_in;
 }
 
-template <int TO_U8, int VEC>
+// GELU: quantise gelu_tanh(x) instead of x (the max in ws is then that of the activated values)
+template <int TO_U8, int VEC, int GELU = 0>
 __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restrict__ x, uint32_t n,
     uint8_t *__restrict__ q, const uint32_t *__restrict__ ws, float s_in, const float *ds_in, int mode,
     float *ds_out)  // ds_in may alias ds_out: the resolved scale is a fixed point of resolve_scale
@@ -214,11 +215,21 @@ __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restri
         v4i *q16 = (v4i *)q;
         for (uint32_t i = tid; i < n16; i += stride) {
             v4f a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+            if (GELU) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = gelu_tanh(a[e]);
+                    b[e] = gelu_tanh(b[e]);
+                    c[e] = gelu_tanh(c[e]);
+                    d[e] = gelu_tanh(d[e]);
+                }
+            }
             v4i o = {(int)q4<TO_U8>(a, s), (int)q4<TO_U8>(b, s), (int)q4<TO_U8>(c, s), (int)q4<TO_U8>(d, s)};
             q16[i] = o;
         }
         for (uint32_t i = n16 * 16 + tid; i < n; i += stride) {
-            q[i] = (uint8_t)(TO_U8 ? q_u8(x[i], s) : q_i8(x[i], s));
+            const float v = GELU ? gelu_tanh(x[i]) : x[i];
+            q[i] = (uint8_t)(TO_U8 ? q_u8(v, s) : q_i8(v, s));
         }
     } else {
         for (uint32_t i = tid; i < n; i += stride) {
@@ -228,10 +239,18 @@ __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restri
 }
 
 hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
-    const float *ds_in, int mode, float *ds_out, hipStream_t st)
+    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu)
 {
     const bool vec = (((uintptr_t)x | (uintptr_t)q) & 15) == 0;
     const uint32_t blocks = grid_for(n, vec ? 16 : 1, 256, 8192);
+    if (gelu) {
+        if (!to_u8 || !vec) {
+            return hipErrorInvalidValue;  // the fused form exists for aligned u8 output only
+        }
+        hipLaunchKernelGGL((quantize_f32_kernel<1, 1, 1>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s_in, ds_in,
+            mode, ds_out);
+        return hipGetLastError();
+    }
 #define BG_LAUNCH_Q(U, V)                                                                                        \
     hipLaunchKernelGGL((quantize_f32_kernel<U, V>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s_in, \
         ds_in, mode, ds_out)

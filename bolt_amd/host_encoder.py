@@ -51,6 +51,6 @@ class EncoderLayer:
         offs = (C.c_size_t * 6)()
         check(lib().bolt_gfx950_encoder_layer_int8_workspace_layout(C.byref(self.L), offs), "encoder_workspace_layout")
         T, H, F = self.tokens, self.hidden, self.L.ffn
-        shapes = (("qkv", 3 * H), ("ctx", H), ("attn_out", H), ("h1", H), ("ffn_act", F), ("ffn_out", H))
+        shapes = (("qkv", 3 * H), ("ctx", H), ("attn_out", H), ("h1", H), ("ffn_pre", F), ("ffn_out", H))
         return {name: self.workspace[offs[i]:offs[i] + T * w * 4].view(self.torch.float32).view(T, w)
                 for i, (name, w) in enumerate(shapes)}

@@ -38,8 +38,8 @@ EE bolt_gfx950_init(void);
 EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
-/* Tuning / test knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 1-2 the
- * register-staged 256x256 / 128x128 tiled kernels (need K % 16 == 0), 7 / 10 / 11 the LDS-DMA
+/* Tuning / test knobs. "gemm_tile": -1 shape heuristic (default), 0 general kernel, 2 the
+ * register-staged 128x128 tiled kernel (needs K % 16 == 0), 7 / 10 / 11 the LDS-DMA
  * kernels (256x256 fragment-prefetch, 128x128 fragment-prefetch, 256x256 ping-pong; need
  * K % 64 == 0), 12 the 256x256 ping-pong kernel that requests A in whole 128-byte lines (needs
  * K % 128 == 0, else it runs as 11), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
@@ -227,8 +227,9 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     size_t workspaceBytes);
 /* Inspection hook: byte offsets inside `workspace` of the fp32 intermediates a call leaves behind, in
  * this order: qkv [T, 3*hidden], attention context [T, hidden], attention output projection
- * [T, hidden], first LayerNorm output [T, hidden], FFN activation after GELU [T, ffn], FFN output
- * [T, hidden]. */
+ * [T, hidden], first LayerNorm output [T, hidden], first FFN product before GELU [T, ffn] (the activated
+ * values are never stored: the quantiser ahead of the second FFN product applies GELU to what it
+ * reads), FFN output [T, hidden]. */
 EE bolt_gfx950_encoder_layer_int8_workspace_layout(const BoltEncoderLayerInt8 *layer, size_t *offsets);
 
 /* The layer's fp32 pieces on their own (device pointers, asynchronous):
