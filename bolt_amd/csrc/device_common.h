@@ -159,7 +159,7 @@ __device__ __forceinline__ float gelu_tanh(float x)
     const float c0 = 1.5957691216057308f;  // 2 * sqrt(2 / pi)
     const float u = (c0 * x) * __builtin_fmaf(0.044715f, x * x, 1.0f);
     const float e = __expf(u);
-    return (2.0f - 2.0f / (1.0f + e)) * (0.5f * x);
+    return (2.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e)) * (0.5f * x);  // v_rcp_f32: 1 ulp, far inside the layer's tolerance
 }
 
 // ---- tensor-wide max through device scratch words --------------------------------------------------
