@@ -27,6 +27,7 @@ struct Ctx {
     // scale through a host pointer read it after the stream has drained: no copy command in between), and
     // the address the device uses for it.
     float *hscale = nullptr, *hscale_dev = nullptr;
+    FusedSync fsync;  // sync area of the one-launch dynamic quantiser
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     struct Buf {
@@ -68,6 +69,9 @@ int g_bnn_mfma = 2;
 // int8 convolution through the filter-panel kernel: gather from the caller's tensor in place for int32 / fp32 results
 // (1, default) or for every result type (2); 0 = always re-lay the input as a padded s8 image first
 int g_conv_direct = 1;
+// dynamic quantisation through the public entry points: 1 = one launch that reads the tensor once where
+// it fits (default), 0 = always the two-pass form (scratch fill, abs-max, quantise)
+int g_quantize_fused = 1;
 
 EE ensure_init()
 {
@@ -84,6 +88,19 @@ EE ensure_init()
     e = hipMalloc((void **)&c.ws, (kWsWords + 64) * sizeof(uint32_t));
     if (e != hipSuccess) {
         return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
+    }
+    {
+        void *p = nullptr;
+        e = hipMalloc(&p, kFusedSyncBytes);
+        if (e == hipSuccess) {
+            e = hipMemset(p, 0, kFusedSyncBytes);
+        }
+        if (e != hipSuccess) {
+            return fail(ALLOC_FAILED, "hipMalloc(quantiser sync area)", e);
+        }
+        c.fsync.slots = (unsigned long long *)p;
+        c.fsync.counter = (uint32_t *)((uint8_t *)p + 64 * 64);
+        c.fsync.release = (unsigned long long *)((uint8_t *)p + 64 * 64 + 64);
     }
     e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
     if (e == hipSuccess) {
@@ -122,6 +139,9 @@ EE take_scale(Ctx &c, float *dst)
     const uint32_t bits = *w;
     if (bits == kScaleUnset) {
         return fail(UNKNOWN, "the kernel did not produce a scale");
+    }
+    if ((bits & 0x7fffffffu) > 0x7f800000u) {  // NaN: the one-launch quantiser gave up waiting for its grid
+        return fail(UNKNOWN, "the quantiser's grid barrier timed out");
     }
     memcpy(dst, &bits, 4);
     return SUCCESS;
@@ -363,6 +383,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         g_bnn_mfma = value;
+        return SUCCESS;
+    }
+    if (strcmp(name, "quantize_fused") == 0) {
+        if (value != 0 && value != 1) {
+            return NOT_MATCH;
+        }
+        g_quantize_fused = value;
         return SUCCESS;
     }
     if (strcmp(name, "conv_direct") == 0) {
@@ -952,21 +979,33 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     arm_scale(c);
     if (f32in) {
         const bool dynamic = (!mode || *scale <= 0);
-        if (dynamic) {
-            HIP_TRY(launch_absmax_f32((const float *)dIn, n, c.ws, c.stream));
+        bool fused = false;
+        if (dynamic && g_quantize_fused) {  // one launch, one read, where the tensor fits a resident grid's registers
+            HIP_TRY(launch_quantize_fused(dIn, n, dOut, 0, qdt == DT_U8_Q, c.fsync, *scale, dscale, c.stream, &fused));
         }
-        HIP_TRY(launch_quantize_f32((const float *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, *scale, nullptr, mode, dscale,
-            c.stream));
+        if (!fused) {
+            if (dynamic) {
+                HIP_TRY(launch_absmax_f32((const float *)dIn, n, c.ws, c.stream));
+            }
+            HIP_TRY(launch_quantize_f32((const float *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, *scale, nullptr, mode, dscale,
+                c.stream));
+        }
         read_back = dynamic;
     } else if (ddt == DT_U8_Q) {
         HIP_TRY(launch_u8_to_i8((const uint8_t *)dIn, n, (int8_t *)dOut, c.stream));
     } else {
         const bool dynamic = (scale[0] < 0 && scale[1] > 0);
-        if (dynamic) {
-            HIP_TRY(launch_absmax_i32((const int32_t *)dIn, n, c.ws, c.stream));
+        bool fused = false;
+        if (dynamic && g_quantize_fused) {
+            HIP_TRY(launch_quantize_fused(dIn, n, dOut, 1, qdt == DT_U8_Q, c.fsync, scale[1], dscale, c.stream, &fused));
         }
-        HIP_TRY(launch_requant_i32((const int32_t *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, scale[0], scale[1], dscale,
-            c.stream));
+        if (!fused) {
+            if (dynamic) {
+                HIP_TRY(launch_absmax_i32((const int32_t *)dIn, n, c.ws, c.stream));
+            }
+            HIP_TRY(launch_requant_i32((const int32_t *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, scale[0], scale[1], dscale,
+                c.stream));
+        }
         read_back = dynamic;
     }
     if (arch == AMD_GFX950 && n) {

@@ -163,6 +163,16 @@ hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *off
     float scaleB, int32_t *out, hipStream_t st);
 hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float rescale, int8_t *out, hipStream_t st);
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
+// One-launch dynamic quantisation (quantize.hip): device sync area and the host's running epoch / arrival target
+struct FusedSync {
+    unsigned long long *slots = nullptr;  // 64 slots, 8 words apart, zeroed once when allocated
+    uint32_t *counter = nullptr;          // arrivals, never reset
+    unsigned long long *release = nullptr;  // 64 words, 8 words apart: (epoch << 32 | max) from the last arrival
+    uint32_t epoch = 0, target = 0;
+};
+constexpr size_t kFusedSyncBytes = 64 * 64 + 64 + 64 * 64;
+hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
+    float *ds_out, hipStream_t st, bool *taken);
 // probe.hip: register-resident int8 MFMA loop, blocks x 8 waves x iters x 32 instructions
 hipError_t launch_mfma_i8_rate(uint32_t blocks, uint32_t iters, int zero, int *sink, hipStream_t st);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]

@@ -327,6 +327,223 @@ hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, 
     return hipGetLastError();
 }
 
+// ---- dynamic quantisation in one launch, one read ----------------------------------------------------
+// The two-pass form reads the tensor twice (max, then quantise) in two launches behind a scratch fill. Here
+// every thread keeps its share of the tensor in registers across a grid-wide barrier: load (up to PER groups
+// of 4 elements per thread), fold max|x| into the sync area, wait until every workgroup has arrived, take
+// the maximum, quantise from the registers, store. The tensor is read once and the call is one launch.
+//
+// The grid is at most two workgroups of 256 threads per CU and never more than the occupancy the runtime reports
+// for the kernel, so every workgroup is running when the first one reaches the barrier; a cooperative launch would have the runtime check that, but costs more than the launches saved.
+// Sync area: 64 slots of (epoch << 32 | max bits), one per 64-byte line, folded with a 64-bit atomic max -- a
+// launch's epoch beats whatever older launches left there, so nothing is ever cleared -- an arrival counter
+// that only grows (the host hands each launch the value it reaches when all of its workgroups have arrived),
+// and 64 release words, one per line. The workgroup that arrives last reads the slots and stores
+// (epoch << 32 | max) into every release word; the others poll the release word of their own line (one
+// thread per workgroup, a dozen pollers per line, sleeping between polls). The poll is bounded: a launch whose
+// bound expires publishes a NaN scale, which the host reports as an error instead of returning garbage.
+constexpr uint32_t kFusedSpinLimit = 1u << 20;  // polls of about a microsecond each: about a second
+
+template <int SRC_I32, int TO_U8, int PER>
+__global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restrict__ xin, uint32_t n, uint8_t *__restrict__ q,
+    unsigned long long *slots, uint32_t *counter, unsigned long long *release, uint32_t epoch, uint32_t target, float s_in,
+    float *ds_out)
+{
+    __shared__ int red[4];
+    __shared__ int bcast[2];
+    const uint32_t n4 = n / 4;
+    const uint32_t tid = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
+    const v4i *x4 = (const v4i *)xin;
+    v4i r[PER];  // lane-contiguous 16-byte loads: a wave's request is 1 KB of whole cache lines
+    int tail = 0;
+    int m = 0;
+    float mf = 0.0f;  // fp32 input: v_max_f32 drops NaNs, as the reference's compare-and-keep does
+#define BG_FOLD(bits)                                                                  \
+    {                                                                                  \
+        int b_ = (bits);                                                               \
+        if (SRC_I32) {                                                                 \
+            int a_ = (b_ == (int)0x80000000) ? b_ : (b_ < 0 ? -b_ : b_); /* vpabsd: |INT32_MIN| stays negative */ \
+            m = a_ > m ? a_ : m;                                                       \
+        } else {                                                                       \
+            mf = fmaxf(mf, fabsf(__int_as_float(b_)));                                 \
+        }                                                                              \
+    }
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const uint32_t u = tid + k * stride;
+        r[k] = (u < n4) ? x4[u] : (v4i){0, 0, 0, 0};
+        BG_FOLD(r[k].x) BG_FOLD(r[k].y) BG_FOLD(r[k].z) BG_FOLD(r[k].w)
+    }
+    if (n4 * 4 + tid < n) {  // fewer than 4 trailing elements, one each for the first threads
+        tail = ((const int *)xin)[n4 * 4 + tid];
+        BG_FOLD(tail)
+    }
+#undef BG_FOLD
+    if (!SRC_I32) {
+        m = __float_as_int(mf);  // non-negative float: integer order == float order
+    }
+    m = wave_reduce_max_i(m);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        red[wave] = m;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w) {
+            m = red[w] > m ? red[w] : m;
+        }
+        const unsigned long long tag = ((unsigned long long)epoch << 32) | (uint32_t)m;
+        atomicMax(slots + (blockIdx.x & 63) * 8, tag);
+        __threadfence();
+        bcast[1] = (atomicAdd(counter, 1u) + 1u == target) ? 2 : 1;  // 2: this workgroup arrived last
+    }
+    __syncthreads();
+    if (bcast[1] == 2) {
+        if (wave == 0) {  // every fold is complete: take the maximum and release the others
+            __threadfence();
+            const unsigned long long t = __hip_atomic_load(slots + lane * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int v = ((uint32_t)(t >> 32) == epoch) ? (int)(uint32_t)t : 0;
+            v = wave_reduce_max_i(v);
+            __hip_atomic_store(release + lane * 8, ((unsigned long long)epoch << 32) | (uint32_t)v, __ATOMIC_RELAXED,
+                __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) {
+                bcast[0] = v;
+            }
+        }
+    } else if (threadIdx.x == 0) {
+        uint32_t spins = 0;
+        unsigned long long t;
+        while ((uint32_t)((t = __hip_atomic_load(release + (blockIdx.x & 63) * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) !=
+            epoch) {
+            __builtin_amdgcn_s_sleep(2);
+            if (++spins > kFusedSpinLimit) {
+                bcast[1] = 0;  // gave up
+                t = 0;
+                break;
+            }
+        }
+        bcast[0] = (int)(uint32_t)t;
+    }
+    __syncthreads();
+    const int gmax = bcast[0];
+    const bool ok = bcast[1] != 0;
+    float s, published;
+    if (SRC_I32) {  // avx512/quantize.cpp:315-416 with scale[0] < 0: r = 127 / max, returned scale = scale[1] * r
+        s = (gmax == 0) ? 1.0f : 127.0f / (float)gmax;
+        published = s_in * s;
+    } else {  // :129-133 / :189-193: max(caller's scale, 127 / max|x|), 127 / 0 replaced by 1
+        const float mx = __int_as_float(gmax);
+        const float dyn = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+        s = (s_in > dyn) ? s_in : dyn;
+        published = s;
+    }
+    if (tid == 0 && ds_out) {
+        *ds_out = ok ? published : __int_as_float(0x7fc00000);
+    }
+#define BG_QF(bits)                                                                                        \
+    ((unsigned)(SRC_I32 ? (TO_U8 ? usat8_u(rne_i32((float)(bits)*s + 128.0f)) : ssat8(rne_i32((float)(bits)*s))) \
+                        : (TO_U8 ? q_u8(__int_as_float(bits), s) : q_i8(__int_as_float(bits), s))) & 0xffu)
+#define BG_QF4(v) ((int)(BG_QF(v.x) | (BG_QF(v.y) << 8) | (BG_QF(v.z) << 16) | (BG_QF(v.w) << 24)))
+    int *q4 = (int *)q;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const uint32_t u = tid + k * stride;
+        if (u < n4) {
+            q4[u] = BG_QF4(r[k]);
+        }
+    }
+    if (n4 * 4 + tid < n) {
+        q[n4 * 4 + tid] = (uint8_t)BG_QF(tail);
+    }
+#undef BG_QF4
+#undef BG_QF
+}
+
+// Workgroups the barrier is allowed to span: two per CU, or one where the kernel's registers allow no more
+// (0 if the device cannot be asked).
+template <int SRC_I32, int TO_U8, int PER>
+static uint32_t fused_max_grid()
+{
+    static int cached = -1;
+    if (cached < 0) {
+        int dev = 0, cus = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quantize_fused_kernel<SRC_I32, TO_U8, PER>, 256, 0) != hipSuccess) {
+            cached = 0;
+        } else {
+            cached = cus * (per_cu >= 2 ? 2 : per_cu);
+        }
+    }
+    return (uint32_t)cached;
+}
+
+template <int SRC_I32, int TO_U8, int PER>
+static hipError_t launch_fused(const void *x, uint32_t n, void *q, FusedSync &fs, float s_in, float *ds_out, hipStream_t st,
+    bool *taken)
+{
+    const uint32_t units = n / 4, per_block = 256 * PER;
+    uint32_t grid = (units + per_block - 1) / per_block;
+    grid = grid ? grid : 1;
+    if (grid > fused_max_grid<SRC_I32, TO_U8, PER>()) {
+        return hipSuccess;  // *taken stays false
+    }
+    fs.epoch += 1;
+    fs.target += grid;
+    hipLaunchKernelGGL((quantize_fused_kernel<SRC_I32, TO_U8, PER>), dim3(grid), dim3(256), 0, st, x, n, (uint8_t *)q, fs.slots,
+        fs.counter, fs.release, fs.epoch, fs.target, s_in, ds_out);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fs.epoch -= 1;  // nothing ran: the counter must not be waited for
+        fs.target -= grid;
+        return e;
+    }
+    *taken = true;
+    return hipSuccess;
+}
+
+// Dynamic fp32 -> u8 / s8 (src_i32 = 0; s_in = the caller's scale, <= 0 for none) or int32 -> u8 / s8 (src_i32 = 1;
+// s_in = scale of the int32 data) in one launch. *taken = false (and nothing launched) when the
+// tensor is larger than the size up to which this form wins (512 K elements), or misaligned: the caller then runs
+// the two-pass form.
+hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
+    float *ds_out, hipStream_t st, bool *taken)
+{
+    *taken = false;
+    // Measured on MI355X against the two-pass form (whose second read comes from the Infinity Cache): 10.4 against
+    // 14.9 us per call at 1 K elements, 12.0 against 15.4 at 64 K, 12.9 against 15.4 at 256 K, 16.3 against 15.4 at
+    // 1 M, slower beyond (the barrier's
+    // arrivals serialise at one address, about 10 ns each, and nothing overlaps the two phases).
+    if (n == 0 || n > (1u << 19) || !fs.slots || ((((uintptr_t)x | (uintptr_t)q) & 15) != 0)) {
+        return hipSuccess;
+    }
+#define BG_TRY(S, U, P)                                                                        \
+    {                                                                                          \
+        hipError_t e_ = launch_fused<S, U, P>(x, n, q, fs, s_in, ds_out, st, taken);           \
+        if (e_ != hipSuccess || *taken) {                                                      \
+            return e_;                                                                         \
+        }                                                                                      \
+    }
+#define BG_TRY_PER(S, U)   \
+    {                      \
+        BG_TRY(S, U, 4)    \
+        BG_TRY(S, U, 8)    \
+    }
+    if (src_i32) {
+        if (to_u8) {
+            BG_TRY_PER(1, 1)
+        } else {
+            BG_TRY_PER(1, 0)
+        }
+    } else if (to_u8) {
+        BG_TRY_PER(0, 1)
+    } else {
+        BG_TRY_PER(0, 0)
+    }
+#undef BG_TRY_PER
+#undef BG_TRY
+    return hipSuccess;
+}
+
 // avx512/quantize.cpp:271-313
 __global__ void u8_to_i8_kernel(const uint8_t *__restrict__ x, uint32_t n, int8_t *__restrict__ q)
 {

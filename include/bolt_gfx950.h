@@ -48,6 +48,10 @@ const char *bolt_gfx950_last_error(void);
  * shared-pipeline kernel. "conv_direct": whether that filter-panel kernel gathers from the caller's
  * u8 tensor in place when the channel count is a multiple of 16: 1 (default) for int32 and fp32
  * results, 2 for u8 results as well, 0 never (the input is first re-laid as a padded s8 image).
+ * "quantize_fused": 1 (default) runs a dynamic quantisation (fp32 or int32 input, scale taken from
+ * the tensor's maximum) as one launch that reads the tensor once and keeps it in registers
+ * across a grid-wide barrier, for tensors of up to 512 K elements that are 16-byte aligned (less
+ * latency per call; larger tensors are faster in two passes); 0 always takes the two-pass form.
  * "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
  * with its operands expanded to E2M1 pairs (v_mfma_scale_f32_16x16x128_f8f6f4) where the shape has
  * that kernel (256+ output channels, 128+ tiles of 256 pixels) and as 1 otherwise; 1 on the int8

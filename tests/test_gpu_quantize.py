@@ -21,6 +21,16 @@ def torch_mod():
     return torch
 
 
+@pytest.fixture(params=[1, 0], ids=["one_launch", "two_pass"])
+def fused(request, torch_mod):
+    """Dynamic quantisation has two implementations: one cooperative launch that reads the tensor once (default
+    where the tensor fits) and the two-pass form. The tests that use this fixture run under both."""
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused", request.param), "set_option")
+    yield request.param
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused", 1), "set_option")
+
+
 def both_modes(torch, x):
     yield "host", np.ascontiguousarray(x), (lambda t: np.asarray(t))
     yield "device", torch.from_numpy(np.ascontiguousarray(x)).cuda(), (lambda t: t.cpu().numpy())
@@ -28,7 +38,7 @@ def both_modes(torch, x):
 
 @pytest.mark.parametrize("n", [1, 15, 16, 17, 1000, 65536, 4096 * 768 + 5])
 @pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
-def test_quantize_f32(torch_mod, oracle, n, qdt):
+def test_quantize_f32(torch_mod, oracle, fused, n, qdt):
     print("quantize_f32", n, qdt, flush=True)
     rng = np.random.default_rng(n)
     x = rng.standard_normal(n).astype(np.float32)
@@ -41,7 +51,7 @@ def test_quantize_f32(torch_mod, oracle, n, qdt):
 
 
 @pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
-def test_quantize_f32_special_inputs(torch_mod, oracle, qdt):
+def test_quantize_f32_special_inputs(torch_mod, oracle, fused, qdt):
     cases = [np.zeros(33, np.float32),
              np.concatenate([np.full(40, 1e-3, np.float32), [1e6]]).astype(np.float32),
              tie_table(1.0), tie_table(0.5), np.array([-3.0, 3.0, -0.0, 1e-30, -1e30], np.float32)]
@@ -72,7 +82,7 @@ def test_quantize_f32_async_device_scale(torch_mod, oracle):
 
 
 @pytest.mark.parametrize("qdt", [DT_U8_Q, DT_I8])
-def test_quantize_i32(torch_mod, oracle, qdt):
+def test_quantize_i32(torch_mod, oracle, fused, qdt):
     rng = np.random.default_rng(5)
     cases = [rng.integers(-200000, 200000, size=n, dtype=np.int32) for n in (1, 15, 16, 17, 4099, 32 * 64 * 56 * 56)]
     cases.append(np.zeros(20, np.int32))
@@ -86,6 +96,38 @@ def test_quantize_i32(torch_mod, oracle, qdt):
                 got = back(host.quantize(buf, DT_I32, qdt, s))
                 assert np.array_equal(np.array(s, np.float32), ws), (name, sc, s, ws)
                 assert np.array_equal(got, want), (name, sc, x.size)
+
+
+@pytest.mark.parametrize("n", [262144 + 3, 1 << 19, (1 << 19) + 16])
+def test_quantize_one_launch_matches_two_pass(torch_mod, n):
+    """Around the size limit of the one-launch form (512 K elements; above it both settings run the two-pass form):
+    fp32 with a NaN and a known extreme, and int32 with INT32_MIN, each to u8 and s8; bytes and returned scales
+    must be identical under both settings."""
+    torch = torch_mod
+    L = capi.lib()
+    g = torch.Generator(device="cuda").manual_seed(n)
+    x = torch.randn(n, device="cuda", generator=g) * 3.0
+    x[n // 3] = float("nan")
+    x[n // 2] = -77.25
+    acc = torch.randint(-2000000, 2000000, (n,), dtype=torch.int32, device="cuda", generator=g)
+    acc[n // 5] = -(1 << 31)
+    out = {}
+    try:
+        for fused in (1, 0):
+            capi.check(L.bolt_gfx950_set_option(b"quantize_fused", fused), "set_option")
+            for qdt in (DT_U8_Q, DT_I8):
+                s = [-1.0]
+                q = host.quantize(x, DT_F32, qdt, s)
+                s2 = [np.float32(-1.0), np.float32(0.37)]
+                q2 = host.quantize(acc, DT_I32, qdt, s2)
+                capi.check(L.bolt_gfx950_synchronize(), "sync")
+                out[(fused, qdt)] = (q.clone(), s[0], q2.clone(), tuple(s2))
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused", 1), "set_option")
+    for qdt in (DT_U8_Q, DT_I8):
+        a, b = out[(1, qdt)], out[(0, qdt)]
+        assert a[1] == b[1] == np.float32(127.0) / np.float32(77.25) and a[3] == b[3]
+        assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[2])
 
 
 def test_u8_to_i8(torch_mod, oracle):
