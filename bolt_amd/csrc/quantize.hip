@@ -210,11 +210,13 @@ __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restri
     }
     const uint32_t stride = gridDim.x * blockDim.x;
     if (VEC) {
-        const uint32_t n16 = n / 16;
+        // lane-contiguous 16-byte loads (a wave's request = 1 KB of whole lines), four in flight, 4-byte stores
+        const uint32_t n4 = n / 4;
         const v4f *x4 = (const v4f *)x;
-        v4i *q16 = (v4i *)q;
-        for (uint32_t i = tid; i < n16; i += stride) {
-            v4f a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+        int *q4w = (int *)q;
+        uint32_t i = tid;
+        for (; i + 3 * stride < n4; i += 4 * stride) {
+            v4f a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
             if (GELU) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -224,10 +226,22 @@ __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restri
                     d[e] = gelu_tanh(d[e]);
                 }
             }
-            v4i o = {(int)q4<TO_U8>(a, s), (int)q4<TO_U8>(b, s), (int)q4<TO_U8>(c, s), (int)q4<TO_U8>(d, s)};
-            q16[i] = o;
+            q4w[i] = (int)q4<TO_U8>(a, s);
+            q4w[i + stride] = (int)q4<TO_U8>(b, s);
+            q4w[i + 2 * stride] = (int)q4<TO_U8>(c, s);
+            q4w[i + 3 * stride] = (int)q4<TO_U8>(d, s);
         }
-        for (uint32_t i = n16 * 16 + tid; i < n; i += stride) {
+        for (; i < n4; i += stride) {
+            v4f a = x4[i];
+            if (GELU) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = gelu_tanh(a[e]);
+                }
+            }
+            q4w[i] = (int)q4<TO_U8>(a, s);
+        }
+        for (i = n4 * 4 + tid; i < n; i += stride) {
             const float v = GELU ? gelu_tanh(x[i]) : x[i];
             q[i] = (uint8_t)(TO_U8 ? q_u8(v, s) : q_i8(v, s));
         }
