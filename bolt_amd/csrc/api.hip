@@ -350,7 +350,13 @@ EE bolt_gfx950_set_stream(void *stream)
     if (e != SUCCESS) {
         return e;
     }
-    ctx().stream = (hipStream_t)stream;
+    Ctx &c = ctx();
+    if (c.stream != (hipStream_t)stream) {
+        // the scratch words and the quantiser's sync area are shared by every call: work enqueued on the old stream
+        // must not overlap with what the new stream will run
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        c.stream = (hipStream_t)stream;
+    }
     return SUCCESS;
 }
 

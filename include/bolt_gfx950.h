@@ -34,7 +34,8 @@ extern "C" {
 /* ---- runtime ------------------------------------------------------------------------- */
 /* No counterpart in the reference (a CPU library needs no device context). */
 EE bolt_gfx950_init(void);
-/* stream: a hipStream_t (NULL = the default stream). The library never creates streams. */
+/* stream: a hipStream_t (NULL = the default stream). The library never creates streams. Changing the
+ * stream first waits for the work enqueued on the previous one (the library's scratch is shared). */
 EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
