@@ -28,6 +28,8 @@ struct Ctx {
     // the address the device uses for it.
     float *hscale = nullptr, *hscale_dev = nullptr;
     FusedSync fsync;  // sync area of the one-launch dynamic quantiser
+    uint32_t *enc_ws = nullptr;  // the encoder layer's four arrays of max slots (behind ws), kept clear between calls
+    bool enc_ws_dirty = true;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     struct Buf {
@@ -85,10 +87,11 @@ EE ensure_init()
     if (e != hipSuccess || n == 0) {
         return fail(NOT_SUPPORTED, "no HIP device available", e);
     }
-    e = hipMalloc((void **)&c.ws, (kWsWords + 64) * sizeof(uint32_t));
+    e = hipMalloc((void **)&c.ws, (kWsWords + 64 + 4 * kWsWords) * sizeof(uint32_t));
     if (e != hipSuccess) {
         return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
     }
+    c.enc_ws = c.ws + kWsWords + 64;
     {
         void *p = nullptr;
         e = hipMalloc(&p, kFusedSyncBytes);
@@ -2374,7 +2377,6 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     hipStream_t st = ctx().stream;
     U8 *w = (U8 *)workspace;
     const U32 T = L.batch * L.seq, H = L.hidden, F = L.ffn;
-    uint32_t *ws0 = (uint32_t *)(w + p.ws), *ws1 = ws0 + kWsWords, *ws2 = ws1 + kWsWords, *ws3 = ws2 + kWsWords;
     float *sc = (float *)(w + p.scales);
     uint8_t *xq = w + p.xq;
     float *qkv = (float *)(w + p.qkv), *cx = (float *)(w + p.ctx), *ao = (float *)(w + p.ao), *h1 = (float *)(w + p.h1),
@@ -2400,22 +2402,32 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
         return launch_gemm_u8s8(g, st);
     };
 
-    HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
+    // The four running maxima live in slots the library owns and keeps clear between calls: each array is zeroed
+    // by the first workgroup of a kernel that runs after the maximum's only reader and before its next producer
+    // (one layer call later). A call that fails half way leaves them in an unknown state, so they are refilled
+    // before the next one.
+    Ctx &c = ctx();
+    uint32_t *ws0 = c.enc_ws, *ws1 = ws0 + kWsWords, *ws2 = ws1 + kWsWords, *ws3 = ws2 + kWsWords;
+    if (c.enc_ws_dirty) {
+        HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
+    }
+    c.enc_ws_dirty = true;
     // x -> u8 (dynamic per-tensor scale), one quantisation shared by Q, K and V
     HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st, true));
     HIP_TRY(launch_quantize_f32(hidden, T * H, xq, 1, ws0, 0.0f, nullptr, 0, sc + 0, st));
     HIP_TRY(gemm(xq, L.wqkv, 3 * H, H, sc + 0, L.sqkv, L.bqkv, qkv));
-    HIP_TRY(launch_attention_f32(qkv, L.batch, L.seq, H, L.heads, cx, ws1, st));
+    HIP_TRY(launch_attention_f32(qkv, L.batch, L.seq, H, L.heads, cx, ws1, st, ws0));
     HIP_TRY(launch_quantize_f32(cx, T * H, xq, 1, ws1, 0.0f, nullptr, 0, sc + 1, st));
     HIP_TRY(gemm(xq, L.wo, H, H, sc + 1, L.so, L.bo, ao));
-    HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st));
+    HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st, ws1));
     HIP_TRY(launch_quantize_f32(h1, T * H, xq, 1, ws2, 0.0f, nullptr, 0, sc + 2, st));
     HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
     // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads
-    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st, false));
+    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st, false, ws2));
     HIP_TRY(launch_quantize_f32(f, T * F, xq, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 1));
     HIP_TRY(gemm(xq, L.w2, H, F, sc + 3, L.s2, L.b2, o));
-    HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st));
+    HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st, ws3));
+    c.enc_ws_dirty = false;
     return SUCCESS;
 }
 

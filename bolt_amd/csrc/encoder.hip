@@ -11,6 +11,15 @@
 
 namespace bg {
 
+// Optional duty of the first workgroup: zero the scratch slots of a maximum that has been consumed, so that the
+// next producer of those slots finds them clear without a launch of its own.
+__device__ __forceinline__ void clear_slots(uint32_t *clear)
+{
+    if (clear && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < kWsSlots) {
+        clear[threadIdx.x * kWsStride] = 0;
+    }
+}
+
 // ---- attention ------------------------------------------------------------------------------------
 // qkv: [batch * S][3 * H] fp32 rows (Q | K | V), head h owns columns h*64 .. h*64+63 of each third.
 // fp32 matrix cores (v_mfma_f32_16x16x4_f32), no LDS: a wave owns 32 queries of one (batch, head) and
@@ -28,8 +37,9 @@ typedef float v4f_t __attribute__((ext_vector_type(4)));
 
 template <int D>
 __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__restrict__ qkv, uint32_t S, uint32_t H,
-    float qscale, float *__restrict__ ctx, uint32_t *ws)
+    float qscale, float *__restrict__ ctx, uint32_t *ws, uint32_t *clear)
 {
+    clear_slots(clear);
     static_assert(D == 64, "head size 64");
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t c = lane & 15, g = lane >> 4;
@@ -160,7 +170,7 @@ __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__re
 }
 
 hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, uint32_t H, uint32_t heads, float *ctx,
-    uint32_t *ws, hipStream_t st)
+    uint32_t *ws, hipStream_t st, uint32_t *clear)
 {
     if (batch == 0 || S == 0 || heads == 0) {
         return hipSuccess;
@@ -169,7 +179,7 @@ hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, ui
         return hipErrorInvalidValue;
     }
     const dim3 grid((S + 127) / 128, heads, batch);
-    hipLaunchKernelGGL((attention_f32_kernel<64>), grid, dim3(256), 0, st, qkv, S, H, 0.125f, ctx, ws);
+    hipLaunchKernelGGL((attention_f32_kernel<64>), grid, dim3(256), 0, st, qkv, S, H, 0.125f, ctx, ws, clear);
     return hipGetLastError();
 }
 
@@ -179,8 +189,9 @@ hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, ui
 template <int V4>
 __global__ __launch_bounds__(256) void add_layernorm_kernel(const float *__restrict__ a, const float *__restrict__ b,
     const float *__restrict__ gamma, const float *__restrict__ beta, uint32_t rows, uint32_t H, float *__restrict__ out,
-    uint32_t *ws)
+    uint32_t *ws, uint32_t *clear)
 {
+    clear_slots(clear);
     __shared__ int red[4];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t row = blockIdx.x * 4 + wave;
@@ -241,7 +252,7 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(const float *__restr
 }
 
 hipError_t launch_add_layernorm(const float *a, const float *b, const float *gamma, const float *beta, uint32_t rows,
-    uint32_t H, float *out, uint32_t *ws, hipStream_t st)
+    uint32_t H, float *out, uint32_t *ws, hipStream_t st, uint32_t *clear)
 {
     if (rows == 0) {
         return hipSuccess;
@@ -251,7 +262,7 @@ hipError_t launch_add_layernorm(const float *a, const float *b, const float *gam
     }
     const dim3 grid((rows + 3) / 4);
     const uint32_t v4 = (H / 4 + 63) / 64;
-#define BG_LN(V) hipLaunchKernelGGL((add_layernorm_kernel<V>), grid, dim3(256), 0, st, a, b, gamma, beta, rows, H, out, ws)
+#define BG_LN(V) hipLaunchKernelGGL((add_layernorm_kernel<V>), grid, dim3(256), 0, st, a, b, gamma, beta, rows, H, out, ws, clear)
     if (v4 <= 1) {
         BG_LN(1);
     } else if (v4 <= 2) {
@@ -271,8 +282,9 @@ hipError_t launch_add_layernorm(const float *a, const float *b, const float *gam
 // STORE = false leaves x as it is and only folds max|gelu(x)| into ws: the quantiser that follows applies the
 // same gelu_tanh to what it reads, so the activated tensor is never written.
 template <bool STORE>
-__global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, uint32_t n4, uint32_t *ws)
+__global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, uint32_t n4, uint32_t *ws, uint32_t *clear)
 {
+    clear_slots(clear);
     __shared__ int red[4];
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -294,7 +306,7 @@ __global__ __launch_bounds__(256) void gelu_f32_kernel(float *__restrict__ x, ui
     }
 }
 
-hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store)
+hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store, uint32_t *clear)
 {
     if (n == 0) {
         return hipSuccess;
@@ -306,9 +318,9 @@ hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, boo
     uint32_t blocks = (n4 + 255) / 256;
     blocks = blocks > 4096 ? 4096 : blocks;
     if (store) {
-        hipLaunchKernelGGL(gelu_f32_kernel<true>, dim3(blocks), dim3(256), 0, st, x, n4, ws);
+        hipLaunchKernelGGL(gelu_f32_kernel<true>, dim3(blocks), dim3(256), 0, st, x, n4, ws, clear);
     } else {
-        hipLaunchKernelGGL(gelu_f32_kernel<false>, dim3(blocks), dim3(256), 0, st, x, n4, ws);
+        hipLaunchKernelGGL(gelu_f32_kernel<false>, dim3(blocks), dim3(256), 0, st, x, n4, ws, clear);
     }
     return hipGetLastError();
 }

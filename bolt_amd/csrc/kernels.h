@@ -122,15 +122,16 @@ hipError_t launch_bnn_expand_filter_fp4(const uint32_t *src, uint32_t OC, uint32
     hipStream_t st);
 
 // ---- fp32 neighbours of the int8 GEMMs in an encoder layer (encoder.hip) --------------------------
-// Each takes an optional `ws` (kWsWords scratch words, zeroed by the caller) into which max|out| is folded.
+// Each takes an optional `ws` (kWsWords scratch words, zeroed by the caller) into which max|out| is folded, and an
+// optional `clear` (another such array, whose maximum has been consumed) that its first workgroup zeroes.
 // qkv rows are [Q | K | V] of 3*H floats; head size 64 (H == heads * 64).
 hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, uint32_t H, uint32_t heads, float *ctx,
-    uint32_t *ws, hipStream_t st);
+    uint32_t *ws, hipStream_t st, uint32_t *clear = nullptr);
 // out = LayerNorm(a + b) (b may be null); H % 4 == 0, H <= 2048
 hipError_t launch_add_layernorm(const float *a, const float *b, const float *gamma, const float *beta, uint32_t rows,
-    uint32_t H, float *out, uint32_t *ws, hipStream_t st);
+    uint32_t H, float *out, uint32_t *ws, hipStream_t st, uint32_t *clear = nullptr);
 // store = false: x is left untouched, only max|gelu(x)| is folded into ws (pair it with launch_quantize_f32(..., gelu = 1))
-hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store = true);
+hipError_t launch_gelu_f32(float *x, size_t n, uint32_t *ws, hipStream_t st, bool store = true, uint32_t *clear = nullptr);
 
 // ---- weight pack --------------------------------------------------------------------------------
 // src: s8, element (k, n) at src[k * sk + n * sn]. Writes the packed matrix and comp[n].

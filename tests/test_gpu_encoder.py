@@ -162,6 +162,24 @@ def test_encoder_layer_bert_base(torch_mod, oracle):
     assert r2 < LAYER_RTOL and rmax < 1e-2 and frac < 1e-3
 
 
+def test_encoder_layer_calls_do_not_leak_maxima(torch_mod):
+    """The layer's running maxima live in scratch slots that are cleared inside the layer's own kernels rather than
+    by a launch of their own: a call on small activations must give the same bits before and after a call on
+    activations a hundred times larger."""
+    torch = torch_mod
+    batch, seq, hidden, heads, ffn = 2, 64, 256, 4, 512
+    rng = np.random.default_rng(11)
+    P = make_params(rng, hidden, ffn, with_bias=True)
+    x = rng.standard_normal((batch * seq, hidden)).astype(np.float32)
+    layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
+    small, big = dev(torch, 0.05 * x), dev(torch, 5.0 * x + 3.0)
+    a = layer(small).clone()
+    layer(big)
+    b = layer(small).clone()
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    assert torch.equal(a, b)
+
+
 def test_encoder_errors(torch_mod):
     L = capi.lib()
     spec = capi.BoltEncoderLayerInt8()
