@@ -22,8 +22,11 @@ __device__ __forceinline__ void clear_slots(uint32_t *clear)
 
 // ---- attention ------------------------------------------------------------------------------------
 // qkv: [batch * S][3 * H] fp32 rows (Q | K | V), head h owns columns h*64 .. h*64+63 of each third.
-// fp32 matrix cores (v_mfma_f32_16x16x4_f32), no LDS: a wave owns 32 queries of one (batch, head) and
-// walks the keys in chunks of 128.
+// fp32 matrix cores (v_mfma_f32_16x16x4_f32): a workgroup owns 64 * NT queries of one (batch, head), each of its
+// four waves 16 * NT of them, and walks the keys in chunks of 16 * KT. A chunk's K and V rows (64 floats each) are
+// brought into LDS once per workgroup with whole-line loads (16 lanes per 256-byte row) and read from there by
+// all four waves; rows are 68 floats apart, which keeps both the 16-byte K reads (16 different rows per
+// quarter wave) and the 4-byte V reads (4 rows x 16 consecutive floats) free of bank conflicts.
 //   scores^T = K . Q^T   : M = key, N = query, contraction over d. A lane (c = lane % 16, g = lane / 16)
 //                          feeds K[key c][16 s + 4 g + t] and Q[query c][16 s + 4 g + t] for step (s, t):
 //                          one 16-byte load covers four steps, and both operands permute d the same way.
@@ -35,7 +38,8 @@ __device__ __forceinline__ void clear_slots(uint32_t *clear)
 // Chunks are merged with the streaming (running max / running sum) form of the max-subtracted softmax.
 typedef float v4f_t __attribute__((ext_vector_type(4)));
 
-template <int D>
+// NT: query tiles of 16 per wave (a workgroup owns 64 * NT queries); KT: key tiles of 16 per chunk.
+template <int D, int NT, int KT>
 __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__restrict__ qkv, uint32_t S, uint32_t H,
     float qscale, float *__restrict__ ctx, uint32_t *ws, uint32_t *clear)
 {
@@ -44,17 +48,18 @@ __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__re
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t c = lane & 15, g = lane >> 4;
     const uint32_t h = blockIdx.y, b = blockIdx.z;
-    const uint32_t q0 = blockIdx.x * 128 + wave * 32;
-    if (q0 >= S) {
-        return;
-    }
+    const uint32_t q0 = blockIdx.x * (64 * NT) + wave * (16 * NT);
+    const bool active = q0 < S;  // a wave past the end of the sequence still helps to load the chunks
+    extern __shared__ __attribute__((aligned(16))) float att_smem[];
+    constexpr uint32_t kRow = 68;  // floats between rows in LDS
+    float *sK = att_smem, *sV = att_smem + KT * 16 * kRow;
     const size_t ld = 3 * (size_t)H;
     const float *Qb = qkv + (size_t)b * S * ld + (size_t)h * D;
     const float *Kb = Qb + H, *Vb = Qb + 2 * (size_t)H;
 
-    v4f_t qf[2][4];
+    v4f_t qf[NT][4];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
         uint32_t q = q0 + nt * 16 + c;
         q = q < S ? q : S - 1;
 #pragma unroll
@@ -63,49 +68,79 @@ __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__re
             qf[nt][s4] = v * qscale;
         }
     }
-    v4f_t o[4][2];
+    v4f_t o[4][NT];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-        o[mt][0] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
-        o[mt][1] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.0f, 0.0f};
-
-    for (uint32_t k0 = 0; k0 < S; k0 += 128) {
-        v4f_t s[8][2];
 #pragma unroll
-        for (int kt = 0; kt < 8; ++kt) {
-            s[kt][0] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
-            s[kt][1] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
-            uint32_t key = k0 + kt * 16 + c;
-            key = key < S ? key : S - 1;
-            const float *kp = Kb + (size_t)key * ld + 4 * g;
+        for (int nt = 0; nt < NT; ++nt) {
+            o[mt][nt] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    float m[NT], l[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        m[nt] = -INFINITY;
+        l[nt] = 0.0f;
+    }
+
+    for (uint32_t k0 = 0; k0 < S; k0 += KT * 16) {
+        if (k0) {
+            __syncthreads();  // everyone is done with the previous chunk
+        }
+        {   // chunk -> LDS: KT * 256 pieces of 16 bytes per matrix, KT per thread; rows past the end repeat the last one
+#pragma unroll
+            for (int r = 0; r < KT; ++r) {
+                const uint32_t piece = threadIdx.x + r * 256, row = piece >> 4, col = (piece & 15) * 4;
+                uint32_t key = k0 + row;
+                key = key < S ? key : S - 1;
+                const v4f_t kv = *(const v4f_t *)(Kb + (size_t)key * ld + col);
+                const v4f_t vv = *(const v4f_t *)(Vb + (size_t)key * ld + col);
+                *(v4f_t *)(sK + row * kRow + col) = kv;
+                *(v4f_t *)(sV + row * kRow + col) = vv;
+            }
+        }
+        __syncthreads();
+        if (!active) {
+            continue;
+        }
+        v4f_t s[KT][NT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                s[kt][nt] = (v4f_t){0.0f, 0.0f, 0.0f, 0.0f};
+            }
+            const float *kp = sK + (kt * 16 + c) * kRow + 4 * g;
 #pragma unroll
             for (int s4 = 0; s4 < 4; ++s4) {
                 const v4f_t kf = *(const v4f_t *)(kp + 16 * s4);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    s[kt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t], qf[0][s4][t], s[kt][0], 0, 0, 0);
-                    s[kt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t], qf[1][s4][t], s[kt][1], 0, 0, 0);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        s[kt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t], qf[nt][s4][t], s[kt][nt], 0, 0, 0);
+                    }
                 }
             }
         }
         // keys past the end of the sequence do not take part
 #pragma unroll
-        for (int kt = 0; kt < 8; ++kt) {
+        for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if (k0 + kt * 16 + 4 * g + i >= S) {
-                    s[kt][0][i] = -INFINITY;
-                    s[kt][1][i] = -INFINITY;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        s[kt][nt][i] = -INFINITY;
+                    }
                 }
             }
         }
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
+        for (int nt = 0; nt < NT; ++nt) {
             float mx = m[nt];
 #pragma unroll
-            for (int kt = 0; kt < 8; ++kt) {
+            for (int kt = 0; kt < KT; ++kt) {
                 mx = fmaxf(mx, fmaxf(fmaxf(s[kt][nt][0], s[kt][nt][1]), fmaxf(s[kt][nt][2], s[kt][nt][3])));
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -113,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__re
             const float corr = __expf(m[nt] - mx);  // exp(-inf) = 0 on the first chunk
             float sum = 0.0f;
 #pragma unroll
-            for (int kt = 0; kt < 8; ++kt) {
+            for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float p = __expf(s[kt][nt][i] - mx);
@@ -131,24 +166,27 @@ __global__ __launch_bounds__(256, 2) void attention_f32_kernel(const float *__re
             }
         }
 #pragma unroll
-        for (int kt = 0; kt < 8; ++kt) {
+        for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                uint32_t key = k0 + kt * 16 + 4 * g + t;
-                key = key < S ? key : S - 1;  // its probability is 0
-                const float *vp = Vb + (size_t)key * ld + c;
+                const float *vp = sV + (kt * 16 + 4 * g + t) * kRow + c;  // rows past the end: probability 0
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) {
                     const float vv = vp[16 * mt];
-                    o[mt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, s[kt][0][t], o[mt][0], 0, 0, 0);
-                    o[mt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, s[kt][1][t], o[mt][1], 0, 0, 0);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        o[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, s[kt][nt][t], o[mt][nt], 0, 0, 0);
+                    }
                 }
             }
         }
     }
+    if (!active) {
+        return;
+    }
     float amax = 0.0f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
         const uint32_t q = q0 + nt * 16 + c;
         const float inv = 1.0f / l[nt];
         if (q < S) {
@@ -178,8 +216,21 @@ hipError_t launch_attention_f32(const float *qkv, uint32_t batch, uint32_t S, ui
     if (H != heads * 64) {
         return hipErrorInvalidValue;
     }
-    const dim3 grid((S + 127) / 128, heads, batch);
-    hipLaunchKernelGGL((attention_f32_kernel<64>), grid, dim3(256), 0, st, qkv, S, H, 0.125f, ctx, ws, clear);
+    // 16 queries per wave and 64 keys per chunk: 64-query workgroups, three of which share a CU (35 KB of LDS each).
+    // At BERT-base (seq 128, 12 heads, batch 32) that is 768 workgroups = 3 waves on every SIMD; with 32 queries
+    // per wave the 384 workgroups leave half the CUs with twice the work of the other half.
+    constexpr int NT = 1, KT = 4;
+    const dim3 grid((S + 64 * NT - 1) / (64 * NT), heads, batch);
+    constexpr uint32_t lds = 2 * KT * 16 * 68 * sizeof(float);  // K and V chunk, rows 68 floats apart
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)attention_f32_kernel<64, NT, KT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) {
+            return e;
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((attention_f32_kernel<64, NT, KT>), grid, dim3(256), lds, st, qkv, S, H, 0.125f, ctx, ws, clear);
     return hipGetLastError();
 }
 
