@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize"],
+    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool"],
                     help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
@@ -324,6 +324,43 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                                                                    dsc.data_ptr(), 0), "q"))
         both("dequantize_i32_f32", 8 * cnt, lambda i: host.dequantize(accs[i], DT_I32, 37.5, out=fo[i]))
         both("requantize_i32_u8_static", 5 * cnt, lambda i: host.quantize(accs[i], DT_I32, DT_U8_Q, [0.02, 37.5], out=q8[i]))
+    # -- u8 pooling (NCHWC16) and s8 concatenation with a common scale: byte work, rotating over 16 inputs (more than
+    #    the Infinity Cache holds) and on one input reused call after call
+    if want("pool"):
+        from bolt_amd import host_pool
+        from bolt_amd.capi import DT_I8, POOLING_MAX, POOLING_MEAN, pooling_param_spec, tensor4df
+        R = 16
+        it = [0]
+
+        def rot(fn):
+            def call():
+                it[0] += 1
+                fn(it[0] % R)
+            return call
+
+        def both(name, nbytes, fn, cfg):
+            t_h = timed(rot(fn), 80, warm=16)
+            t_c = timed(lambda: fn(0), 50)
+            res[name] = {"config": cfg, "ms": t_h, "algorithmic_bytes": nbytes, "gbps": nbytes / t_h / 1e6,
+                         "frac_hbm_peak": nbytes / t_h / 1e6 / HBM_PEAK_GBS, "ms_cache_resident": t_c,
+                         "gbps_cache_resident": nbytes / t_c / 1e6}
+        n, c, ih, iw = 32, 64, 112, 112
+        xs = [torch.randint(0, 256, (n * c * ih * iw,), dtype=torch.uint8, device=dev, generator=g) for _ in range(R)]
+        ys = [torch.empty(n * c * 56 * 56, dtype=torch.uint8, device=dev) for _ in range(R)]
+        pmax = pooling_param_spec(POOLING_MAX, 3, 3, 2, 2, 1, 1, 1, 1)
+        pmean = pooling_param_spec(POOLING_MEAN, 2, 2, 2, 2, 0, 0, 0, 0)
+        nb = n * c * (ih * iw + 56 * 56)
+        both("pooling_u8_max_3x3_s2", nb, lambda i: host_pool.pooling_u8(xs[i], n, c, ih, iw, pmax, 4.0, 56, 56, out=ys[i]),
+             "32 x 64 x 112 x 112 -> 56 x 56, pad 1")
+        both("pooling_u8_mean_2x2_s2", nb, lambda i: host_pool.pooling_u8(xs[i], n, c, ih, iw, pmean, 4.0, 56, 56, out=ys[i]),
+             "32 x 64 x 112 x 112 -> 56 x 56")
+        half = n * c * ih * iw // 2
+        d_in = tensor4df(DT_I8, DF_NCHWC16, n, 128, 56, 56)
+        d_out = tensor4df(DT_I8, DF_NCHWC16, n, 256, 56, 56)
+        cat = [torch.empty(2 * half, dtype=torch.uint8, device=dev) for _ in range(R)]
+        both("concat_i8_rescale_channels", 4 * half,
+             lambda i: host_pool.concat([xs[i][:half], xs[i][half:]], [d_in, d_in], 1, d_out, [9.0, 6.5], out=cat[i]),
+             "2 x (32 x 128 x 56 x 56) -> 32 x 256 x 56 x 56, one input rescaled by 6.5 / 9, the other copied")
     return res
 
 

@@ -41,6 +41,14 @@ def tensor4df(dt, df, n, c, h, w):
     return d
 
 
+def tensor_num_bytes(d):
+    """tensorNumBytes (tensor_desc.h) for byte-sized and wider element types."""
+    n = 1
+    for i in range(d.nDims):
+        n *= d.dims[i]
+    return n * {DT_U8: 1, DT_I8: 1, DT_U32: 4, DT_I32: 4, DT_F16: 2, DT_F32: 4, DT_U8_Q: 1}[d.dt]
+
+
 def tensor2df(dt, df, rows, cols):
     d = tensor4df(dt, df, 1, 1, rows, cols)
     d.nDims = 2
@@ -84,6 +92,32 @@ def conv_param_spec(oc, fh, fw, stride, pad, dilation=1, group=1):
     p.group, p.dilatedRate_t, p.dilatedRate_h, p.dilatedRate_w = group, 1, dilation, dilation
     p.num_outputs_origin = oc
     p.convolution_type = 3  # CONVOLUTION_DEPTHWISE_POINTWISE, what the reference's tests pass
+    return p
+
+
+class PoolingParamSpec(C.Structure):
+    """common/uni/include/parameter_spec.h:285-301"""
+    _fields_ = [(k, C.c_uint32) for k in (
+        "kernel_t", "kernel_h", "kernel_w", "stride_t", "stride_h", "stride_w", "pad_before", "pad_after", "pad_top",
+        "pad_bottom", "pad_left", "pad_right", "round_mode", "mode")] + [("count_include_pad", C.c_bool)]
+
+
+class ConcatParamSpec(C.Structure):
+    """common/uni/include/parameter_spec.h:451-454"""
+    _fields_ = [("axis", C.c_int32), ("num_concat", C.c_int32)]
+
+
+assert C.sizeof(PoolingParamSpec) == 60 and C.sizeof(ConcatParamSpec) == 8
+POOLING_MAX, POOLING_MEAN = 0, 1
+
+
+def pooling_param_spec(mode, kh, kw, sh, sw, pt, pb, pl, pr, count_include_pad=False, round_mode=0):
+    """createPoolingParamSpec (parameter_spec.h:936-970) for the 2-D case."""
+    p = PoolingParamSpec()
+    p.kernel_t, p.kernel_h, p.kernel_w = 1, kh, kw
+    p.stride_t, p.stride_h, p.stride_w = 1, sh, sw
+    p.pad_top, p.pad_bottom, p.pad_left, p.pad_right = pt, pb, pl, pr
+    p.round_mode, p.mode, p.count_include_pad = round_mode, mode, bool(count_include_pad)
     return p
 
 
@@ -146,6 +180,10 @@ SIGNATURES = {
     "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),
     "convolution_bnn_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, ConvolutionParamSpec, TensorDesc, _vp,
                                          TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, ActivationParamSpec, C.c_int]),
+    "pooling_gfx950": (C.c_int, [TensorDesc, _vp, PoolingParamSpec, _vp, TensorDesc, _vp, _vp, C.c_int]),
+    "concat_infer_forward_tmp_bytes_gfx950": (C.c_int, [_u32, _TDp, TensorDesc, _u32p, C.c_int]),
+    "concat_gfx950": (C.c_int, [_u32, _TDp, C.POINTER(_vp), _f32p, ConcatParamSpec, _vp, TensorDesc, _vp, _f32p,
+                                C.c_int]),
     "bolt_gfx950_encoder_layer_int8_workspace_bytes": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),
                                                                  C.POINTER(C.c_size_t)]),
     "bolt_gfx950_encoder_layer_int8_workspace_layout": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),

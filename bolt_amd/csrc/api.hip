@@ -2271,6 +2271,240 @@ EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F
     return SUCCESS;
 }
 
+// ---- u8 pooling (compute/tensor/src/cpu/x86/int8/avx512/pooling_int8.cpp:316-429) ---------------------
+EE pooling_gfx950(TensorDesc inputDesc, const void *input, PoolingParamSpec p, void *scale, TensorDesc outputDesc,
+    void *output, void *idx, Arch arch)
+{
+    (void)idx;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!input || !output) {
+        return NULL_POINTER;
+    }
+    U32 n, ic, ih, iw, on, oc, oh, ow;
+    if (get4d(inputDesc, &n, &ic, &ih, &iw) != SUCCESS || get4d(outputDesc, &on, &oc, &oh, &ow) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (inputDesc.dt != DT_U8_Q) {
+        return NOT_SUPPORTED;   // pooling_x86 routes only DT_U8_Q to the quantised kernels
+    }
+    if (outputDesc.dt != DT_U8_Q || n != on || ic != oc || inputDesc.df != DF_NCHWC16 || outputDesc.df != DF_NCHWC16 ||
+        ic % 16 != 0) {
+        return NOT_MATCH;
+    }
+    if (p.mode != POOLING_MAX && p.mode != POOLING_MEAN) {
+        return NOT_SUPPORTED;
+    }
+    // a zero kernel extent means the whole image (update_param, compute/tensor/src/pooling.cpp:107-131)
+    if (p.kernel_w == 0) {
+        p.kernel_w = iw;
+    }
+    if (p.kernel_h == 0) {
+        p.kernel_h = ih;
+    }
+    if (p.kernel_h == 0 || p.kernel_w == 0 || p.stride_h == 0 || p.stride_w == 0 || p.pad_top >= p.kernel_h ||
+        p.pad_left >= p.kernel_w) {
+        return NOT_SUPPORTED;
+    }
+    const unsigned long long window = (unsigned long long)p.kernel_h * p.kernel_w;
+    if (window > 65536ull) {
+        return NOT_SUPPORTED;   // 65536 / window < 1
+    }
+    const U32 factor = 65536u / (U32)window;
+    const size_t inB = (size_t)n * ic * ih * iw, outB = (size_t)n * ic * oh * ow;
+    if (outB == 0) {
+        return SUCCESS;
+    }
+    if (inB == 0 || outB / 16 > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    // the last window in each direction must still start inside the image
+    if ((unsigned long long)(oh - 1) * p.stride_h >= (unsigned long long)ih + p.pad_top ||
+        (unsigned long long)(ow - 1) * p.stride_w >= (unsigned long long)iw + p.pad_left) {
+        return NOT_SUPPORTED;
+    }
+    if (scale) {
+        F32 *sc = (F32 *)scale;
+        if (p.mode == POOLING_MAX) {
+            sc[1] = sc[0];
+        } else {
+            sc[1] = sc[0] * (F32)(I32)factor * (F32)(U32)window / (F32)65536;
+        }
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    bg::PoolArgs a;
+    a.total = (uint32_t)(outB / 16);
+    a.IH = ih;
+    a.IW = iw;
+    a.OH = oh;
+    a.OW = ow;
+    a.kh = p.kernel_h;
+    a.kw = p.kernel_w;
+    a.sh = p.stride_h;
+    a.sw = p.stride_w;
+    a.pt = p.pad_top;
+    a.pl = p.pad_left;
+    a.mean = p.mode == POOLING_MEAN;
+    a.count_include_pad = p.count_include_pad ? 1 : 0;
+    a.pool_full = factor;
+    if (arch == AMD_GFX950) {
+        Stage st;
+        void *di = st.get(inB), *dout = st.get(outB);
+        if (!di || !dout) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        HIP_TRY(hipMemcpyAsync(di, input, inB, hipMemcpyHostToDevice, c.stream));
+        a.in = (const uint8_t *)di;
+        a.out = (uint8_t *)dout;
+        HIP_TRY(bg::launch_pool_u8_c16(a, c.stream));
+        HIP_TRY(hipMemcpyAsync(output, dout, outB, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        return SUCCESS;
+    }
+    a.in = (const uint8_t *)input;
+    a.out = (uint8_t *)output;
+    HIP_TRY(bg::launch_pool_u8_c16(a, c.stream));
+    return SUCCESS;
+}
+
+// ---- concatenation with a common scale (compute/tensor/src/cpu/concat.cpp:90-189) -----------------------
+EE concat_infer_forward_tmp_bytes_gfx950(U32 num, const TensorDesc *inputDesc, TensorDesc outputDesc, U32 *bytes,
+    Arch arch)
+{
+    (void)num;
+    (void)inputDesc;
+    (void)outputDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    *bytes = 0;   // no format conversion is done here, so nothing is staged
+    return SUCCESS;
+}
+
+EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const F32 *inputScale, ConcatParamSpec p,
+    void *tmp, TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch)
+{
+    (void)tmp;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!output || (num && (!inputDesc || !input))) {
+        return NULL_POINTER;
+    }
+    const bool rescale = outputDesc.dt == DT_I8 && inputScale && outputScale;
+    F32 oscale = 0;
+    if (rescale && num > 0) {
+        oscale = inputScale[0];
+        for (U32 j = 1; j < num; ++j) {
+            oscale = std::min(inputScale[j], oscale);
+        }
+        *outputScale = oscale;
+    }
+    const int dim = (int)outputDesc.nDims;
+    if (dim < 1 || dim > (int)DIM_LEN) {
+        return NOT_MATCH;
+    }
+    int axis = ((p.axis % dim) + dim) % dim;
+    axis = dim - 1 - axis;   // index into dims[], which runs innermost first
+    size_t tile = bytesOf(outputDesc.dt);
+    for (int i = 0; i < axis; ++i) {
+        tile *= outputDesc.dims[i];
+    }
+    size_t loops = 1;
+    for (int i = axis + 1; i < dim; ++i) {
+        loops *= outputDesc.dims[i];
+    }
+    const U32 cblock = outputDesc.df == DF_NCHWC8 ? 8 : outputDesc.df == DF_NCHWC16 ? 16 : 1;
+    const bool blocked = cblock > 1 && dim == 4;
+    if (blocked && axis < dim - 2) {
+        tile *= cblock;   // joined along h or w: a "row" of the copy spans the channel block as well
+        loops /= cblock;
+    }
+    // validate: same type / format / rank, same extents off the axis, extents on the axis add up
+    U32 sum = 0;
+    for (U32 j = 0; j < num; ++j) {
+        if (!input[j] || tensorNumElements(inputDesc[j]) == 0) {
+            continue;
+        }
+        const TensorDesc &d = inputDesc[j];
+        if (d.dt != outputDesc.dt || (int)d.nDims != dim) {
+            return NOT_MATCH;
+        }
+        if (d.df != outputDesc.df) {
+            return NOT_SUPPORTED;
+        }
+        for (int i = 0; i < dim; ++i) {
+            if (i != axis && d.dims[i] != outputDesc.dims[i]) {
+                return NOT_MATCH;
+            }
+        }
+        if (blocked && axis == dim - 2 && d.dims[axis] % cblock != 0) {
+            return NOT_SUPPORTED;
+        }
+        sum += d.dims[axis];
+    }
+    if (sum == 0) {
+        return SUCCESS;
+    }
+    if (sum != outputDesc.dims[axis]) {
+        return NOT_MATCH;
+    }
+    if (loops > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    const size_t ostride = (size_t)sum * tile;
+    const size_t outB = ostride * loops;
+    Stage st;
+    uint8_t *dout = (uint8_t *)output;
+    if (arch == AMD_GFX950) {
+        dout = (uint8_t *)st.get(outB);
+        if (!dout) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+    }
+    size_t off = 0;
+    for (U32 j = 0; j < num; ++j) {
+        if (!input[j] || tensorNumElements(inputDesc[j]) == 0) {
+            continue;
+        }
+        const size_t len = (size_t)inputDesc[j].dims[axis] * tile;
+        if (len > 0xffffffffull) {
+            return NOT_SUPPORTED;
+        }
+        const void *src = input[j];
+        if (arch == AMD_GFX950) {
+            void *d = st.get(len * loops);
+            if (!d) {
+                return fail(ALLOC_FAILED, "device staging");
+            }
+            HIP_TRY(hipMemcpyAsync(d, input[j], len * loops, hipMemcpyHostToDevice, c.stream));
+            src = d;
+        }
+        const bool rs = rescale && inputScale[j] != oscale;
+        HIP_TRY(bg::launch_concat_i8(src, dout + off, (uint32_t)loops, (uint32_t)len, ostride, rs ? 1 : 0,
+            rs ? oscale / inputScale[j] : 1.0f, c.stream));
+        off += len;
+    }
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(output, dout, outB, hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
 // ---- BERT-style int8 encoder layer --------------------------------------------------------------------
 namespace {
 struct EncoderPlan {

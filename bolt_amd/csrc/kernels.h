@@ -178,4 +178,20 @@ hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32
 hipError_t launch_mfma_i8_rate(uint32_t blocks, uint32_t iters, int zero, int *sink, hipStream_t st);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]
 
+// ---- u8 pooling and s8 concatenation (pool.hip) ---------------------------------------------------
+struct PoolArgs {
+    const uint8_t *in = nullptr;   // [planes][IH][IW][16]
+    uint8_t *out = nullptr;        // [planes][OH][OW][16]
+    uint32_t total = 0;            // planes * OH * OW, one lane each
+    uint32_t IH = 0, IW = 0, OH = 0, OW = 0;
+    uint32_t kh = 0, kw = 0, sh = 0, sw = 0, pt = 0, pl = 0;
+    int mean = 0, count_include_pad = 0;
+    uint32_t pool_full = 0;        // 65536 / (kh * kw)
+};
+// Every window must overlap the image (the caller checks); mean needs kh * kw <= 65536
+hipError_t launch_pool_u8_c16(const PoolArgs &a, hipStream_t st);
+// rows x len bytes from contiguous rows into rows `ostride` bytes apart; rescale: out = (s8)(r * in)
+hipError_t launch_concat_i8(const void *in, void *out, uint32_t rows, uint32_t len, size_t ostride, int rescale,
+    float r, hipStream_t st);
+
 }  // namespace bg

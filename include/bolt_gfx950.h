@@ -205,6 +205,37 @@ EE convolution_bnn_gfx950(TensorDesc inputDesc, const void *input, TensorDesc fi
     ConvolutionParamSpec convParamSpec, TensorDesc scaleDesc, const void *scale, TensorDesc biasDesc, const void *bias,
     U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, ActivationParamSpec activationDesc, Arch arch);
 
+/* ---- quantised pooling and concatenation --------------------------------------------- */
+/* pooling_x86 with DT_U8_Q data (compute/tensor/src/cpu/x86/pooling.cpp:22-61 ->
+ * pooling_uint8, compute/tensor/src/cpu/x86/int8/avx512/pooling_int8.cpp:316-429). Input and output
+ * DT_U8_Q in DF_NCHWC16, channels a multiple of 16, pad_top < kernel_h and pad_left < kernel_w as
+ * in the reference; outputDesc carries the output height and width (pooling_infer_output_size is
+ * the caller's, compute/tensor/src/pooling.cpp). Windows are clipped to the image. POOLING_MAX:
+ * byte maximum. POOLING_MEAN: the reference's fixed-point form -- (sum of (u8 - 128)) * (65536 /
+ * taps) >> 16 with a logical shift, + 128, unsigned saturation; taps = the clipped window, or
+ * kernel_h * kernel_w with count_include_pad. scale: F32[2] in host memory, scale[0] = input scale
+ * (read), scale[1] = output scale (written): scale[0] for max, scale[0] * (65536 / (kh*kw)) *
+ * (kh*kw) / 65536 for mean. idx is unused for u8 data (as in the reference). Every window must
+ * overlap the image, otherwise NOT_SUPPORTED. */
+EE pooling_gfx950(TensorDesc inputDesc, const void *input, PoolingParamSpec poolingParamSpec, void *scale,
+    TensorDesc outputDesc, void *output, void *idx, Arch arch);
+
+/* concat_cpu (compute/tensor/src/cpu/concat.cpp:164-189): num inputs joined along
+ * p.axis (counted from the outermost dimension, negative from the innermost, as in the reference).
+ * With outputDesc.dt == DT_I8 and both scale pointers set, *outputScale = min(inputScale[0..num))
+ * and every input is rescaled to it with requantize_cpu's arithmetic (compute/tensor/src/cpu/
+ * requantize.cpp:20-50) while it is copied; the reference rescales its inputs in place first and
+ * then copies, this entry point leaves the inputs untouched. Without scales it is a plain
+ * concatenation of any element type. inputDesc / input / inputScale are host arrays of num entries;
+ * inputScale and outputScale point to host memory; null or empty inputs are skipped (their scales
+ * still take part in the minimum, as in the reference). All inputs must already be in the output's
+ * data format (the reference's transformFormat step is not provided): DF_NCHWC8 / DF_NCHWC16
+ * tensors join along the channel axis in whole channel blocks. tmp is unused. */
+EE concat_infer_forward_tmp_bytes_gfx950(U32 num, const TensorDesc *inputDesc, TensorDesc outputDesc, U32 *bytes,
+    Arch arch);
+EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const F32 *inputScale, ConcatParamSpec p,
+    void *tmp, TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch);
+
 /* ---- BERT-style int8 encoder layer (device pointers only, asynchronous) ------------- */
 /* One post-LayerNorm transformer encoder layer as Bolt runs it for an int8 BERT model: the four
  * FullyConnected operators (QKV merged into one, as model_tools' FC+FC merge does for BERT,

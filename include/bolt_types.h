@@ -16,6 +16,7 @@
 #ifndef BOLT_GFX950_TYPES_H
 #define BOLT_GFX950_TYPES_H
 
+#include <stdbool.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -251,6 +252,38 @@ typedef struct {
 } ConvolutionParamSpec;
 #pragma pack()
 
+/* common/uni/include/parameter_spec.h:21 */
+typedef enum {
+    POOLING_MAX = 0,
+    POOLING_MEAN = 1,
+    POOLING_MODE_FORCE_U32 = 0x7fffffff
+} PoolingMode;
+
+/* common/uni/include/parameter_spec.h:285-301 (60 bytes) */
+typedef struct {
+    U32 kernel_t;
+    U32 kernel_h;
+    U32 kernel_w;
+    U32 stride_t;
+    U32 stride_h;
+    U32 stride_w;
+    U32 pad_before;
+    U32 pad_after;
+    U32 pad_top;
+    U32 pad_bottom;
+    U32 pad_left;
+    U32 pad_right;
+    RoundMode round_mode;
+    PoolingMode mode;
+    bool count_include_pad;
+} PoolingParamSpec;
+
+/* common/uni/include/parameter_spec.h:451-454 */
+typedef struct {
+    I32 axis;
+    I32 num_concat;
+} ConcatParamSpec;
+
 static inline U32 bolt_align(U32 x, U32 a)
 {
     return a == 0 ? 0 : (x + a - 1) / a * a;
@@ -315,6 +348,7 @@ static inline U32 tensorNumBytes(TensorDesc d)
 #ifdef __cplusplus
 }
 static_assert(sizeof(TensorDesc) == 92, "TensorDesc must match Bolt's 92-byte record");
+static_assert(sizeof(PoolingParamSpec) == 60, "PoolingParamSpec must match Bolt's record");
 static_assert(sizeof(DataType) == 4 && sizeof(DataFormat) == 4, "enums are 32-bit in Bolt");
 #endif
 

@@ -84,6 +84,17 @@ void orc_bnn_conv(const orc_bnn_desc *d, const uint8_t *in_bits, const uint8_t *
 void orc_bnn_conv_bruteforce(const orc_bnn_desc *d, const float *x_nchw, const float *w_nchw,
     int32_t *sums_nchw);
 
+/* ---- u8 pooling (NCHWC16) and s8 concatenation ------------------------------------- */
+typedef struct {
+    uint32_t n, c, ih, iw, oh, ow;
+    uint32_t kh, kw, sh, sw, pt, pl;
+    int mean;              /* 0 = POOLING_MAX, 1 = POOLING_MEAN */
+    int count_include_pad;
+} orc_pool_desc;
+int orc_pooling_u8_c16(const orc_pool_desc *d, const uint8_t *in, uint8_t *out, float *scale /* [in, out] */);
+void orc_concat_i8(uint32_t num, const int8_t *const *in, const uint32_t *len, const float *scales, uint32_t loops,
+    int8_t *out, float *oscale);
+
 #ifdef __cplusplus
 }
 #endif

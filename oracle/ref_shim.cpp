@@ -14,6 +14,8 @@
 #include "tensor_desc.h"
 #include "parameter_spec.h"
 #include "cpu/x86/int8/tensor_computing_int8.h"
+#include "cpu/tensor_computing_cpu.h"
+#include <vector>
 
 // internal (non-public) reference prototypes, compute/tensor/src/cpu/x86/tensor_computing_x86.h
 EE quantize_x86(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *qData, F32 *scale, int mode);
@@ -192,6 +194,46 @@ int ref_conv_int8(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 fw
     free(tmp);
     free(ftm);
     return e;
+}
+
+// u8 pooling on NCHWC16 (compute/tensor/src/cpu/x86/int8/avx512/pooling_int8.cpp:316). scale[2] = {in, out}.
+int ref_pooling_u8(U32 n, U32 c, U32 ih, U32 iw, U32 oh, U32 ow, U32 kh, U32 kw, U32 sh, U32 sw, U32 pt, U32 pl,
+    int mean, int count_include_pad, const uint8_t *in, uint8_t *out, float *scale)
+{
+    PoolingParamSpec p;
+    memset(&p, 0, sizeof(p));
+    p.kernel_t = 1;
+    p.kernel_h = kh;
+    p.kernel_w = kw;
+    p.stride_t = 1;
+    p.stride_h = sh;
+    p.stride_w = sw;
+    p.pad_top = pt;
+    p.pad_left = pl;
+    p.mode = mean ? POOLING_MEAN : POOLING_MAX;
+    p.count_include_pad = count_include_pad != 0;
+    TensorDesc inputDesc = tensor4df(DT_U8_Q, DF_NCHWC16, n, c, ih, iw);
+    TensorDesc outputDesc = tensor4df(DT_U8_Q, DF_NCHWC16, n, c, oh, ow);
+    return pooling_uint8(inputDesc, in, p, outputDesc, out, scale);
+}
+
+// s8 concatenation with a common scale (compute/tensor/src/cpu/concat.cpp:164). Inputs are 4-D tensors in `df`
+// that differ in dims[axis_from_outermost]; they are rescaled in place by the reference, so pass copies.
+int ref_concat_i8(U32 num, const U32 *dims4 /* num x {n,c,h,w} */, int df, int axis, int8_t **in, float *scales,
+    const U32 *odims4, int8_t *out, float *oscale)
+{
+    std::vector<TensorDesc> descs;
+    std::vector<void *> ptrs;
+    for (U32 j = 0; j < num; ++j) {
+        descs.push_back(tensor4df(DT_I8, (DataFormat)df, dims4[4 * j], dims4[4 * j + 1], dims4[4 * j + 2],
+            dims4[4 * j + 3]));
+        ptrs.push_back(in[j]);
+    }
+    TensorDesc od = tensor4df(DT_I8, (DataFormat)df, odims4[0], odims4[1], odims4[2], odims4[3]);
+    ConcatParamSpec p;
+    p.axis = axis;
+    p.num_concat = (I32)num;
+    return concat_cpu(descs, ptrs, scales, p, nullptr, od, out, oscale, X86_AVX512);
 }
 
 }  // extern "C"

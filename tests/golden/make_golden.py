@@ -18,6 +18,7 @@ sys.path.insert(0, os.path.dirname(HERE))
 
 from checkers import DT_F32, DT_I8, DT_I32, DT_U8_Q, Oracle, Ref  # noqa: E402
 from checkers_conv import DF_NCHWC8, ConvOracle, ref_conv, to_nchwc  # noqa: E402
+from checkers_pool import pool_desc, ref_concat, ref_pooling  # noqa: E402
 
 SEED = 20240601
 
@@ -190,6 +191,30 @@ def gen_conv(ref, orc):
     save("conv_int8", out)
 
 
+def gen_pool(ref):
+    """u8 pooling (pooling_uint8) and s8 concatenation (concat_cpu) as the reference computes them."""
+    from test_oracle_pool import CONCAT_CASES, POOL_CASES, concat_inputs, concat_layout, pool_input
+    out = {"pool_cases": np.array(POOL_CASES, np.int64)}
+    for i, case in enumerate(POOL_CASES):
+        d = pool_desc(case)
+        x = pool_input(case, SEED + 60 + i, relu=(i % 3 != 2))
+        y, s = ref_pooling(ref, d, x, 12.75)
+        out[f"pool_x{i}"], out[f"pool_y{i}"], out[f"pool_s{i}"] = x, y, np.float32(s)
+    out["concat_n"] = np.array(len(CONCAT_CASES), np.int64)
+    for i, case in enumerate(CONCAT_CASES):
+        df, axis, dims, scales = case
+        parts = concat_inputs(case, SEED + 80 + i)
+        _, _, odims = concat_layout(case)
+        y, s = ref_concat(ref, parts, dims, df, axis, scales, odims)
+        out[f"cat_meta{i}"] = np.array([df, axis], np.int64)
+        out[f"cat_dims{i}"] = np.array(dims, np.int64)
+        out[f"cat_scales{i}"] = np.array(scales, np.float32)
+        for j, part in enumerate(parts):
+            out[f"cat_in{i}_{j}"] = part
+        out[f"cat_y{i}"], out[f"cat_s{i}"] = y, np.float32(s)
+    save("pool_concat", out)
+
+
 if __name__ == "__main__":
     if not Ref.available():
         sys.exit("oracle/_ref/libboltref.so is missing or this host has no avx512_vnni")
@@ -199,3 +224,4 @@ if __name__ == "__main__":
     gen_mvm(ref, orc)
     gen_quantize(ref, orc)
     gen_conv(ref, orc)
+    gen_pool(ref)

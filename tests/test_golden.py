@@ -94,3 +94,20 @@ def test_conv_int8(oracle):
                 got, gs = co.conv(d, g[f"xq{i}"], g[f"W{i}"], g[f"bias{i}"], [g[f"sI{i}"], -1.0, g[f"sF{i}"]])
                 assert same(gs, g[f"{nm}_relu{relu}_scale{i}"]), (case, nm, relu)
                 assert same(got, g[f"{nm}_relu{relu}_{i}"]), (case, nm, relu)
+
+
+def test_pool_and_concat(oracle):
+    from checkers_pool import orc_concat, orc_pooling, pool_desc
+    g = load("pool_concat")
+    for i, case in enumerate(g["pool_cases"]):
+        d = pool_desc(tuple(int(v) for v in case))
+        y, s = orc_pooling(oracle, d, g[f"pool_x{i}"], 12.75)
+        assert same(y, g[f"pool_y{i}"]) and same(np.float32(s), g[f"pool_s{i}"])
+    for i in range(int(g["concat_n"])):
+        dims = g[f"cat_dims{i}"]
+        axis = int(g[f"cat_meta{i}"][1]) % 4
+        parts = [g[f"cat_in{i}_{j}"] for j in range(len(dims))]
+        lens = [int(np.prod(d[axis:])) for d in dims]
+        loops = int(np.prod(dims[0][:axis]))
+        y, s = orc_concat(oracle, parts, lens, loops, g[f"cat_scales{i}"])
+        assert same(y, g[f"cat_y{i}"]) and same(np.float32(s), g[f"cat_s{i}"])
