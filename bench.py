@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool"],
+    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool", "lstm"],
                     help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
@@ -361,6 +361,25 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         both("concat_i8_rescale_channels", 4 * half,
              lambda i: host_pool.concat([xs[i][:half], xs[i][half:]], [d_in, d_in], 1, d_out, [9.0, 6.5], out=cat[i]),
              "2 x (32 x 128 x 56 x 56) -> 32 x 256 x 56 x 56, one input rescaled by 6.5 / 9, the other copied")
+    # -- int8 LSTM cell at the decode shape: 256 rows, x 2048 + h 2048 -> 4 x 2048 gates (the headline GEMV, N = 8192,
+    #    K = 4096, inside its caller: per-row quantisation, one batched GEMV launch, gates and state update)
+    if want("lstm"):
+        from bolt_amd import host_lstm
+        batch, xdim, hdim = 256, 2048, 2048
+        Wl = torch.randint(-127, 128, (4 * hdim, xdim + hdim), dtype=torch.int8, device=dev, generator=g)
+        blob = host_lstm.transform_weight(Wl, 4 * hdim, xdim + hdim)
+        xl = torch.randn((batch, xdim), device=dev, generator=g)
+        bl = torch.randn((batch, 4 * hdim), device=dev, generator=g) * 0.5
+        stl = torch.randn((batch, 2 * hdim), device=dev, generator=g) * 0.7
+        ol = torch.empty((batch, hdim), device=dev)
+        pl = host_lstm.lstm_param_spec(hdim)
+        tmp = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+        t = timed(lambda: host_lstm.lstmcell(xl, blob, bl, [-1.0, 250.0], stl, pl, batch, xdim, ol, tmp=tmp), 30)
+        per_row = 4 * hdim * (xdim + hdim) + 4 * (xdim + 2 * hdim + 4 * hdim + 2 * hdim + hdim)
+        res["lstmcell_int8_decode"] = {"config": "256 rows, x 2048, h 2048 (weight 8192 x 4096 s8, read once per row)",
+                                       "ms": t, "rows_per_s": batch / (t * 1e-3), "algorithmic_bytes": batch * per_row,
+                                       "gbps": batch * per_row / t / 1e6,
+                                       "frac_hbm_peak": batch * per_row / t / 1e6 / HBM_PEAK_GBS}
     return res
 
 

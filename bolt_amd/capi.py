@@ -121,6 +121,17 @@ def pooling_param_spec(mode, kh, kw, sh, sw, pt, pb, pl, pr, count_include_pad=F
     return p
 
 
+class RNNParamSpec(C.Structure):
+    """common/uni/include/parameter_spec.h:380-393"""
+    _fields_ = [("mode", C.c_uint32), ("num_outputs", C.c_uint32), ("steps", C.c_int32), ("num_projection", C.c_int32),
+                ("zoneout_cell", C.c_float), ("zoneout_output", C.c_float), ("bi_direction", C.c_bool),
+                ("forget_bias", C.c_float), ("activation_type", C.c_uint32)]
+
+
+assert C.sizeof(RNNParamSpec) == 36
+RNN_LSTM, ACTIVATION_TANH, DF_NKN32 = 1, 6, 19
+
+
 _vp, _u32, _f32p, _u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
 _TDp = C.POINTER(TensorDesc)
 
@@ -184,6 +195,9 @@ SIGNATURES = {
     "concat_infer_forward_tmp_bytes_gfx950": (C.c_int, [_u32, _TDp, TensorDesc, _u32p, C.c_int]),
     "concat_gfx950": (C.c_int, [_u32, _TDp, C.POINTER(_vp), _f32p, ConcatParamSpec, _vp, TensorDesc, _vp, _f32p,
                                 C.c_int]),
+    "rnncell_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, RNNParamSpec, _u32p, C.c_int]),
+    "rnncell_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, C.POINTER(_vp), _TDp, C.POINTER(_vp), _f32p, _vp, _u32, _vp,
+                                 RNNParamSpec, _u32, _u32, TensorDesc, _vp, C.c_int]),
     "bolt_gfx950_encoder_layer_int8_workspace_bytes": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),
                                                                  C.POINTER(C.c_size_t)]),
     "bolt_gfx950_encoder_layer_int8_workspace_layout": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),

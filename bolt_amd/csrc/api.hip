@@ -2505,6 +2505,186 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
     return SUCCESS;
 }
 
+// ---- int8 LSTM cell (compute/tensor/src/cpu/x86/int8/lstm.cpp:20-179) -----------------------------------
+namespace {
+struct LstmShape {
+    U32 batch, xDim, hDim, N, K;
+    size_t quantOff, dscaleOff, scaleWOff, interOff, total;
+};
+
+EE lstm_shape(TensorDesc xDesc, RNNParamSpec p, LstmShape *s)
+{
+    DataType dt;
+    DataFormat df;
+    if (get2d(xDesc, &dt, &df, &s->batch, &s->xDim) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (p.mode != RNN_LSTM || p.num_projection > 0) {
+        return NOT_SUPPORTED;
+    }
+    s->hDim = p.num_outputs;
+    s->N = 4 * s->hDim;
+    s->K = s->xDim + s->hDim;
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    s->quantOff = 0;
+    s->dscaleOff = up((size_t)s->batch * s->K);
+    s->scaleWOff = s->dscaleOff + up((size_t)s->batch * 4);
+    s->interOff = s->scaleWOff + up((size_t)s->N * 4);
+    s->total = s->interOff + up((size_t)s->batch * s->N * 4);
+    return SUCCESS;
+}
+}  // namespace
+
+EE rnncell_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    RNNParamSpec p, U32 *bytes, Arch arch)
+{
+    (void)filterDesc;
+    (void)outputDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    LstmShape s;
+    EE e = lstm_shape(inputDesc, p, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (s.total > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)s.total;
+    return SUCCESS;
+}
+
+EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filterDesc, const void **filter,
+    const TensorDesc *biasDesc, const void **bias, F32 *scale, void *state, U32 tmpBytes, void *tmp, RNNParamSpec p,
+    U32 batchStrideX, U32 batchStrideH, TensorDesc hDesc, void *output, Arch arch)
+{
+    (void)biasDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!filter || !bias || !state || !tmp || !output || !filterDesc || !scale || !filter[0] || !bias[0]) {
+        return NULL_POINTER;
+    }
+    LstmShape s;
+    EE e = lstm_shape(xDesc, p, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    DataType fdt, odt;
+    DataFormat fdf, odf;
+    U32 fn, fk, on, oh;
+    if (get2d(filterDesc[0], &fdt, &fdf, &fn, &fk) != SUCCESS || get2d(hDesc, &odt, &odf, &on, &oh) != SUCCESS) {
+        return NOT_MATCH;
+    }
+    if (xDesc.dt != DT_F32 || fdt != DT_I8 || odt != DT_F32 || fn != s.N || fk != s.K || on != s.batch || oh != s.hDim) {
+        return NOT_MATCH;   // lstm.cpp:65-70 (an fp32 filter is another back end's)
+    }
+    if (p.activation_type != ACTIVATION_TANH) {
+        return NOT_SUPPORTED;
+    }
+    if (s.batch == 0 || s.hDim == 0) {
+        return SUCCESS;
+    }
+    if (s.xDim > 0 && !currentX) {
+        return NULL_POINTER;
+    }
+    if (tmpBytes < s.total) {
+        return NOT_MATCH;
+    }
+    if (s.batch > 65535 || batchStrideH < s.hDim || (s.xDim > 0 && batchStrideX < s.xDim)) {
+        return NOT_SUPPORTED;
+    }
+    const U32 steps = batchStrideH / s.hDim / (p.bi_direction ? 2 : 1);   // lstm.cpp:64
+    const size_t biasStride = (size_t)steps * s.N;
+    if (biasStride > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    Stage st;
+    const size_t blobB = (size_t)packed_matrix_bytes(s.N, s.K) + (size_t)s.N * 4;
+    const size_t stateB = (size_t)s.batch * 2 * s.hDim * 4;
+    bg::LstmArgs a;
+    a.batch = s.batch;
+    a.xdim = s.xDim;
+    a.hdim = a.column = s.hDim;
+    a.scale_in = scale[0];
+    a.forget_bias = p.forget_bias;
+    a.zoneout_cell = p.zoneout_cell;
+    a.zoneout_output = p.zoneout_output;
+    const void *dW = filter[0];
+    U8 *dT = (U8 *)tmp;
+    float *dOut = nullptr, *dState = nullptr;
+    if (arch == AMD_GFX950) {
+        // host pointers: rows are gathered into compact device copies
+        float *dx = (float *)st.get((size_t)s.batch * std::max<U32>(s.xDim, 1) * 4);
+        float *db = (float *)st.get((size_t)s.batch * s.N * 4);
+        void *w = st.get(blobB);
+        dState = (float *)st.get(stateB);
+        dOut = (float *)st.get((size_t)s.batch * s.hDim * 4);
+        dT = (U8 *)st.get(s.total);
+        if (!dx || !db || !w || !dState || !dOut || !dT) {
+            return fail(ALLOC_FAILED, "device staging");
+        }
+        for (U32 m = 0; m < s.batch; ++m) {
+            if (s.xDim) {
+                HIP_TRY(hipMemcpyAsync(dx + (size_t)m * s.xDim, (const float *)currentX + (size_t)m * batchStrideX,
+                    (size_t)s.xDim * 4, hipMemcpyHostToDevice, c.stream));
+            }
+            HIP_TRY(hipMemcpyAsync(db + (size_t)m * s.N, (const float *)bias[0] + m * biasStride, (size_t)s.N * 4,
+                hipMemcpyHostToDevice, c.stream));
+        }
+        HIP_TRY(hipMemcpyAsync(w, filter[0], blobB, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(dState, state, stateB, hipMemcpyHostToDevice, c.stream));
+        dW = w;
+        a.x = dx;
+        a.x_stride = s.xDim;
+        a.bias = db;
+        a.bias_stride = s.N;
+        a.state = dState;
+        a.out = dOut;
+        a.out_stride = s.hDim;
+    } else {
+        a.x = (const float *)currentX;
+        a.x_stride = batchStrideX;
+        a.bias = (const float *)bias[0];
+        a.bias_stride = (uint32_t)biasStride;
+        a.state = (float *)state;
+        a.out = (float *)output;
+        a.out_stride = batchStrideH;
+    }
+    a.quant = dT + s.quantOff;
+    a.dscale = (float *)(dT + s.dscaleOff);
+    float *scaleW = (float *)(dT + s.scaleWOff);
+    float *inter = (float *)(dT + s.interOff);
+    a.inter = inter;
+    uint32_t wbits;
+    memcpy(&wbits, &scale[1], 4);
+    HIP_TRY(bg::launch_fill_u32((uint32_t *)scaleW, s.N, wbits, c.stream));
+    HIP_TRY(bg::launch_lstm_xh_quant(a, c.stream));
+    e = bolt_gfx950_mvm_int8_strided_batch(s.batch, s.N, s.K, dW, 0, 1, a.quant, inter, a.dscale, scaleW, nullptr);
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(bg::launch_lstm_gates(a, c.stream));
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipMemcpyAsync(state, dState, stateB, hipMemcpyDeviceToHost, c.stream));
+        for (U32 m = 0; m < s.batch; ++m) {
+            HIP_TRY(hipMemcpyAsync((float *)output + (size_t)m * batchStrideH, dOut + (size_t)m * s.hDim,
+                (size_t)s.hDim * 4, hipMemcpyDeviceToHost, c.stream));
+        }
+        HIP_TRY(hipStreamSynchronize(c.stream));
+    }
+    return SUCCESS;
+}
+
 // ---- BERT-style int8 encoder layer --------------------------------------------------------------------
 namespace {
 struct EncoderPlan {

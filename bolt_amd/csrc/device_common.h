@@ -68,6 +68,18 @@ __device__ __forceinline__ unsigned epi_u8(int acc, float factor)
     return usat8_u((int)((unsigned)rne_i32(f) + 128u));
 }
 
+// fp32 -> u8 around the zero point 128
+__device__ __forceinline__ unsigned q_u8(float x, float s)
+{
+    // avx512/quantize.cpp:150-155: vmulps, vaddps 128.0f, vcvtps2dq {rn}, clamp [1, 255]
+    float t = x * s;
+    float u = t + 128.0f;
+    int v = rne_i32(u);
+    v = v < 1 ? 1 : v;
+    v = v > 255 ? 255 : v;
+    return (unsigned)v;
+}
+
 __device__ __forceinline__ unsigned epi_u8_trunc(int acc, float factor)
 {
     float f = (float)acc * factor;

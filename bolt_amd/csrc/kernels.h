@@ -194,4 +194,23 @@ hipError_t launch_pool_u8_c16(const PoolArgs &a, hipStream_t st);
 hipError_t launch_concat_i8(const void *in, void *out, uint32_t rows, uint32_t len, size_t ostride, int rescale,
     float r, hipStream_t st);
 
+// ---- int8 LSTM cell (lstm.hip) ----------------------------------------------------------------------
+struct LstmArgs {
+    uint32_t batch = 0, xdim = 0, hdim = 0, column = 0;   // column = hdim when there is no projection
+    const float *x = nullptr;      // row m at x + m * x_stride
+    uint32_t x_stride = 0;
+    float *state = nullptr;        // row m: [C (column) | H (hdim)]
+    const float *bias = nullptr;   // row m at bias + m * bias_stride, 4 * column floats: i, g, f, o
+    uint32_t bias_stride = 0;
+    float scale_in = 0;            // caller's activation scale; <= 0: dynamic per row
+    uint8_t *quant = nullptr;      // [batch][xdim + hdim]
+    float *dscale = nullptr;       // [batch]
+    const float *inter = nullptr;  // [batch][4 * column] products
+    float *out = nullptr;          // row m at out + m * out_stride
+    uint32_t out_stride = 0;
+    float forget_bias = 0, zoneout_cell = 0, zoneout_output = 0;
+};
+hipError_t launch_lstm_xh_quant(const LstmArgs &a, hipStream_t st);
+hipError_t launch_lstm_gates(const LstmArgs &a, hipStream_t st);
+
 }  // namespace bg

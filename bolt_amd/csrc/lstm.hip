@@ -1,0 +1,95 @@
+// int8 LSTM cell around the batched GEMV (compute/tensor/src/cpu/x86/int8/lstm.cpp:20-179):
+//   lstm_xh_quant_kernel   per batch row: [x | h] gathered, its own dynamic (or the caller's static) scale,
+//                          fp32 -> u8 with the quantiser's arithmetic (lstm.cpp:89-109)
+//   lstm_gates_kernel      bias add, gates, cell / hidden state update with zoneout (lstm.cpp:113-176)
+// The matrix-vector products in between are one launch of gemv_s8u8_kernel over all rows.
+#include "kernels.h"
+
+namespace bg {
+
+__global__ __launch_bounds__(256) void lstm_xh_quant_kernel(const LstmArgs a)
+{
+    __shared__ float red[4];
+    const uint32_t m = blockIdx.x;
+    const float *x = a.x + (size_t)m * a.x_stride;
+    const float *h = a.state + (size_t)m * (a.column + a.hdim) + a.column;
+    const uint32_t K = a.xdim + a.hdim;
+    float mx = 0.0f;
+    for (uint32_t k = threadIdx.x; k < K; k += 256) {
+        const float v = k < a.xdim ? x[k] : h[k - a.xdim];
+        mx = fmaxf(mx, fabsf(v));
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        mx = fmaxf(mx, __shfl_xor(mx, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = mx;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    // quantize with mode 1 (avx512/quantize.cpp:129-133): the caller's scale if it is positive, else 127 / max
+    float s = a.scale_in;
+    if (s <= 0) {
+        const float dyn = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+        s = (s > dyn) ? s : dyn;
+    }
+    uint8_t *q = a.quant + (size_t)m * K;
+    for (uint32_t k = threadIdx.x; k < K; k += 256) {
+        const float v = k < a.xdim ? x[k] : h[k - a.xdim];
+        q[k] = (uint8_t)q_u8(v, s);
+    }
+    if (threadIdx.x == 0) {
+        a.dscale[m] = s;
+    }
+}
+
+__device__ __forceinline__ float sigmoid_f(float v)
+{
+    return 1.0f / (1.0f + expf(-v));
+}
+
+__global__ __launch_bounds__(256) void lstm_gates_kernel(const LstmArgs a)
+{
+    const uint32_t h = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t m = blockIdx.y;
+    if (h >= a.column) {
+        return;
+    }
+    const float *g = a.inter + (size_t)m * 4 * a.column;
+    const float *b = a.bias + (size_t)m * a.bias_stride;
+    const float gi = g[h] + b[h];
+    const float gg = g[h + a.column] + b[h + a.column];
+    const float gf = g[h + 2 * a.column] + b[h + 2 * a.column];
+    const float go = g[h + 3 * a.column] + b[h + 3 * a.column];
+    float *stC = a.state + (size_t)m * (a.column + a.hdim);
+    float *stH = stC + a.column;
+    const float c0 = stC[h];
+    const float I = sigmoid_f(gi), F = sigmoid_f(gf + a.forget_bias), O = sigmoid_f(go), G = tanhf(gg);
+    const float c1 = c0 * F + I * G;
+    const float hid = O * tanhf(c1);
+    if (a.zoneout_cell != 0) {
+        stC[h] = c1 * (1 - a.zoneout_cell) + c0 * a.zoneout_cell;
+    } else {
+        stC[h] = c1;
+    }
+    a.out[(size_t)m * a.out_stride + h] = hid;
+    if (a.zoneout_output != 0) {
+        stH[h] = hid * (1 - a.zoneout_output) + stH[h] * a.zoneout_output;
+    } else {
+        stH[h] = hid;
+    }
+}
+
+hipError_t launch_lstm_xh_quant(const LstmArgs &a, hipStream_t st)
+{
+    hipLaunchKernelGGL(lstm_xh_quant_kernel, dim3(a.batch), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_lstm_gates(const LstmArgs &a, hipStream_t st)
+{
+    hipLaunchKernelGGL(lstm_gates_kernel, dim3((a.column + 255) / 256, a.batch), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+}  // namespace bg

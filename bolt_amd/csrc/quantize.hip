@@ -156,17 +156,6 @@ hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStre
 }
 
 // ---- fp32 -> u8 / s8 ----------------------------------------------------------------------------
-__device__ __forceinline__ unsigned q_u8(float x, float s)
-{
-    // avx512/quantize.cpp:150-155: vmulps, vaddps 128.0f, vcvtps2dq {rn}, clamp [1, 255]
-    float t = x * s;
-    float u = t + 128.0f;
-    int v = rne_i32(u);
-    v = v < 1 ? 1 : v;
-    v = v > 255 ? 255 : v;
-    return (unsigned)v;
-}
-
 __device__ __forceinline__ unsigned q_i8(float x, float s)
 {
     // avx512/quantize.cpp:208-212: vmulps, vcvtps2dq, clamp [-127, 127]

@@ -236,6 +236,33 @@ EE concat_infer_forward_tmp_bytes_gfx950(U32 num, const TensorDesc *inputDesc, T
 EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const F32 *inputScale, ConcatParamSpec p,
     void *tmp, TensorDesc outputDesc, void *output, F32 *outputScale, Arch arch);
 
+/* ---- int8 LSTM cell -------------------------------------------------------------------- */
+/* rnncell_int8 -> lstmcell_int8 (compute/tensor/src/cpu/x86/int8/rnn.cpp:16-44, lstm.cpp:20-179), the
+ * caller of the int8 matrix-vector product in recurrent models (compute/tensor/src/cpu/rnn.cpp:467-504).
+ * Per batch row m: [x_m | h_m] is quantised to u8 with its own scale (scale[0] if positive, else
+ * 127 / max|.|), multiplied with the int8 weight, dequantised with scale[1] as the weight scale, the
+ * row's bias is added, then i, g, f, o gates (sigmoid, tanh, sigmoid(f + forget_bias), sigmoid), cell and
+ * hidden state update with the reference's zoneout arithmetic.
+ *   xDesc        DT_F32 [batch, xDim]; row m of currentX starts at currentX + m * batchStrideX floats
+ *   filterDesc[0] DT_I8 [4 * num_outputs, xDim + num_outputs], tagged DF_NKN32 as the reference does;
+ *   filter[0]    the output of matrix_vector_multiply_transform_weight_gfx950 for that matrix (packed
+ *                rows followed by the compensation vector, which is where the reference reads offsetC)
+ *   bias[0]      DT_F32; row m reads 4 * num_outputs floats at bias[0] + m * steps * 4 * num_outputs with
+ *                steps = batchStrideH / num_outputs / (bi_direction + 1), exactly as the reference
+ *   scale        host F32[2] = {activation scale or <= 0 for dynamic, weight scale}; not written
+ *   state        DT_F32 [batch][num_outputs (C) | num_outputs (H)], updated in place
+ *   output       row m at output + m * batchStrideH floats, num_outputs floats
+ *   tmp          rnncell_infer_forward_tmp_bytes_gfx950 bytes
+ * Integer accumulators are exact; the gates use expf / tanhf where the reference's vector loop uses its
+ * polynomial exp and its scalar tail uses double-precision libm: results agree to about 1e-6.
+ * num_projection > 0 (an fp32 projection matrix), modes other than RNN_LSTM and activation types other
+ * than ACTIVATION_TANH return NOT_SUPPORTED. */
+EE rnncell_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    RNNParamSpec rnnParamSpec, U32 *bytes, Arch arch);
+EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filterDesc, const void **filter,
+    const TensorDesc *biasDesc, const void **bias, F32 *scale, void *state, U32 tmpBytes, void *tmp,
+    RNNParamSpec rnnParamSpec, U32 batchStrideX, U32 batchStrideH, TensorDesc hDesc, void *output, Arch arch);
+
 /* ---- BERT-style int8 encoder layer (device pointers only, asynchronous) ------------- */
 /* One post-LayerNorm transformer encoder layer as Bolt runs it for an int8 BERT model: the four
  * FullyConnected operators (QKV merged into one, as model_tools' FC+FC merge does for BERT,

@@ -284,6 +284,28 @@ typedef struct {
     I32 num_concat;
 } ConcatParamSpec;
 
+/* common/uni/include/parameter_spec.h:126 */
+typedef enum {
+    RNN_RNN = 0,
+    RNN_LSTM = 1,
+    RNN_GRU = 2,
+    RNN_GRU_LBR = 3,
+    RNN_MODE_FORCE_U32 = 0x7fffffff
+} RNNMode;
+
+/* common/uni/include/parameter_spec.h:380-393 (36 bytes) */
+typedef struct {
+    RNNMode mode;
+    U32 num_outputs;
+    I32 steps; /* >= 0: multi-step RNN, -1: RNNCell */
+    I32 num_projection;
+    float zoneout_cell;
+    float zoneout_output;
+    bool bi_direction;
+    float forget_bias;
+    ActivationMode activation_type;
+} RNNParamSpec;
+
 static inline U32 bolt_align(U32 x, U32 a)
 {
     return a == 0 ? 0 : (x + a - 1) / a * a;
@@ -349,6 +371,7 @@ static inline U32 tensorNumBytes(TensorDesc d)
 }
 static_assert(sizeof(TensorDesc) == 92, "TensorDesc must match Bolt's 92-byte record");
 static_assert(sizeof(PoolingParamSpec) == 60, "PoolingParamSpec must match Bolt's record");
+static_assert(sizeof(RNNParamSpec) == 36, "RNNParamSpec must match Bolt's record");
 static_assert(sizeof(DataType) == 4 && sizeof(DataFormat) == 4, "enums are 32-bit in Bolt");
 #endif
 

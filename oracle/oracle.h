@@ -95,6 +95,11 @@ int orc_pooling_u8_c16(const orc_pool_desc *d, const uint8_t *in, uint8_t *out, 
 void orc_concat_i8(uint32_t num, const int8_t *const *in, const uint32_t *len, const float *scales, uint32_t loops,
     int8_t *out, float *oscale);
 
+/* ---- int8 LSTM cell ---------------------------------------------------------------- */
+void orc_lstmcell_int8(uint32_t batch, uint32_t xdim, uint32_t hdim, const float *x, uint32_t x_stride,
+    const int8_t *W, const float *bias, uint32_t bias_stride, const float *scale, float *state, float forget_bias,
+    float zoneout_cell, float zoneout_output, float *out, uint32_t out_stride);
+
 #ifdef __cplusplus
 }
 #endif

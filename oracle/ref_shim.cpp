@@ -236,4 +236,50 @@ int ref_concat_i8(U32 num, const U32 *dims4 /* num x {n,c,h,w} */, int df, int a
     return concat_cpu(descs, ptrs, scales, p, nullptr, od, out, oscale, X86_AVX512);
 }
 
+// int8 LSTM cell (compute/tensor/src/cpu/x86/int8/lstm.cpp:20). W: s8 [4*hdim][xdim+hdim] row-major, packed here
+// with the reference's own matrix_vector_multiply_transform_weight. state rows [C | H]; scale = {activation, weight}.
+int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_stride, const int8_t *W, const float *bias,
+    float *scale, float *state, float forget_bias, float zoneout_cell, float zoneout_output, float *out, U32 out_stride)
+{
+    const U32 N = 4 * hdim, K = xdim + hdim;
+    TensorDesc wDesc = tensor2df(DT_I8, DF_NORMAL, N, K);
+    U32 bytes = 0;
+    EE e = matrix_vector_multiply_transform_weight_bytes(wDesc, &bytes, X86_AVX512);
+    if (e != SUCCESS) {
+        return 1000 + e;
+    }
+    INT8 *blob = (INT8 *)calloc((size_t)bytes + 64, 1);
+    TensorDesc tDesc;
+    e = matrix_vector_multiply_transform_weight(wDesc, W, &tDesc, blob, X86_AVX512);
+    if (e != SUCCESS) {
+        free(blob);
+        return 2000 + e;
+    }
+    RNNParamSpec p;
+    memset(&p, 0, sizeof(p));
+    p.mode = RNN_LSTM;
+    p.num_outputs = hdim;
+    p.steps = -1;
+    p.num_projection = 0;
+    p.zoneout_cell = zoneout_cell;
+    p.zoneout_output = zoneout_output;
+    p.bi_direction = false;
+    p.forget_bias = forget_bias;
+    p.activation_type = ACTIVATION_TANH;
+    TensorDesc xDesc = tensor2df(DT_F32, DF_NORMAL, batch, xdim);
+    TensorDesc hDesc = tensor2df(DT_F32, DF_NORMAL, batch, hdim);
+    TensorDesc fDesc = tensor2df(DT_I8, DF_NKN32, N, K);
+    TensorDesc bDesc = tensor1d(DT_F32, N);
+    const void *filters[2] = {blob, nullptr};
+    const void *biases[2] = {bias, nullptr};
+    U32 tmpBytes = (K + N) * 4 + K + 256;
+    void *tmp = calloc(tmpBytes, 1);
+    // out_stride doubles as batchStrideH, so the reference reads bias row m at m * (out_stride / hdim) * N
+    e = lstmcell_int8(xDesc, x, &fDesc, filters, &bDesc, biases, scale, state, tmpBytes, tmp, p, x_stride, out_stride,
+        hDesc, out, X86_AVX512);
+    free(tmp);
+    free(blob);
+    return e;
+}
+
 }  // extern "C"
