@@ -657,7 +657,22 @@ __global__ void requantize_i8_kernel(const int8_t *__restrict__ in, uint32_t n, 
 
 hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float r, int8_t *out, hipStream_t st)
 {
-    hipLaunchKernelGGL(requantize_i8_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, in, n, r, out);
+    // 16 bytes per lane through the concatenation kernel (one row) where both pointers allow it; the last
+    // n % 16 bytes, or everything when a pointer is not 16-byte aligned, one byte per lane
+    uint32_t body = 0;
+    if ((((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+        body = n & ~15u;
+        if (body) {
+            hipError_t e = launch_concat_i8(in, out, 1, body, body, 1, r, st);
+            if (e != hipSuccess) {
+                return e;
+            }
+        }
+    }
+    if (n > body) {
+        hipLaunchKernelGGL(requantize_i8_kernel, dim3(grid_for(n - body, 4, 256, 8192)), dim3(256), 0, st, in + body,
+            n - body, r, out + body);
+    }
     return hipGetLastError();
 }
 

@@ -178,6 +178,20 @@ def test_requantize(torch_mod, oracle):
             assert np.array_equal(back(host.requantize(buf, si, so)), oracle.requantize(x, si, so)), (si, so)
 
 
+def test_requantize_ragged_and_unaligned(torch_mod, oracle):
+    """Lengths that leave a tail behind the 16-byte body, and a device pointer that is not 16-byte aligned."""
+    torch = torch_mod
+    rng = np.random.default_rng(12)
+    for n in (1, 15, 16, 17, 4099, 65536 + 3):
+        x = rng.integers(-128, 128, size=n, dtype=np.int8)
+        want = oracle.requantize(x, 5.0, 3.5)
+        assert np.array_equal(host.requantize(x, 5.0, 3.5), want)
+        big = torch.from_numpy(np.concatenate([np.zeros(3, np.int8), x])).cuda()
+        got = host.requantize(big[3:], 5.0, 3.5)
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        assert np.array_equal(got.cpu().numpy(), want)
+
+
 def test_roundtrip_properties_at_full_size(torch_mod):
     """Size-independent properties at the BERT FFN activation size (4096 x 3072): the extreme value
     maps to 1 / 255, zero maps to 128, quantize is monotone, and dequantize(quantize(x)) is within
