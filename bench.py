@@ -376,6 +376,13 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         tmp = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
         t = timed(lambda: host_lstm.lstmcell(xl, blob, bl, [-1.0, 250.0], stl, pl, batch, xdim, ol, tmp=tmp), 30)
         per_row = 4 * hdim * (xdim + hdim) + 4 * (xdim + 2 * hdim + 4 * hdim + 2 * hdim + hdim)
+        blob2 = host_lstm.rnn_transform_filter(Wl, 4 * hdim, xdim + hdim, pl)
+        t2 = timed(lambda: host_lstm.lstmcell(xl, blob2, bl, [-1.0, 250.0], stl, pl, batch, xdim, ol, tmp=tmp,
+                                              both_packings=True), 50)
+        res["lstmcell_int8_decode_matrix_cores"] = {
+            "config": "same call with a weight that also carries the GEMM packing: the 256 rows go through the matrix "
+                      "cores as one product that reads the weight once (same bytes out)",
+            "ms": t2, "rows_per_s": batch / (t2 * 1e-3), "int8_tops": 2.0 * batch * 4 * hdim * (xdim + hdim) / t2 / 1e9}
         res["lstmcell_int8_decode"] = {"config": "256 rows, x 2048, h 2048 (weight 8192 x 4096 s8, read once per row)",
                                        "ms": t, "rows_per_s": batch / (t * 1e-3), "algorithmic_bytes": batch * per_row,
                                        "gbps": batch * per_row / t / 1e6,

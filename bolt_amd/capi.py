@@ -129,7 +129,7 @@ class RNNParamSpec(C.Structure):
 
 
 assert C.sizeof(RNNParamSpec) == 36
-RNN_LSTM, ACTIVATION_TANH, DF_NKN32 = 1, 6, 19
+RNN_LSTM, ACTIVATION_TANH, DF_NKN32, DF_NKNx_NKN32 = 1, 6, 19, 40
 
 
 _vp, _u32, _f32p, _u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
@@ -196,6 +196,8 @@ SIGNATURES = {
     "concat_gfx950": (C.c_int, [_u32, _TDp, C.POINTER(_vp), _f32p, ConcatParamSpec, _vp, TensorDesc, _vp, _f32p,
                                 C.c_int]),
     "rnncell_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, RNNParamSpec, _u32p, C.c_int]),
+    "rnn_transform_filter_bytes_gfx950": (C.c_int, [TensorDesc, RNNParamSpec, _u32p, C.c_int]),
+    "rnn_transform_filter_gfx950": (C.c_int, [TensorDesc, _vp, RNNParamSpec, _TDp, _vp, C.c_int]),
     "rnncell_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, C.POINTER(_vp), _TDp, C.POINTER(_vp), _f32p, _vp, _u32, _vp,
                                  RNNParamSpec, _u32, _u32, TensorDesc, _vp, C.c_int]),
     "bolt_gfx950_encoder_layer_int8_workspace_bytes": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),

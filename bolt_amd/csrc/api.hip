@@ -71,6 +71,8 @@ int g_bnn_mfma = 2;
 // int8 convolution through the filter-panel kernel: gather from the caller's tensor in place for int32 / fp32 results
 // (1, default) or for every result type (2); 0 = always re-lay the input as a padded s8 image first
 int g_conv_direct = 1;
+// LSTM cell: from this many batch rows on, a weight that carries the GEMM packing goes through the matrix cores
+int g_lstm_gemm_rows = 4;
 // dynamic quantisation through the public entry points: 1 = one launch that reads the tensor once where
 // it fits (default), 0 = always the two-pass form (scratch fill, abs-max, quantise)
 int g_quantize_fused = 1;
@@ -392,6 +394,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         g_bnn_mfma = value;
+        return SUCCESS;
+    }
+    if (strcmp(name, "lstm_gemm_rows") == 0) {
+        if (value < 1) {
+            return NOT_MATCH;
+        }
+        g_lstm_gemm_rows = value;
         return SUCCESS;
     }
     if (strcmp(name, "quantize_fused") == 0) {
@@ -2535,6 +2544,76 @@ EE lstm_shape(TensorDesc xDesc, RNNParamSpec p, LstmShape *s)
 }
 }  // namespace
 
+// Cell weight for both routes: [matrix-vector blob | the same matrix in the GEMM's packed layout]
+EE rnn_transform_filter_bytes_gfx950(TensorDesc filterDesc, RNNParamSpec p, U32 *bytes, Arch arch)
+{
+    (void)p;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    DataType dt;
+    DataFormat df;
+    U32 N, K;
+    if (get2d(filterDesc, &dt, &df, &N, &K) != SUCCESS || dt != DT_I8) {
+        return NOT_MATCH;
+    }
+    if (df == DF_NKNx_NKN32) {
+        *bytes = 0;   // already transformed
+        return SUCCESS;
+    }
+    const size_t b = 2 * (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4;
+    if (b > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)b;
+    return SUCCESS;
+}
+
+EE rnn_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, RNNParamSpec p, TensorDesc *ftmDesc,
+    void *filterTransformed, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!filter || !ftmDesc || !filterTransformed) {
+        return NULL_POINTER;
+    }
+    DataType dt;
+    DataFormat df;
+    U32 N, K;
+    if (get2d(filterDesc, &dt, &df, &N, &K) != SUCCESS || dt != DT_I8 || df != DF_NORMAL) {
+        return NOT_MATCH;   // s8 [4 * num_outputs][xDim + num_outputs], row-major
+    }
+    if (p.mode != RNN_LSTM || p.num_projection > 0 || N != 4 * p.num_outputs) {
+        return NOT_SUPPORTED;
+    }
+    const size_t mat = packed_matrix_bytes(N, K), mvmB = mat + (size_t)N * 4;
+    *ftmDesc = tensor2df(DT_I8, DF_NKNx_NKN32, N, K);
+    if (N == 0 || K == 0) {
+        return SUCCESS;
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    U8 *dst = (U8 *)filterTransformed;
+    if (arch == AMD_GFX950) {
+        std::vector<I32> comp(N);
+        pack_host(false, (const INT8 *)filter, 1, K, K, N, (INT8 *)dst, (I32 *)(dst + mat));
+        pack_host(true, (const INT8 *)filter, 1, K, K, N, (INT8 *)(dst + mvmB), comp.data());
+        return SUCCESS;
+    }
+    // the GEMM packing's compensation vector is the same as the matrix-vector one: it lands there twice
+    HIP_TRY(launch_pack_mvm((const int8_t *)filter, 1, K, K, N, (int8_t *)dst, (int32_t *)(dst + mat), c.stream));
+    HIP_TRY(launch_pack_mmm((const int8_t *)filter, 1, K, K, N, (int8_t *)(dst + mvmB), (int32_t *)(dst + mat),
+        c.stream));
+    return SUCCESS;
+}
+
 EE rnncell_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
     RNNParamSpec p, U32 *bytes, Arch arch)
 {
@@ -2580,6 +2659,9 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
     if (get2d(filterDesc[0], &fdt, &fdf, &fn, &fk) != SUCCESS || get2d(hDesc, &odt, &odf, &on, &oh) != SUCCESS) {
         return NOT_MATCH;
     }
+    if (fdf != DF_NKN32 && fdf != DF_NKNx_NKN32) {
+        return NOT_MATCH;   // lstm.cpp:54-56
+    }
     if (xDesc.dt != DT_F32 || fdt != DT_I8 || odt != DT_F32 || fn != s.N || fk != s.K || on != s.batch || oh != s.hDim) {
         return NOT_MATCH;   // lstm.cpp:65-70 (an fp32 filter is another back end's)
     }
@@ -2609,7 +2691,8 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
     }
     Ctx &c = ctx();
     Stage st;
-    const size_t blobB = (size_t)packed_matrix_bytes(s.N, s.K) + (size_t)s.N * 4;
+    const size_t blobB = (size_t)packed_matrix_bytes(s.N, s.K) + (size_t)s.N * 4;   // matrix-vector part
+    const size_t filterB = blobB + (fdf == DF_NKNx_NKN32 ? (size_t)packed_matrix_bytes(s.N, s.K) : 0);
     const size_t stateB = (size_t)s.batch * 2 * s.hDim * 4;
     bg::LstmArgs a;
     a.batch = s.batch;
@@ -2626,7 +2709,7 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
         // host pointers: rows are gathered into compact device copies
         float *dx = (float *)st.get((size_t)s.batch * std::max<U32>(s.xDim, 1) * 4);
         float *db = (float *)st.get((size_t)s.batch * s.N * 4);
-        void *w = st.get(blobB);
+        void *w = st.get(filterB);
         dState = (float *)st.get(stateB);
         dOut = (float *)st.get((size_t)s.batch * s.hDim * 4);
         dT = (U8 *)st.get(s.total);
@@ -2641,7 +2724,7 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
             HIP_TRY(hipMemcpyAsync(db + (size_t)m * s.N, (const float *)bias[0] + m * biasStride, (size_t)s.N * 4,
                 hipMemcpyHostToDevice, c.stream));
         }
-        HIP_TRY(hipMemcpyAsync(w, filter[0], blobB, hipMemcpyHostToDevice, c.stream));
+        HIP_TRY(hipMemcpyAsync(w, filter[0], filterB, hipMemcpyHostToDevice, c.stream));
         HIP_TRY(hipMemcpyAsync(dState, state, stateB, hipMemcpyHostToDevice, c.stream));
         dW = w;
         a.x = dx;
@@ -2665,6 +2748,28 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
     float *scaleW = (float *)(dT + s.scaleWOff);
     float *inter = (float *)(dT + s.interOff);
     a.inter = inter;
+    if (fdf == DF_NKNx_NKN32 && s.batch >= (U32)g_lstm_gemm_rows) {
+        // enough rows to share one pass over the weight: all rows through the matrix cores as one GEMM with exact
+        // int32 results; the gates kernel dequantises them with each row's own scale, in the arithmetic of the
+        // matrix-vector epilogue
+        HIP_TRY(bg::launch_lstm_xh_quant(a, c.stream));
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = a.quant;
+        g.lda = s.K;
+        g.Bp = (const int8_t *)dW + blobB;
+        g.M = s.batch;
+        g.N = s.N;
+        g.K = s.K;
+        g.comp = (const int32_t *)((const U8 *)dW + packed_matrix_bytes(s.N, s.K));
+        g.ob = g.comp;
+        g.C = inter;
+        g.epi.mode = EPI_I32;
+        HIP_TRY(launch_gemm_u8s8(g, c.stream));
+        a.acc_i32 = 1;
+        a.scale_w = scale[1];
+        HIP_TRY(bg::launch_lstm_gates(a, c.stream));
+    } else {
     uint32_t wbits;
     memcpy(&wbits, &scale[1], 4);
     HIP_TRY(bg::launch_fill_u32((uint32_t *)scaleW, s.N, wbits, c.stream));
@@ -2674,6 +2779,7 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
         return e;
     }
     HIP_TRY(bg::launch_lstm_gates(a, c.stream));
+    }
     if (arch == AMD_GFX950) {
         HIP_TRY(hipMemcpyAsync(state, dState, stateB, hipMemcpyDeviceToHost, c.stream));
         for (U32 m = 0; m < s.batch; ++m) {

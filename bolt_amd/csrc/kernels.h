@@ -205,7 +205,10 @@ struct LstmArgs {
     float scale_in = 0;            // caller's activation scale; <= 0: dynamic per row
     uint8_t *quant = nullptr;      // [batch][xdim + hdim]
     float *dscale = nullptr;       // [batch]
-    const float *inter = nullptr;  // [batch][4 * column] products
+    const float *inter = nullptr;  // [batch][4 * column] products: fp32, or (acc_i32) exact int32 sums still to be
+                                   // divided by dscale[m] * scale_w
+    int acc_i32 = 0;
+    float scale_w = 0;
     float *out = nullptr;          // row m at out + m * out_stride
     uint32_t out_stride = 0;
     float forget_bias = 0, zoneout_cell = 0, zoneout_output = 0;

@@ -57,10 +57,24 @@ __global__ __launch_bounds__(256) void lstm_gates_kernel(const LstmArgs a)
     }
     const float *g = a.inter + (size_t)m * 4 * a.column;
     const float *b = a.bias + (size_t)m * a.bias_stride;
-    const float gi = g[h] + b[h];
-    const float gg = g[h + a.column] + b[h + a.column];
-    const float gf = g[h + 2 * a.column] + b[h + 2 * a.column];
-    const float go = g[h + 3 * a.column] + b[h + 3 * a.column];
+    float p[4];
+    if (a.acc_i32) {
+        // the matrix-vector epilogue's arithmetic: cvt(acc) * (1 / (row scale * weight scale))
+        const float f = 1.0f / (a.dscale[m] * a.scale_w);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            p[k] = (float)((const int32_t *)g)[h + k * a.column] * f;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            p[k] = g[h + k * a.column];
+        }
+    }
+    const float gi = p[0] + b[h];
+    const float gg = p[1] + b[h + a.column];
+    const float gf = p[2] + b[h + 2 * a.column];
+    const float go = p[3] + b[h + 3 * a.column];
     float *stC = a.state + (size_t)m * (a.column + a.hdim);
     float *stH = stC + a.column;
     const float c0 = stC[h];

@@ -6,7 +6,7 @@ import ctypes as C
 import numpy as np
 
 from . import capi, host
-from .capi import (ACTIVATION_TANH, DF_NKN32, DF_NORMAL, DT_F32, DT_I8, RNN_LSTM, RNNParamSpec, TensorDesc, check, lib,
+from .capi import (ACTIVATION_TANH, DF_NKN32, DF_NKNx_NKN32, DF_NORMAL, DT_F32, DT_I8, RNN_LSTM, RNNParamSpec, TensorDesc, check, lib,
                    tensor1d, tensor2df)
 from .host import _empty_like_mode, arch_of, ptr
 
@@ -25,16 +25,30 @@ def transform_weight(W, N, K):
     return blob
 
 
-def lstmcell(x, blob, bias, scale, state, p, batch, xdim, out, x_stride=None, out_stride=None, tmp=None, fshape=None):
+def rnn_transform_filter(W, N, K, p):
+    """s8 [N][K] -> blob tagged DF_NKNx_NKN32: the matrix-vector blob followed by the GEMM packing."""
+    arch = arch_of(W)
+    desc = tensor2df(DT_I8, DF_NORMAL, N, K)
+    nbytes = C.c_uint32(0)
+    check(lib().rnn_transform_filter_bytes_gfx950(desc, p, C.byref(nbytes), arch), "rnn_transform_filter_bytes")
+    blob = _empty_like_mode(W, nbytes.value)
+    ftm = TensorDesc()
+    check(lib().rnn_transform_filter_gfx950(desc, ptr(W), p, C.byref(ftm), ptr(blob), arch), "rnn_transform_filter")
+    assert ftm.df == DF_NKNx_NKN32
+    return blob
+
+
+def lstmcell(x, blob, bias, scale, state, p, batch, xdim, out, x_stride=None, out_stride=None, tmp=None, fshape=None, both_packings=False):
     """One step for `batch` rows; `state` ([batch][C | H]) and `out` are updated in place. fshape: (rows, cols) the
-    filter descriptor declares, by default what `p` and xdim imply."""
+    filter descriptor declares, by default what `p` and xdim imply; both_packings: `blob` comes from
+    rnn_transform_filter."""
     hdim = p.num_outputs
     x_stride = xdim if x_stride is None else x_stride
     out_stride = hdim if out_stride is None else out_stride
     xdesc = tensor2df(DT_F32, DF_NORMAL, batch, xdim)
     hdesc = tensor2df(DT_F32, DF_NORMAL, batch, hdim)
     frows, fcols = fshape or (4 * hdim, xdim + hdim)
-    fdesc = (TensorDesc * 1)(tensor2df(DT_I8, DF_NKN32, frows, fcols))
+    fdesc = (TensorDesc * 1)(tensor2df(DT_I8, DF_NKNx_NKN32 if both_packings else DF_NKN32, frows, fcols))
     bdesc = (TensorDesc * 1)(tensor1d(DT_F32, 4 * hdim))
     arch = arch_of(state)
     nbytes = C.c_uint32(0)

@@ -56,7 +56,9 @@ const char *bolt_gfx950_last_error(void);
  * "bnn_mfma": how the 1-bit convolution runs: 2 (default) on the matrix cores
  * with its operands expanded to E2M1 pairs (v_mfma_scale_f32_16x16x128_f8f6f4) where the shape has
  * that kernel (256+ output channels, 128+ tiles of 256 pixels) and as 1 otherwise; 1 on the int8
- * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount). Every variant
+ * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount).
+ * "lstm_gemm_rows" (>= 1, default 4): the LSTM cell sends calls with at least this many batch rows through the
+ * matrix cores when its weight carries the GEMM packing (rnn_transform_filter_gfx950). Every variant
  * returns the same bytes. */
 EE bolt_gfx950_set_option(const char *name, int value);
 void *bolt_gfx950_malloc(size_t bytes);
@@ -246,7 +248,8 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
  *   xDesc        DT_F32 [batch, xDim]; row m of currentX starts at currentX + m * batchStrideX floats
  *   filterDesc[0] DT_I8 [4 * num_outputs, xDim + num_outputs], tagged DF_NKN32 as the reference does;
  *   filter[0]    the output of matrix_vector_multiply_transform_weight_gfx950 for that matrix (packed
- *                rows followed by the compensation vector, which is where the reference reads offsetC)
+ *                rows followed by the compensation vector, which is where the reference reads offsetC),
+ *                or, tagged DF_NKNx_NKN32, the output of rnn_transform_filter_gfx950 below
  *   bias[0]      DT_F32; row m reads 4 * num_outputs floats at bias[0] + m * steps * 4 * num_outputs with
  *                steps = batchStrideH / num_outputs / (bi_direction + 1), exactly as the reference
  *   scale        host F32[2] = {activation scale or <= 0 for dynamic, weight scale}; not written
@@ -259,6 +262,15 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
  * than ACTIVATION_TANH return NOT_SUPPORTED. */
 EE rnncell_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
     RNNParamSpec rnnParamSpec, U32 *bytes, Arch arch);
+/* rnn_transform_filter_bytes / rnn_transform_filter (compute/tensor/src/rnn.cpp:33-141) for the int8 LSTM weight:
+ * s8 [4 * num_outputs][xDim + num_outputs] row-major (DF_NORMAL) -> a blob tagged DF_NKNx_NKN32 that holds the
+ * matrix-vector blob above followed by the same matrix in the GEMM's packed layout. Given such a blob,
+ * rnncell_gfx950 sends a call with at least `lstm_gemm_rows` batch rows (option, default 4) through the matrix
+ * cores as ONE product that reads the weight once, instead of once per row; results are bit for bit those of
+ * the matrix-vector route (exact int32 sums, the same dequantisation arithmetic). */
+EE rnn_transform_filter_bytes_gfx950(TensorDesc filterDesc, RNNParamSpec rnnParamSpec, U32 *bytes, Arch arch);
+EE rnn_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, RNNParamSpec rnnParamSpec,
+    TensorDesc *ftmDesc, void *filterTransformed, Arch arch);
 EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filterDesc, const void **filter,
     const TensorDesc *biasDesc, const void **bias, F32 *scale, void *state, U32 tmpBytes, void *tmp,
     RNNParamSpec rnnParamSpec, U32 batchStrideX, U32 batchStrideH, TensorDesc hDesc, void *output, Arch arch);

@@ -124,3 +124,47 @@ def test_lstmcell_decode_shape_properties(torch_mod, oracle):
         host_lstm.lstmcell(put(x[m:m + 1].copy()), blob, put(bias[m:m + 1].copy()), [-1.0, W_SCALE], st1, p, 1, xdim, out1)
         capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
         assert torch.equal(out1[0], out[m]) and torch.equal(st1[0], st[m])
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+@pytest.mark.parametrize("shape", [(1, 48, 32), (4, 64, 64), (5, 100, 20), (9, 33, 36), (70, 40, 88), (300, 64, 64)])
+def test_lstmcell_gemm_route_returns_the_same_bits(torch_mod, oracle, shape, device_mode):
+    """A weight that carries the GEMM packing sends calls of 4+ rows through the matrix cores; outputs and states
+    must be the bytes of the matrix-vector route, and both within tolerance of the oracle."""
+    torch = torch_mod
+    batch, xdim, hdim = shape
+    print("lstm gemm route", shape, device_mode, flush=True)
+    x, W, bias, state = lstm_case(batch, xdim, hdim, 61)
+    put = (lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()) if device_mode else np.ascontiguousarray
+    p = host_lstm.lstm_param_spec(hdim, 1.0, 0.1, 0.2)
+    res = []
+    for both in (False, True):
+        blob = (host_lstm.rnn_transform_filter(put(W), 4 * hdim, xdim + hdim, p) if both
+                else host_lstm.transform_weight(put(W), 4 * hdim, xdim + hdim))
+        st, out = put(state.copy()), put(np.zeros((batch, hdim), np.float32))
+        host_lstm.lstmcell(put(x), blob, put(bias), [-1.0, W_SCALE], st, p, batch, xdim, out, both_packings=both)
+        if device_mode:
+            capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+            st, out = st.cpu().numpy(), out.cpu().numpy()
+        res.append((out, st))
+    assert res[0][0].tobytes() == res[1][0].tobytes() and res[0][1].tobytes() == res[1][1].tobytes()
+    want, wst = orc_lstmcell(oracle, x, W, bias, [-1.0, W_SCALE], state, hdim, 1.0, 0.1, 0.2)
+    assert np.abs(res[1][0] - want).max() <= TOL and np.abs(res[1][1] - wst).max() <= TOL
+
+
+def test_lstmcell_gemm_route_decode_shape(torch_mod):
+    """256 rows x 8192 x 4096 through both routes: identical bytes."""
+    torch = torch_mod
+    batch, xdim, hdim = 256, 2048, 2048
+    x, W, bias, state = lstm_case(batch, xdim, hdim, 78)
+    put = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    p = host_lstm.lstm_param_spec(hdim)
+    outs = []
+    for both in (False, True):
+        blob = (host_lstm.rnn_transform_filter(put(W), 4 * hdim, xdim + hdim, p) if both
+                else host_lstm.transform_weight(put(W), 4 * hdim, xdim + hdim))
+        st, out = put(state.copy()), torch.zeros((batch, hdim), device="cuda")
+        host_lstm.lstmcell(put(x), blob, put(bias), [-1.0, W_SCALE], st, p, batch, xdim, out, both_packings=both)
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        outs.append((out, st))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
