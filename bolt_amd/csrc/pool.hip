@@ -23,7 +23,9 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b)
 
 // The sixteen channels of a pixel as packed 16-bit lanes: lo[d] holds bytes 0 and 2 of dword d, hi[d]
 // bytes 1 and 3. 16-bit sums hold 257 taps of 255; WIDE keeps 32-bit sums for larger windows.
-template <bool MEAN, bool WIDE>
+// KS > 0: the window is at most KS x KS taps (KS = 2, 3): all of them are requested before any is used, taps
+// outside the clipped window re-read the first one and are masked out. KS = 0: any window, one tap at a time.
+template <bool MEAN, bool WIDE, int KS>
 __global__ __launch_bounds__(256) void pool_u8_c16_kernel(const PoolArgs a)
 {
     const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
@@ -55,6 +57,37 @@ __global__ __launch_bounds__(256) void pool_u8_c16_kernel(const PoolArgs a)
         }
     }
     uint32_t taps = 0;
+    if (KS > 0) {
+        uint4 v[KS > 0 ? KS * KS : 1];
+#pragma unroll
+        for (int y = 0; y < KS; ++y) {
+#pragma unroll
+            for (int x = 0; x < KS; ++x) {
+                const bool ok = (uint32_t)y < kh && (uint32_t)x < kw;
+                v[y * KS + x] = src[ok ? (size_t)y * a.IW + x : 0];
+            }
+        }
+#pragma unroll
+        for (int y = 0; y < KS; ++y) {
+#pragma unroll
+            for (int x = 0; x < KS; ++x) {
+                const uint32_t keep = ((uint32_t)y < kh && (uint32_t)x < kw) ? 0xffffffffu : 0u;
+                const uint32_t w4[4] = {v[y * KS + x].x & keep, v[y * KS + x].y & keep, v[y * KS + x].z & keep,
+                    v[y * KS + x].w & keep};
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t l = w4[d] & 0x00ff00ffu, h = (w4[d] >> 8) & 0x00ff00ffu;
+                    if (MEAN) {
+                        lo[d] += l;
+                        hi[d] += h;
+                    } else {
+                        lo[d] = pk_max_u16(lo[d], l);
+                        hi[d] = pk_max_u16(hi[d], h);
+                    }
+                }
+            }
+        }
+    } else {
     for (uint32_t y = 0; y < kh; ++y) {
         const uint4 *row = src + (size_t)y * a.IW;
         for (uint32_t x = 0; x < kw; ++x) {
@@ -83,6 +116,7 @@ __global__ __launch_bounds__(256) void pool_u8_c16_kernel(const PoolArgs a)
                 taps = 0;
             }
         }
+    }
     }
 
     uint32_t o4[4];
@@ -122,13 +156,26 @@ hipError_t launch_pool_u8_c16(const PoolArgs &a, hipStream_t st)
     }
     const dim3 grid((a.total + 255) / 256), block(256);
     const bool wide = a.kh * a.kw > 256;
+    const int ks = (a.kh <= 2 && a.kw <= 2) ? 2 : (a.kh <= 3 && a.kw <= 3) ? 3 : 0;
+#define BG_POOL(M, W, K) hipLaunchKernelGGL((pool_u8_c16_kernel<M, W, K>), grid, block, 0, st, a)
     if (!a.mean) {
-        hipLaunchKernelGGL((pool_u8_c16_kernel<false, false>), grid, block, 0, st, a);
+        if (ks == 2) {
+            BG_POOL(false, false, 2);
+        } else if (ks == 3) {
+            BG_POOL(false, false, 3);
+        } else {
+            BG_POOL(false, false, 0);
+        }
     } else if (wide) {
-        hipLaunchKernelGGL((pool_u8_c16_kernel<true, true>), grid, block, 0, st, a);
+        BG_POOL(true, true, 0);
+    } else if (ks == 2) {
+        BG_POOL(true, false, 2);
+    } else if (ks == 3) {
+        BG_POOL(true, false, 3);
     } else {
-        hipLaunchKernelGGL((pool_u8_c16_kernel<true, false>), grid, block, 0, st, a);
+        BG_POOL(true, false, 0);
     }
+#undef BG_POOL
     return hipGetLastError();
 }
 
