@@ -148,3 +148,52 @@ def test_error_codes_follow_the_reference():
     s = (C.c_float * 2)(1, 1)
     assert L.quantize_gfx950(tensor1d(DT_F32, 8), host.ptr(f), C.byref(qd2), host.ptr(x), C.cast(s, C.c_void_p), 0,
                              AMD_GFX950) == capi.NOT_SUPPORTED
+
+
+def test_pool_concat_lstm_argument_checks_and_size_queries():
+    """Shape validation and size queries of the pooling / concatenation / LSTM-cell entry points answer before
+    anything touches a GPU."""
+    from bolt_amd.capi import (AMD_GFX950, DF_NCHWC8, DF_NCHWC16, DF_NKNx_NKN32, DT_F32, POOLING_MAX, RNNParamSpec,
+                               pooling_param_spec, tensor4df)
+    from bolt_amd.host_lstm import lstm_param_spec
+    L = capi.lib()
+    buf = np.zeros(16 * 8 * 8, np.uint8)
+    vp = buf.ctypes.data
+    good = pooling_param_spec(POOLING_MAX, 2, 2, 2, 2, 0, 0, 0, 0)
+    d16, o16 = tensor4df(DT_U8_Q, DF_NCHWC16, 1, 16, 8, 8), tensor4df(DT_U8_Q, DF_NCHWC16, 1, 16, 4, 4)
+    assert L.pooling_gfx950(d16, vp, good, None, o16, vp, None, capi.X86_AVX512) == capi.NOT_SUPPORTED
+    assert L.pooling_gfx950(d16, None, good, None, o16, vp, None, AMD_GFX950) == capi.NULL_POINTER
+    assert L.pooling_gfx950(tensor4df(DT_U8_Q, DF_NCHWC8, 1, 16, 8, 8), vp, good, None, o16, vp, None,
+                            AMD_GFX950) == capi.NOT_MATCH
+    assert L.pooling_gfx950(tensor4df(DT_F32, DF_NCHWC16, 1, 16, 8, 8), vp, good, None, o16, vp, None,
+                            AMD_GFX950) == capi.NOT_SUPPORTED
+    pad = pooling_param_spec(POOLING_MAX, 2, 2, 2, 2, 2, 0, 0, 0)       # pad >= kernel (pooling_int8.cpp:352-354)
+    assert L.pooling_gfx950(d16, vp, pad, None, o16, vp, None, AMD_GFX950) == capi.NOT_SUPPORTED
+    far = tensor4df(DT_U8_Q, DF_NCHWC16, 1, 16, 9, 4)                    # a window that starts below the image
+    assert L.pooling_gfx950(d16, vp, good, None, far, vp, None, AMD_GFX950) == capi.NOT_SUPPORTED
+    # concat: tmp bytes are zero; extents that do not add up are refused before any launch
+    nb = C.c_uint32(7)
+    descs = (capi.TensorDesc * 2)(tensor4df(DT_I8, 0, 2, 3, 5, 7), tensor4df(DT_I8, 0, 2, 5, 5, 7))
+    assert L.concat_infer_forward_tmp_bytes_gfx950(2, descs, tensor4df(DT_I8, 0, 2, 8, 5, 7), C.byref(nb),
+                                                   AMD_GFX950) == capi.SUCCESS and nb.value == 0
+    ptrs = (C.c_void_p * 2)(vp, vp)
+    sc = (C.c_float * 2)(2.0, 3.0)
+    osc = C.c_float(0)
+    assert L.concat_gfx950(2, descs, ptrs, sc, capi.ConcatParamSpec(1, 2), None, tensor4df(DT_I8, 0, 2, 9, 5, 7), vp,
+                           C.byref(osc), AMD_GFX950) == capi.NOT_MATCH
+    assert osc.value == 2.0   # the common scale is the smallest input scale (concat.cpp:175-177)
+    # LSTM weight: matrix-vector blob + GEMM packing; a transformed descriptor needs no further bytes
+    p = lstm_param_spec(64)
+    N, K = 256, 96
+    assert L.rnn_transform_filter_bytes_gfx950(tensor2df(DT_I8, DF_NORMAL, N, K), p, C.byref(nb), AMD_GFX950) == capi.SUCCESS
+    assert nb.value == 2 * N * K + 4 * N
+    assert L.rnn_transform_filter_bytes_gfx950(tensor2df(DT_I8, DF_NKNx_NKN32, N, K), p, C.byref(nb),
+                                               AMD_GFX950) == capi.SUCCESS and nb.value == 0
+    xd, hd = tensor2df(DT_F32, DF_NORMAL, 3, 32), tensor2df(DT_F32, DF_NORMAL, 3, 64)
+    assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, N, K), hd, p, C.byref(nb),
+                                                    AMD_GFX950) == capi.SUCCESS and nb.value >= 3 * (K + 4 + 4 * N)
+    proj = lstm_param_spec(64)
+    proj.num_projection = 32
+    assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, N, K), hd, proj, C.byref(nb),
+                                                    AMD_GFX950) == capi.NOT_SUPPORTED
+    assert C.sizeof(RNNParamSpec) == 36
