@@ -2484,7 +2484,11 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
             return fail(ALLOC_FAILED, "device staging");
         }
     }
-    size_t off = 0;
+    // gather the inputs that take part; in host-pointer mode they are staged on the device first
+    std::vector<const void *> srcs;
+    std::vector<size_t> lens;
+    std::vector<float> factors;
+    std::vector<char> scaled;
     for (U32 j = 0; j < num; ++j) {
         if (!input[j] || tensorNumElements(inputDesc[j]) == 0) {
             continue;
@@ -2503,9 +2507,36 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
             src = d;
         }
         const bool rs = rescale && inputScale[j] != oscale;
-        HIP_TRY(bg::launch_concat_i8(src, dout + off, (uint32_t)loops, (uint32_t)len, ostride, rs ? 1 : 0,
-            rs ? oscale / inputScale[j] : 1.0f, c.stream));
-        off += len;
+        srcs.push_back(src);
+        lens.push_back(len);
+        factors.push_back(rs ? oscale / inputScale[j] : 1.0f);
+        scaled.push_back(rs ? 1 : 0);
+    }
+    bg::ConcatMulti cm;
+    if (srcs.size() <= 8) {
+        size_t off = 0;
+        for (size_t j = 0; j < srcs.size(); ++j) {
+            cm.in[j] = (const uint8_t *)srcs[j];
+            cm.len[j] = (uint32_t)lens[j];
+            cm.off[j] = off;
+            cm.r[j] = factors[j];
+            cm.rescale[j] = (uint8_t)scaled[j];
+            off += lens[j];
+        }
+        cm.num = (uint32_t)srcs.size();
+        cm.rows = (uint32_t)loops;
+        cm.ostride = ostride;
+        cm.out = dout;
+    }
+    if (cm.num && bg::concat_multi_fits(cm)) {
+        HIP_TRY(bg::launch_concat_i8_multi(cm, c.stream));
+    } else {
+        size_t off = 0;
+        for (size_t j = 0; j < srcs.size(); ++j) {
+            HIP_TRY(bg::launch_concat_i8(srcs[j], dout + off, (uint32_t)loops, (uint32_t)lens[j], ostride,
+                scaled[j], factors[j], c.stream));
+            off += lens[j];
+        }
     }
     if (arch == AMD_GFX950) {
         HIP_TRY(hipMemcpyAsync(output, dout, outB, hipMemcpyDeviceToHost, c.stream));

@@ -194,6 +194,20 @@ hipError_t launch_pool_u8_c16(const PoolArgs &a, hipStream_t st);
 hipError_t launch_concat_i8(const void *in, void *out, uint32_t rows, uint32_t len, size_t ostride, int rescale,
     float r, hipStream_t st);
 
+// All inputs of a concatenation in one launch (at most 8, everything 16-byte aligned: concat_multi_fits)
+struct ConcatMulti {
+    const uint8_t *in[8] = {};
+    uint32_t len[8] = {};      // bytes per row of input j
+    size_t off[8] = {};        // where input j starts inside an output row
+    float r[8] = {};
+    uint8_t rescale[8] = {};
+    uint32_t num = 0, rows = 0;
+    size_t ostride = 0;
+    uint8_t *out = nullptr;
+};
+bool concat_multi_fits(const ConcatMulti &a);
+hipError_t launch_concat_i8_multi(const ConcatMulti &a, hipStream_t st);
+
 // ---- int8 LSTM cell (lstm.hip) ----------------------------------------------------------------------
 struct LstmArgs {
     uint32_t batch = 0, xdim = 0, hdim = 0, column = 0;   // column = hdim when there is no projection

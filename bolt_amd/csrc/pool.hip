@@ -247,4 +247,54 @@ hipError_t launch_concat_i8(const void *in, void *out, uint32_t rows, uint32_t l
     return hipGetLastError();
 }
 
+// Up to eight inputs in ONE launch: blockIdx.y selects the input. Every length, offset, the stride and every
+// pointer are multiples of 16 bytes (the launcher checks), so each lane moves 16 bytes.
+__global__ __launch_bounds__(256) void concat_i8_multi_kernel(const ConcatMulti a)
+{
+    const uint32_t j = blockIdx.y;
+    const uint32_t per_row = a.len[j] / 16;
+    const size_t total = (size_t)a.rows * per_row;
+    const size_t step = (size_t)gridDim.x * 256u;
+    const v4i *in = (const v4i *)a.in[j];
+    uint8_t *out = a.out + a.off[j];
+    const float r = a.r[j];
+    const bool scale = a.rescale[j] != 0;
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < total; i += step) {
+        const uint32_t row = (uint32_t)(i / per_row), col = (uint32_t)(i % per_row);
+        v4i v = __builtin_nontemporal_load(in + i);
+        if (scale) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                v[d] = (int)rescale4((uint32_t)v[d], r);
+            }
+        }
+        __builtin_nontemporal_store(v, (v4i *)(out + (size_t)row * a.ostride) + col);
+    }
+}
+
+bool concat_multi_fits(const ConcatMulti &a)
+{
+    if (a.num == 0 || a.num > 8 || a.rows == 0 || (a.ostride & 15) || ((uintptr_t)a.out & 15)) {
+        return false;
+    }
+    for (uint32_t j = 0; j < a.num; ++j) {
+        if (a.len[j] == 0 || (a.len[j] & 15) || (a.off[j] & 15) || ((uintptr_t)a.in[j] & 15)) {
+            return false;
+        }
+    }
+    return true;
+}
+
+hipError_t launch_concat_i8_multi(const ConcatMulti &a, hipStream_t st)
+{
+    uint32_t longest = 0;
+    for (uint32_t j = 0; j < a.num; ++j) {
+        longest = std::max(longest, a.len[j]);
+    }
+    const size_t total = (size_t)a.rows * (longest / 16);
+    const uint32_t blocks = (uint32_t)std::min<size_t>((total + 255) / 256, 256 * 64 / a.num + 1);
+    hipLaunchKernelGGL(concat_i8_multi_kernel, dim3(blocks, a.num), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
 }  // namespace bg
