@@ -208,10 +208,16 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                             "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
             del A, W, blob, tmp, out
         rate = {}
-        for key, zero in (("random_operands_tops", 0), ("zero_operands_tops", 1)):
-            v = C.c_float(0)
-            capi.check(L.bolt_gfx950_mfma_int8_rate(zero, C.byref(v)), "mfma_int8_rate")
-            rate[key] = v.value
+        probe_so = os.path.join(ROOT, "bolt_amd", "libbolt_gfx950_benchprobe.so")   # bench-only library, not the product
+        if os.path.exists(probe_so):
+            P = C.CDLL(probe_so)
+            P.bench_probe_mfma_int8_rate.argtypes = [C.c_int, C.POINTER(C.c_float)]
+            torch.cuda.synchronize()
+            for key, zero in (("random_operands_tops", 0), ("zero_operands_tops", 1)):
+                v = C.c_float(0)
+                if P.bench_probe_mfma_int8_rate(zero, C.byref(v)) != 0:
+                    raise RuntimeError("bench_probe_mfma_int8_rate failed")
+                rate[key] = v.value
         rate["note"] = ("v_mfma_i32_16x16x64_i8 back to back from registers, 8 waves per CU, no memory traffic: the device "
                         "lowers its clock when the operand bits are random")
         res["gemm_int8_8192_by_operand_data"] = by_data

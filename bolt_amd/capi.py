@@ -145,7 +145,12 @@ class BoltEncoderLayerInt8(C.Structure):
 
 SIGNATURES = {
     "bolt_gfx950_init": (C.c_int, []),
-    "bolt_gfx950_mfma_int8_rate": (C.c_int, [C.c_int, C.POINTER(C.c_float)]),
+    "vector_vector_axpby_gfx950": (C.c_int, [C.c_float, TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_int]),
+    "convolution_infer_output_size_gfx950": (C.c_int, [TensorDesc, TensorDesc, ConvolutionParamSpec, _TDp, C.c_int,
+                                                       C.c_int]),
+    "convolution_infer_forward_algorithm_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, ConvolutionParamSpec,
+                                                             C.c_int, C.POINTER(C.c_int), C.c_int, ActivationParamSpec,
+                                                             C.c_int]),
     "bolt_gfx950_set_stream": (C.c_int, [_vp]),
     "bolt_gfx950_synchronize": (C.c_int, []),
     "bolt_gfx950_last_error": (C.c_char_p, []),

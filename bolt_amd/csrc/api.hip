@@ -495,50 +495,50 @@ EE bolt_gfx950_timer_stop(float *ms)
     return SUCCESS;
 }
 
-EE bolt_gfx950_mfma_int8_rate(int zero_operands, float *tops)
+// ---- axpby ---------------------------------------------------------------------------------------
+// y = a * x + b * y (compute/blas_enhance/src/axpby.cpp:24-60). The x86 build supports DT_F32 only.
+EE vector_vector_axpby_gfx950(F32 a, TensorDesc xDesc, const void *x, F32 b, TensorDesc yDesc, void *y, Arch arch)
 {
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!x || !y) {
+        return NULL_POINTER;
+    }
+    DataType xdt, ydt;
+    U32 xn, yn;
+    if (get1d(xDesc, &xdt, &xn) != SUCCESS || get1d(yDesc, &ydt, &yn) != SUCCESS || xdt != ydt || xn != yn) {
+        return NOT_MATCH;
+    }
+    if (xdt != DT_F32) {
+        return NOT_SUPPORTED;
+    }
+    if (xn == 0) {
+        return SUCCESS;
+    }
     EE e = ensure_init();
     if (e != SUCCESS) {
         return e;
     }
-    if (!tops) {
-        return fail(NULL_POINTER, "mfma_int8_rate: tops is null");
-    }
     Ctx &c = ctx();
-    int dev = 0, cus = 0;
-    HIP_TRY(hipGetDevice(&dev));
-    HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    const uint32_t blocks = (uint32_t)cus;
-    const uint32_t iters = 8000;  // 2 waves per SIMD x 8000 x 32 x 16 cycles: a few milliseconds
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    float best = 0.0f;
-    hipError_t err = launch_mfma_i8_rate(blocks, iters / 8, zero_operands, nullptr, c.stream);  // warm-up
-    for (int r = 0; r < 3 && err == hipSuccess; ++r) {
-        float ms = 0.0f;
-        err = hipEventRecord(e0, c.stream);
-        if (err == hipSuccess) {
-            err = launch_mfma_i8_rate(blocks, iters, zero_operands, nullptr, c.stream);
+    if (arch == AMD_GFX950_DEVICE) {
+        if (!aligned4(x) || !aligned4(y)) {
+            return fail(NOT_SUPPORTED, "device x / y must be 4-byte aligned");
         }
-        if (err == hipSuccess) {
-            err = hipEventRecord(e1, c.stream);
-        }
-        if (err == hipSuccess) {
-            err = hipEventSynchronize(e1);
-        }
-        if (err == hipSuccess) {
-            err = hipEventElapsedTime(&ms, e0, e1);
-        }
-        if (err == hipSuccess && (best == 0.0f || ms < best)) {
-            best = ms;
-        }
+        HIP_TRY(launch_axpby_f32(xn, a, (const float *)x, b, (float *)y, c.stream));
+        return SUCCESS;
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    HIP_TRY(err);
-    const double ops = (double)blocks * 8.0 * (double)iters * 32.0 * (2.0 * 16 * 16 * 64);
-    *tops = (float)(ops / ((double)best * 1e-3) / 1e12);
+    Stage st;
+    const size_t bytes = (size_t)xn * 4;
+    void *dx = st.get(bytes), *dy = st.get(bytes);
+    if (!dx || !dy) {
+        return fail(ALLOC_FAILED, "device staging");
+    }
+    HIP_TRY(hipMemcpyAsync(dx, x, bytes, hipMemcpyHostToDevice, c.stream));
+    HIP_TRY(hipMemcpyAsync(dy, y, bytes, hipMemcpyHostToDevice, c.stream));
+    HIP_TRY(launch_axpby_f32(xn, a, (const float *)dx, b, (float *)dy, c.stream));
+    HIP_TRY(hipMemcpyAsync(y, dy, bytes, hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
     return SUCCESS;
 }
 
@@ -992,11 +992,17 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     } else if (!aligned4(data) && ddt != DT_U8_Q) {
         return fail(NOT_SUPPORTED, "device data must be 4-byte aligned");
     }
-    float *dscale = c.hscale_dev;
+    // Only a call that returns a freshly computed scale lets its kernel write the pinned word (and waits for it
+    // below). A static-scale kernel that wrote it too would do so at some later time, without the host waiting,
+    // and could land its value after the NEXT call has armed the word.
+    float *dscale = nullptr;
     bool read_back = false;
-    arm_scale(c);
     if (f32in) {
         const bool dynamic = (!mode || *scale <= 0);
+        if (dynamic) {
+            arm_scale(c);
+            dscale = c.hscale_dev;
+        }
         bool fused = false;
         if (dynamic && g_quantize_fused) {  // one launch, one read, where the tensor fits a resident grid's registers
             HIP_TRY(launch_quantize_fused(dIn, n, dOut, 0, qdt == DT_U8_Q, c.fsync, *scale, dscale, c.stream, &fused));
@@ -1014,6 +1020,10 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     } else {
         const bool dynamic = (scale[0] < 0 && scale[1] > 0);
         bool fused = false;
+        if (dynamic) {
+            arm_scale(c);
+            dscale = c.hscale_dev;
+        }
         if (dynamic && g_quantize_fused) {
             HIP_TRY(launch_quantize_fused(dIn, n, dOut, 1, qdt == DT_U8_Q, c.fsync, scale[1], dscale, c.stream, &fused));
         }
@@ -1444,7 +1454,8 @@ EE conv_shape(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc
     if (p.group != 1) {
         return NOT_SUPPORTED;  // depthwise / grouped int8 convolution is a different reference kernel
     }
-    if (fc != s->ic || on != s->n || s->ic % 8 != 0 || s->oc % 8 != 0) {
+    // a transformed filter's desc carries the channel count rounded up to 16 (convolution_transform.cpp:70-87)
+    if ((fc != s->ic && fc != align_up(s->ic, 16)) || on != s->n || s->ic % 8 != 0 || s->oc % 8 != 0) {
         return NOT_MATCH;
     }
     s->sh = p.stride_h;
@@ -1596,6 +1607,88 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
 
 }  // namespace
 
+EE convolution_infer_output_size_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, ConvolutionParamSpec p,
+    TensorDesc *outputDesc, DataType targetDataType, Arch arch)
+{
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!outputDesc) {
+        return NULL_POINTER;
+    }
+    U32 in, ic, ih, iw, fn, fc, fh, fw;
+    if (get4d(inputDesc, &in, &ic, &ih, &iw) != SUCCESS || get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS) {
+        return NOT_SUPPORTED;  // 5-D (3-D convolution) is not on the int8 path
+    }
+    EE ret = SUCCESS;
+    if (fh < 1 || fw < 1) {
+        ret = NOT_SUPPORTED;
+    }
+    const U32 dh = p.dilatedRate_h ? p.dilatedRate_h : 1, dw = p.dilatedRate_w ? p.dilatedRate_w : 1;
+    if (p.stride_h == 0 || p.stride_w == 0) {
+        return NOT_MATCH;
+    }
+    const I32 fhD = (I32)((fh - 1) * dh + 1), fwD = (I32)((fw - 1) * dw + 1);
+    I32 oh, ow;
+    switch (p.round_mode) {  // convolution.cpp:62-82
+        case ROUND_SAME_UPPER:
+            oh = (I32)((ih + p.stride_h - 1) / p.stride_h);
+            ow = (I32)((iw + p.stride_w - 1) / p.stride_w);
+            break;
+        case ROUND_SAME_LOWER:
+            oh = (I32)(ih / p.stride_h);
+            ow = (I32)(iw / p.stride_w);
+            break;
+        default: {
+            // unsigned arithmetic like the reference's (U32 operands): a window larger than the padded image wraps
+            const U32 th = ih + p.pad_top + p.pad_bottom - (U32)fhD, tw = iw + p.pad_left + p.pad_right - (U32)fwD;
+            oh = (I32)(th / p.stride_h + 1);
+            ow = (I32)(tw / p.stride_w + 1);
+            break;
+        }
+    }
+    if (oh < 0 || ow < 0) {
+        ret = NOT_MATCH;
+    }
+    if (fn % 8 != 0) {
+        return NOT_SUPPORTED;  // :93-95
+    }
+    DataFormat odf = DF_NCHWC8;
+    if (targetDataType == DT_U8_Q && fn != 8) {
+        odf = DF_NCHWC16;  // :97-101
+    }
+    *outputDesc = tensor4df(targetDataType, odf, in, fn, (U32)oh, (U32)ow);
+    return ret;
+}
+
+EE convolution_infer_forward_algorithm_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec p, ConvolutionPolicy policy, ConvolutionForwardAlgorithm *algorithm, DataType targetDataType,
+    ActivationParamSpec activationDesc, Arch arch)
+{
+    (void)outputDesc;
+    (void)p;
+    (void)policy;
+    (void)activationDesc;
+    if (!IS_GFX950(arch)) {
+        return NOT_SUPPORTED;
+    }
+    if (!algorithm) {
+        return NULL_POINTER;
+    }
+    if (*algorithm != CONVOLUTION_ALGORITHM_NULL) {
+        return SUCCESS;  // cpu/x86/convolution.cpp:39-41
+    }
+    if (targetDataType != DT_U8_Q && targetDataType != DT_I8) {
+        return NOT_SUPPORTED;  // only the quantised convolution runs here
+    }
+    U32 in, ic, ih, iw, fn, fc, fh, fw;
+    if (get4d(inputDesc, &in, &ic, &ih, &iw) != SUCCESS || get4d(filterDesc, &fn, &fc, &fh, &fw) != SUCCESS) {
+        return NOT_SUPPORTED;
+    }
+    *algorithm = (fh == 1 && fw == 1) ? CONVOLUTION_ALGORITHM_POINTWISE : CONVOLUTION_ALGORITHM_DIRECT;  // :79-82, :101
+    return SUCCESS;
+}
+
 EE convolution_transform_filter_bytes_gfx950(TensorDesc filterDesc, ConvolutionParamSpec p,
     ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch)
 {
@@ -1650,6 +1743,7 @@ EE convolution_transform_filter_gfx950(TensorDesc filterDesc, const void *filter
     }
     *ftmDesc = filterDesc;
     ftmDesc->df = DF_NCHWC2NxC4;  // convolution_transform.cpp:207-211
+    ftmDesc->dims[2] = s.ICp;      // channels rounded up to the 16 of the packed layout (:70-87)
     return SUCCESS;
 }
 

@@ -163,6 +163,7 @@ hipError_t launch_dequant_u8(const uint8_t *q, uint32_t n, const float *dscale, 
 hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *offsetC, const float *dscaleA,
     float scaleB, int32_t *out, hipStream_t st);
 hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float rescale, int8_t *out, hipStream_t st);
+hipError_t launch_axpby_f32(uint32_t n, float a, const float *x, float b, float *y, hipStream_t st);  // y = fma(a, x, y * b)
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
 // One-launch dynamic quantisation (quantize.hip): device sync area and the host's running epoch / arrival target
 struct FusedSync {
@@ -174,8 +175,6 @@ struct FusedSync {
 constexpr size_t kFusedSyncBytes = 64 * 64 + 64 + 64 * 64;
 hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
     float *ds_out, hipStream_t st, bool *taken);
-// probe.hip: register-resident int8 MFMA loop, blocks x 8 waves x iters x 32 instructions
-hipError_t launch_mfma_i8_rate(uint32_t blocks, uint32_t iters, int zero, int *sink, hipStream_t st);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]
 
 // ---- u8 pooling and s8 concatenation (pool.hip) ---------------------------------------------------

@@ -562,6 +562,36 @@ hipError_t launch_u8_to_i8(const uint8_t *x, uint32_t n, int8_t *q, hipStream_t 
     return hipGetLastError();
 }
 
+// y = a * x + b * y in fp32 (compute/blas_enhance/src/cpu/x86/fp32/axpby.cpp:16-34): the vector body there is
+// fmadd(a, x, y * b) -- one multiply rounded, then one fused multiply-add.
+__global__ __launch_bounds__(256) void axpby_f32_kernel(uint32_t n, float a, const float *__restrict__ x, float b,
+    float *__restrict__ y)
+{
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    uint32_t done = 0;
+    if ((((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
+        const uint32_t n4 = n / 4;
+        const v4f *x4 = (const v4f *)x;
+        v4f *y4 = (v4f *)y;
+        for (uint32_t i = tid; i < n4; i += stride) {
+            const v4f u = x4[i], v = y4[i];
+            y4[i] = (v4f){__builtin_fmaf(a, u.x, v.x * b), __builtin_fmaf(a, u.y, v.y * b), __builtin_fmaf(a, u.z, v.z * b),
+                __builtin_fmaf(a, u.w, v.w * b)};
+        }
+        done = n4 * 4;
+    }
+    for (uint32_t i = done + tid; i < n; i += stride) {
+        y[i] = __builtin_fmaf(a, x[i], y[i] * b);
+    }
+}
+
+hipError_t launch_axpby_f32(uint32_t n, float a, const float *x, float b, float *y, hipStream_t st)
+{
+    hipLaunchKernelGGL(axpby_f32_kernel, dim3(grid_for(n, 4, 256, 8192)), dim3(256), 0, st, n, a, x, b, y);
+    return hipGetLastError();
+}
+
 // ---- dequantize: avx512/dequantize.cpp:18-101, f = cvt(q) * (1 / s) -----------------------------
 __global__ __launch_bounds__(256) void dequant_i32_kernel(const int32_t *__restrict__ q, uint32_t n, const float *__restrict__ ds,
     float s, float *__restrict__ out)

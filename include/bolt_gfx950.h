@@ -68,11 +68,12 @@ EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes);
 /* Event pair on the library stream; stop returns the elapsed milliseconds after waiting. */
 EE bolt_gfx950_timer_start(void);
 EE bolt_gfx950_timer_stop(float *ms);
-/* Measurement aid with no counterpart in the reference: the rate (TOP/s) that the int8 matrix cores of
- * this device sustain on v_mfma_i32_16x16x64_i8 issued back to back from registers by 8 waves on every
- * CU, with random operand bits (zero_operands = 0: the device lowers its clock under that load) or with
- * all-zero operands (1). Takes a few milliseconds. The GEMM figures are read against these two. */
-EE bolt_gfx950_mfma_int8_rate(int zero_operands, float *tops);
+
+/* ---- blas_enhance: axpby -------------------------------------------------------------- */
+/* compute/blas_enhance/include/blas_enhance.h:25-26  vector_vector_axpby: y = a * x + b * y. DT_F32 only, as in the
+ * x86 build (compute/blas_enhance/src/cpu/x86/axpby.cpp); every element is fma(a, x, y * b) like the reference's
+ * 8-wide body (cpu/x86/fp32/axpby.cpp:23-29). */
+EE vector_vector_axpby_gfx950(F32 a, TensorDesc xDesc, const void *x, F32 b, TensorDesc yDesc, void *y, Arch arch);
 
 /* ---- blas_enhance: int8 GEMM --------------------------------------------------------- */
 /* compute/blas_enhance/include/blas_enhance.h:36-37  matrix_matrix_multiply_tmp_bytes */
@@ -167,6 +168,19 @@ EE matmul_gfx950(TensorDesc matrixADesc, bool transposeA, const void *matrixA, F
  * trailing block is 8 wide when oc % 16 == 8) or DF_NCHWC8; DT_F32 (optionally + eltwiseInput, laid
  * out like the output), DT_I32, or DT_U8_Q with the tensor-wide dynamic output scale.
  * scale[3] = {input scale, output scale (written), filter scale}, host memory. group must be 1. */
+/* convolution_infer_output_size_cpu (compute/tensor/src/convolution.cpp:28-109) as the AVX-512 build answers it:
+ * oh / ow from the padding, dilation, stride and round mode; DF_NCHWC16 for a DT_U8_Q target with fn != 8, else
+ * DF_NCHWC8; NOT_SUPPORTED when fn % 8 != 0. convolution_infer_forward_algorithm_x86 (cpu/x86/convolution.cpp:23-103)
+ * for a quantised target: POINTWISE for 1x1 filters, DIRECT otherwise; an algorithm already chosen is kept. */
+EE convolution_infer_output_size_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, ConvolutionParamSpec convParamSpec,
+    TensorDesc *outputDesc, DataType targetDataType, Arch arch);
+EE convolution_infer_forward_algorithm_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec convParamSpec, ConvolutionPolicy policy, ConvolutionForwardAlgorithm *algorithm,
+    DataType targetDataType, ActivationParamSpec activationDesc, Arch arch);
+/* Filter blob bytes: fn * 4 + ALIGN(fn, 16) * ALIGN(fh * fw * ALIGN(fc, 16), 64) + 32. That equals the reference's
+ * fn * ALIGN(fc, 16) * fh * fw + fn * 4 + 32 whenever fn % 16 == 0 and fh * fw * ALIGN(fc, 16) % 64 == 0 (every
+ * BASELINE shape) and is larger otherwise, so allocate from THIS query. ftmDesc = the filter's desc with
+ * df = DF_NCHWC2NxC4 and the channel dim rounded up to 16, as convolution_transform_filter_int8 returns it. */
 EE convolution_transform_filter_bytes_gfx950(TensorDesc filterDesc, ConvolutionParamSpec convParamSpec,
     ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch);
 EE convolution_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, ConvolutionParamSpec convParamSpec,

@@ -174,6 +174,14 @@ typedef struct ActivationParamSpec {
 #pragma pack()
 
 typedef enum {
+    CONVOLUTION_NO_TMP_MEM = 0,
+    CONVOLUTION_FASTEST = 1,
+    CONVOLUTION_TUNNING = 2,
+    CONVOLUTION_LIBRARY_SEARCH = 3,
+    CONVOLUTION_POLICY_FORCE_U32 = 0x7fffffff
+} ConvolutionPolicy; /* common/uni/include/parameter_spec.h:150-155 */
+
+typedef enum {
     CONVOLUTION_ALGORITHM_POINTWISE = 0,
     CONVOLUTION_ALGORITHM_DIRECT = 1,
     CONVOLUTION_ALGORITHM_IM2COL_GEMM = 2,

@@ -23,7 +23,8 @@ def quantize_weight_per_channel(W):
     """W: fp32 [N, K] -> (s8 [N, K], scale [N]) with scale[n] = 127 / max|W[n]| (quantised = real * scale)."""
     W = np.asarray(W, F)
     m = np.abs(W).max(axis=1)
-    s = np.where(m > 0, F(127.0) / m, F(1.0)).astype(F)
+    with np.errstate(divide="ignore"):
+        s = np.where(m > 0, F(127.0) / m, F(1.0)).astype(F)
     q = np.clip(np.rint(W * s[:, None]), -127, 127).astype(np.int8)
     return q, s
 

@@ -185,6 +185,62 @@ class Oracle:
                                           C.c_float(scaleW), _p(b), _p(out), odt, _p(s))
         return out, s[0]
 
+    def matmul(self, A, tA, B, tB, cdt, scaleA=-1.0, scaleB=-1.0):
+        """Batched int8 matmul as the reference's x86 branch composes it (compute/tensor/src/matmul.cpp:367-431,
+        495-554) for matrix results: fp32 A -> u8 and fp32 B -> s8 over the WHOLE tensor (scaleA / scaleB are the
+        operand tensors' scales, lower bounds of the dynamic ones), scaleO = sA * sB, then per 2-D slice one
+        u8 x s8 product starting from zero with cvt(acc) * (1 / scaleO) (cdt DT_F32) or the raw int32 (DT_I32).
+        A: [.., M, K] or [.., K, M] if tA; B: [.., K, N] or [.., N, K] if tB. A smaller batch is broadcast.
+        Returns (stacked slices, sA, sB)."""
+        qa, sa = self.quantize_f32(np.ascontiguousarray(A).reshape(-1), DT_U8_Q, scaleA)
+        qb, sb = self.quantize_f32(np.ascontiguousarray(B).reshape(-1), DT_I8, scaleB)
+        qa, qb = qa.reshape(A.shape), qb.reshape(B.shape)
+        A3 = qa.reshape((-1,) + A.shape[-2:])
+        B3 = qb.reshape((-1,) + B.shape[-2:])
+        batch = max(A3.shape[0], B3.shape[0])
+        outs = []
+        s = np.float32(sa) * np.float32(sb)
+        for i in range(batch):
+            a = A3[i % A3.shape[0]]
+            b = B3[i % B3.shape[0]]
+            W = b if tB else np.ascontiguousarray(b.T)          # [N, K]
+            M = a.shape[1] if tA else a.shape[0]
+            N = W.shape[0]
+            off = self.offsetC(W, True)
+            if cdt == DT_F32:
+                outs.append(self.mmm(a, W, off, np.zeros((M, N), np.float32), DT_F32, scale=[s], transA=tA))
+            else:
+                outs.append(self.mmm(a, W, off, np.zeros((M, N), np.int32), DT_I32, transA=tA))
+        return np.stack(outs), sa, sb
+
+
+    def matmul_vector(self, A, tA, B, tB, cdt):
+        """Vector result (one of M, N is 1): A -> I8, B -> U8_Q over the whole tensors, then one
+        matrix_vector_multiply per slice (compute/tensor/src/matmul.cpp:374-382, 531-548)."""
+        oracle = self
+        qa, sa = oracle.quantize_f32(np.ascontiguousarray(A).reshape(-1), DT_I8)
+        qb, sb = oracle.quantize_f32(np.ascontiguousarray(B).reshape(-1), DT_U8_Q)
+        A3 = qa.reshape((-1,) + A.shape[-2:])
+        B3 = qb.reshape((-1,) + B.shape[-2:])
+        batch = max(A3.shape[0], B3.shape[0])
+        s = np.float32(sa) * np.float32(sb)
+        M = A.shape[-1] if tA else A.shape[-2]
+        N = B.shape[-2] if tB else B.shape[-1]
+        ydt = np.float32 if cdt == DT_F32 else np.int32
+        sc = [s] if cdt == DT_F32 else None
+        outs = []
+        for i in range(batch):
+            a = A3[i % A3.shape[0]]
+            b = B3[i % B3.shape[0]]
+            if M == 1:
+                # u8 matrix b ([K, N], or [N, K] if tB) times the s8 vector a
+                outs.append(oracle.mvm_u8mat(b, a.reshape(-1), np.zeros(N, ydt), cdt, scale=sc, a_is_KM=not tB))
+            else:
+                # s8 matrix a ([M, K], or [K, M] if tA) times the u8 vector b
+                off = oracle.offsetC(a, not tA)
+                outs.append(oracle.mvm(a, b.reshape(-1), off, np.zeros(M, ydt), cdt, scale=sc, w_is_NK=not tA))
+        return np.stack(outs), sa, sb
+
 
 class Ref:
     """The reference's own compiled path. bfmt / wfmt: 0 = DF_NORMAL, 1 = DF_TRANSPOSE, 2 = packed."""

@@ -215,13 +215,66 @@ def gen_pool(ref):
     save("pool_concat", out)
 
 
+def gen_encoder_fp32():
+    """fp32 neighbours of the int8 GEMMs in an encoder layer as the reference's x86 kernels compute them:
+    layer_norm_fp32, softmax_fp32 and the GELU of activation_fp32."""
+    from checkers_tensor import RefTensor
+    from test_oracle_encoder import gelu_inputs, ln_inputs, softmax_inputs
+    r = RefTensor()
+    x, g, b = ln_inputs()
+    gx = gelu_inputs()
+    s = softmax_inputs()
+    small = s[:32, :64] / np.float32(4.0)
+    save("encoder_fp32", {"ln_x": x, "ln_g": g, "ln_b": b, "ln_y": r.layer_norm(x, g, b), "gelu_x": gx,
+                          "gelu_y": r.gelu(gx), "softmax_x": s, "softmax_y": r.softmax(s),
+                          "softmax_small_y": r.softmax(small)})
+
+
+def gen_orchestration(orc):
+    """The reference's Tensor-level callers: fully_connected(), matmul() and the convolution's query functions."""
+    from checkers_tensor import RefTensor
+    from test_oracle_orchestration import CONV_QUERY_CASES, FC_CASES, MATMUL_CASES, fc_inputs, matmul_inputs
+    r = RefTensor()
+    out = {}
+    for i, case in enumerate(FC_CASES):
+        M, K, N, odt, scaleO, mvm, with_bias = case
+        x, sI, W, sW, bias = fc_inputs(case, SEED + 100 + i)
+        y, so, tb = r.fully_connected(x, sI, W, sW, bias if with_bias else None, odt, scaleO, mvm=bool(mvm))
+        out[f"fc_y{i}"], out[f"fc_scale{i}"], out[f"fc_tmp{i}"] = y, np.float32(so), np.int64(tb)
+    for i, case in enumerate(MATMUL_CASES):
+        a_shape, tA, b_shape, tB = case
+        A, B, c_shape = matmul_inputs(case, SEED + 200 + i)
+        y, tb = r.matmul(A, DT_F32, tA, -1.0, B, DT_F32, tB, -1.0, c_shape)
+        out[f"mm_y{i}"], out[f"mm_tmp{i}"] = y, np.int64(tb)
+    rows = []
+    for case in CONV_QUERY_CASES:
+        q = r.conv_queries(*case)
+        rows.append(list(q["out"]) + [q["alg"], q["filter_bytes"]] + list(q["ftm"]) + [q["tmp_bytes"]])
+    out["conv_queries"] = np.array(rows, np.int64)
+    save("orchestration", out)
+
+
 if __name__ == "__main__":
     if not Ref.available():
         sys.exit("oracle/_ref/libboltref.so is missing or this host has no avx512_vnni")
     ref, orc = Ref(threads=1), Oracle()
-    gen_sizes(ref)
-    gen_mmm(ref, orc)
-    gen_mvm(ref, orc)
-    gen_quantize(ref, orc)
-    gen_conv(ref, orc)
-    gen_pool(ref)
+    only = set(sys.argv[1:])   # e.g. `make_golden.py encoder_fp32 orchestration` rewrites just those files
+
+    def want(name):
+        return not only or name in only
+    if want("sizes"):
+        gen_sizes(ref)
+    if want("mmm"):
+        gen_mmm(ref, orc)
+    if want("mvm"):
+        gen_mvm(ref, orc)
+    if want("quantize"):
+        gen_quantize(ref, orc)
+    if want("conv_int8"):
+        gen_conv(ref, orc)
+    if want("pool_concat"):
+        gen_pool(ref)
+    if want("encoder_fp32"):
+        gen_encoder_fp32()
+    if want("orchestration"):
+        gen_orchestration(orc)

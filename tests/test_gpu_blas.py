@@ -358,3 +358,68 @@ def test_per_channel_epilogue(torch_mod, oracle):
                        "mvm_perchannel")
             capi.check(L.bolt_gfx950_synchronize(), "sync")
             assert np.array_equal(y.cpu().numpy().view(np.int32), want[0].view(np.int32))
+
+
+def _strided_batch_case(torch, oracle, N, K, batch, copies, with_bias, seed, pad=0):
+    """One call of bolt_gfx950_mvm_int8_strided_batch checked row by row: slice b multiplies weight copy
+    b % copies (every copy holds DIFFERENT weights, so a wrong copy index shows), has its own activation scale,
+    shares the per-channel weight scales and the optional fp32 bias. Integer part: the reference's GEMV
+    (mvm_avx512_vnni.cpp:703-759) on that copy; fp32 part: the per-channel closed form."""
+    L = capi.lib()
+    rng = np.random.default_rng(seed)
+    Ws = rng.integers(-127, 128, size=(copies, N, K), dtype=np.int8)
+    X = rng.integers(0, 256, size=(batch, K), dtype=np.uint8)
+    sI = rng.uniform(5.0, 60.0, size=batch).astype(np.float32)
+    sW = (1.0 / rng.uniform(0.005, 0.02, size=N)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32) if with_bias else None
+    blobs = [host.mvm_transform_weight(dev(torch, Ws[c]), DF_NORMAL, N, K)[0] for c in range(copies)]
+    blob_bytes = (N + 15) // 16 * 16 * ((K + 7) // 8 * 8) + 4 * N
+    stride = (blob_bytes + 255) // 256 * 256 + pad
+    wbuf = torch.zeros(copies * stride, dtype=torch.uint8, device="cuda")
+    for c in range(copies):
+        wbuf[c * stride:c * stride + blob_bytes] = blobs[c][:blob_bytes]
+    dX, dsI, dsW = dev(torch, X), dev(torch, sI), dev(torch, sW)
+    dbias = dev(torch, bias) if with_bias else None
+    y = torch.full((batch, N), float("nan"), dtype=torch.float32, device="cuda")
+    capi.check(L.bolt_gfx950_mvm_int8_strided_batch(batch, N, K, wbuf.data_ptr(), stride, copies, dX.data_ptr(),
+                                                    y.data_ptr(), dsI.data_ptr(), dsW.data_ptr(),
+                                                    dbias.data_ptr() if with_bias else None), "mvm_strided_batch")
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    got = y.cpu().numpy()
+    offs = [oracle.offsetC(Ws[c], True) for c in range(copies)]
+    zero = np.zeros(N, np.int32)
+    for b in range(batch):
+        c = b % copies
+        acc = oracle.mvm(Ws[c], X[b], offs[c], zero, DT_I32)
+        want = oracle.dequant_per_channel(acc.reshape(1, N), sI[b], sW, bias).reshape(-1)
+        assert np.array_equal(got[b].view(np.int32), want.view(np.int32)), (N, K, batch, copies, with_bias, b)
+
+
+@pytest.mark.parametrize("copies", [1, 3, 64])
+@pytest.mark.parametrize("with_bias", [False, True], ids=["nobias", "bias"])
+def test_mvm_strided_batch_decode_shape(torch_mod, oracle, copies, with_bias):
+    """The benchmark's launch at its full shape: N = K = 4096, 256 vectors, rotating over `copies` weight blobs."""
+    say("mvm_strided_batch", 4096, 4096, 256, copies, with_bias)
+    _strided_batch_case(torch_mod, oracle, 4096, 4096, 256, copies, with_bias, seed=100 + copies)
+
+
+@pytest.mark.parametrize("N,K,batch,copies", [(100, 77, 5, 2), (100, 77, 5, 1), (9, 1, 3, 3), (33, 4100, 7, 4),
+                                               (16, 16, 1, 1), (257, 520, 300, 5)])
+def test_mvm_strided_batch_ragged(torch_mod, oracle, N, K, batch, copies):
+    """N % 16, K % 8 and K % 16 tails, fewer vectors than copies, more than 256 vectors, a stride with slack."""
+    say("mvm_strided_batch ragged", N, K, batch, copies)
+    _strided_batch_case(torch_mod, oracle, N, K, batch, copies, True, seed=N * 7 + K, pad=256)
+    _strided_batch_case(torch_mod, oracle, N, K, batch, copies, False, seed=N * 7 + K + 1)
+
+
+def test_mvm_strided_batch_arguments(torch_mod):
+    L = capi.lib()
+    torch = torch_mod
+    t = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    f = torch.zeros(64, dtype=torch.float32, device="cuda")
+    p, q = t.data_ptr(), f.data_ptr()
+    assert L.bolt_gfx950_mvm_int8_strided_batch(1, 16, 16, None, 0, 1, p, q, q, q, None) == capi.NULL_POINTER
+    assert L.bolt_gfx950_mvm_int8_strided_batch(1, 16, 16, p, 0, 0, p, q, q, q, None) == capi.NOT_MATCH
+    assert L.bolt_gfx950_mvm_int8_strided_batch(2, 16, 16, p, 16, 2, p, q, q, q, None) == capi.NOT_MATCH   # stride < blob
+    assert L.bolt_gfx950_mvm_int8_strided_batch(2, 16, 16, p, 322, 2, p, q, q, q, None) == capi.NOT_MATCH  # stride % 4
+    assert L.bolt_gfx950_mvm_int8_strided_batch(0, 16, 16, p, 0, 1, p, q, q, q, None) == capi.SUCCESS

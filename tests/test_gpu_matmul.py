@@ -19,27 +19,9 @@ def torch_mod():
 
 
 def oracle_matmul(oracle, A, tA, B, tB, cdt):
-    """A: [batch.., M, K] or [.., K, M] if tA; B: [batch.., K, N] or [.., N, K] if tB (fp32)."""
-    qa, sa = oracle.quantize_f32(A.reshape(-1), DT_U8_Q)
-    qb, sb = oracle.quantize_f32(B.reshape(-1), DT_I8)
-    qa, qb = qa.reshape(A.shape), qb.reshape(B.shape)
-    A3 = qa.reshape((-1,) + A.shape[-2:])
-    B3 = qb.reshape((-1,) + B.shape[-2:])
-    batch = max(A3.shape[0], B3.shape[0])
-    outs = []
-    s = np.float32(sa) * np.float32(sb)
-    for i in range(batch):
-        a = A3[i % A3.shape[0]]
-        b = B3[i % B3.shape[0]]
-        W = b if tB else np.ascontiguousarray(b.T)          # [N, K]
-        M = a.shape[1] if tA else a.shape[0]
-        N = W.shape[0]
-        off = oracle.offsetC(W, True)
-        if cdt == DT_F32:
-            outs.append(oracle.mmm(a, W, off, np.zeros((M, N), np.float32), DT_F32, scale=[s], transA=tA))
-        else:
-            outs.append(oracle.mmm(a, W, off, np.zeros((M, N), np.int32), DT_I32, transA=tA))
-    return np.stack(outs), sa, sb
+    """The oracle's composition (checkers.Oracle.matmul), itself pinned against the reference's matmul() in
+    tests/test_oracle_orchestration.py and tests/golden/orchestration.npz."""
+    return oracle.matmul(A, tA, B, tB, cdt)
 
 
 CASES = [  # (A shape, transposeA, B shape, transposeB)
@@ -105,29 +87,7 @@ def test_matmul_errors(torch_mod):
 
 
 def oracle_matmul_vector(oracle, A, tA, B, tB, cdt):
-    """Vector result: A -> I8, B -> U8_Q, then matrix_vector_multiply per slice (matmul.cpp:374-382, :531-548)."""
-    qa, sa = oracle.quantize_f32(A.reshape(-1), DT_I8)
-    qb, sb = oracle.quantize_f32(B.reshape(-1), DT_U8_Q)
-    A3 = qa.reshape((-1,) + A.shape[-2:])
-    B3 = qb.reshape((-1,) + B.shape[-2:])
-    batch = max(A3.shape[0], B3.shape[0])
-    s = np.float32(sa) * np.float32(sb)
-    M = A.shape[-1] if tA else A.shape[-2]
-    N = B.shape[-2] if tB else B.shape[-1]
-    ydt = np.float32 if cdt == DT_F32 else np.int32
-    sc = [s] if cdt == DT_F32 else None
-    outs = []
-    for i in range(batch):
-        a = A3[i % A3.shape[0]]
-        b = B3[i % B3.shape[0]]
-        if M == 1:
-            # u8 matrix b ([K, N], or [N, K] if tB) times the s8 vector a
-            outs.append(oracle.mvm_u8mat(b, a.reshape(-1), np.zeros(N, ydt), cdt, scale=sc, a_is_KM=not tB))
-        else:
-            # s8 matrix a ([M, K], or [K, M] if tA) times the u8 vector b
-            off = oracle.offsetC(a, not tA)
-            outs.append(oracle.mvm(a, b.reshape(-1), off, np.zeros(M, ydt), cdt, scale=sc, w_is_NK=not tA))
-    return np.stack(outs), sa, sb
+    return oracle.matmul_vector(A, tA, B, tB, cdt)
 
 
 VECTOR_CASES = [  # (A shape, transposeA, B shape, transposeB): one of M, N is 1

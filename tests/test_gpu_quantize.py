@@ -213,3 +213,48 @@ def test_roundtrip_properties_at_full_size(torch_mod):
     back = host.dequantize(q, DT_U8_Q, s[0])
     capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
     assert float((back - x).abs().max().item()) <= 0.5 / float(s[0]) * 1.0001
+
+
+def test_static_then_dynamic_without_sync(torch_mod, oracle):
+    """Device-pointer mode: calls with a caller-given (static) scale return without waiting for their kernels. A
+    dynamic call issued right behind them must return ITS scale, not a value that one of the earlier kernels
+    left in the word the host reads the scale from. Large static tensors first, so that their kernels are still
+    running when the dynamic calls are issued; no synchronisation anywhere in between."""
+    torch = torch_mod
+    L = capi.lib()
+    rng = np.random.default_rng(77)
+    big_f = torch.from_numpy(rng.standard_normal(4096 * 3072).astype(np.float32)).cuda()
+    big_i = torch.from_numpy(rng.integers(-300000, 300000, size=4096 * 3072, dtype=np.int32)).cuda()
+    small = rng.standard_normal(3000).astype(np.float32) * 5.0
+    dsmall = torch.from_numpy(small).cuda()
+    M, K, N = 8, 256, 64
+    xq = rng.integers(1, 256, size=(M, K), dtype=np.uint8)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    blob, bdesc, rhs = host.mmm_transform_rhs(torch.from_numpy(W).cuda(), capi.DF_TRANSPOSE, K, N)
+    dxq, dbias = torch.from_numpy(xq).cuda(), torch.from_numpy(bias).cuda()
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    want_q, want_s = oracle.quantize_f32(small, DT_U8_Q, -1.0, 0)
+    want_fc, want_fs = oracle.fully_connected(xq, np.float32(21.0), W, np.float32(33.0), bias, DT_U8_Q)
+    for fused in (1, 0):
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused", fused), "set_option")
+        try:
+            for rep in range(4):
+                print("static_then_dynamic", fused, rep, flush=True)
+                s_static = [np.float32(17.5)]
+                host.quantize(big_f, DT_F32, DT_U8_Q, s_static, 1)        # static fp32 -> u8
+                s_req = [np.float32(0.011), np.float32(0.37)]
+                host.quantize(big_i, DT_I32, DT_U8_Q, s_req)               # static int32 -> u8
+                s = [-1.0]
+                q = host.quantize(dsmall, DT_F32, DT_U8_Q, s)              # dynamic, straight behind them
+                assert s[0] == want_s, (fused, rep, s[0], want_s)
+                host.quantize(big_f, DT_F32, DT_I8, [np.float32(3.25)], 1)
+                host.quantize(big_i, DT_I32, DT_I8, [np.float32(0.02), np.float32(0.37)])
+                out, so = host.fully_connected(dxq, 21.0, blob, capi.DF_NKNxKx, 33.0, dbias, M, K, N, DT_U8_Q, -1.0)
+                assert so == want_fs, (fused, rep, so, want_fs)
+                capi.check(L.bolt_gfx950_synchronize(), "sync")
+                assert np.array_equal(q.cpu().numpy(), want_q)
+                assert np.array_equal(out.cpu().numpy(), want_fc)
+                assert s_static[0] == np.float32(17.5) and s_req[0] == np.float32(0.011)
+        finally:
+            capi.check(L.bolt_gfx950_set_option(b"quantize_fused", 1), "set_option")
