@@ -408,6 +408,17 @@ void orc_requantize_i8(const int8_t *in, uint32_t n, float inScale, int8_t *out,
     }
 }
 
+/* vector_vector_axpby, fp32 (compute/blas_enhance/src/cpu/x86/fp32/axpby.cpp:16-34): y = fmadd(a, x, y * b) --
+ * the product y * b rounded to fp32, then one fused multiply-add. The scalar tail `a * x[i] + b * y[i]` compiles to
+ * the same contraction under the reference's -O3 -mfma (checked against the compiled reference for every length). */
+void orc_axpby_f32(uint32_t n, float a, const float *x, float b, float *y)
+{
+    for (uint32_t i = 0; i < n; ++i) {
+        volatile float t = y[i] * b;
+        y[i] = fmaf(a, x[i], t);
+    }
+}
+
 /* Per-output-channel dequantisation with fp32 bias: not in the reference (Tensor carries one
  * scale, common/memory/include/tensor.hpp:83-96). Closed form that reduces to the reference's
  * per-tensor epilogue when every scaleW[n] is equal and bias is NULL:

@@ -51,6 +51,7 @@ void orc_dequantize_u8_f32(const uint8_t *q, uint32_t n, const float *scale, flo
 void orc_requantize_i8(const int8_t *in, uint32_t n, float inScale, int8_t *out, float outScale);
 
 /* ---- per-output-channel epilogue (superset of the reference, closed form) --------- */
+void orc_axpby_f32(uint32_t n, float a, const float *x, float b, float *y);
 void orc_dequant_per_channel(const int32_t *acc, uint32_t M, uint32_t N, const float *scaleI,
     const float *scaleW, const float *bias, float *out);
 

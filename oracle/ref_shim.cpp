@@ -59,6 +59,12 @@ void ref_set_threads(int n)
     OMP_NUM_THREADS = n;
 }
 
+// y = a * x + b * y, fp32 (compute/blas_enhance/src/axpby.cpp:24-60)
+int ref_axpby_f32(U32 n, float a, const float *x, float b, float *y)
+{
+    return vector_vector_axpby(a, tensor1d(DT_F32, n), x, b, tensor1d(DT_F32, n), y, X86_AVX512);
+}
+
 int ref_mmm_transform_rhs_bytes(int bfmt, U32 K, U32 N, U32 *bytes, U32 *rhsBytes)
 {
     return matrix_matrix_multiply_transform_rhs_bytes(rhs_desc(bfmt, K, N), bytes, rhsBytes, X86_AVX512);

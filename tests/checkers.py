@@ -163,6 +163,13 @@ class Oracle:
         self.lib.orc_requantize_i8(_p(x), u32(x.size), C.c_float(inScale), _p(out), C.c_float(outScale))
         return out
 
+    def axpby(self, a, x, b, y):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.array(y, dtype=np.float32).copy()
+        self.lib.orc_axpby_f32.argtypes = [u32, C.c_float, vp, C.c_float, vp]
+        self.lib.orc_axpby_f32(u32(x.size), C.c_float(a), _p(x), C.c_float(b), _p(out))
+        return out
+
     def dequant_per_channel(self, acc, scaleI, scaleW, bias=None):
         acc = np.ascontiguousarray(acc, dtype=np.int32)
         M, N = acc.shape
@@ -253,6 +260,13 @@ class Ref:
         self.lib = C.CDLL(REF_SO)
         self.lib.ref_requantize.argtypes = [vp, u32, C.c_float, vp, C.c_float]
         self.lib.ref_set_threads(int(threads))
+
+    def axpby(self, a, x, b, y):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.array(y, dtype=np.float32).copy()
+        self.lib.ref_axpby_f32.argtypes = [u32, C.c_float, vp, C.c_float, vp]
+        assert self.lib.ref_axpby_f32(u32(x.size), C.c_float(a), _p(x), C.c_float(b), _p(out)) == 0
+        return out
 
     def mmm_transform_rhs_bytes(self, bfmt, K, N):
         b, r = u32(0), u32(0)

@@ -251,6 +251,11 @@ def gen_orchestration(orc):
         q = r.conv_queries(*case)
         rows.append(list(q["out"]) + [q["alg"], q["filter_bytes"]] + list(q["ftm"]) + [q["tmp_bytes"]])
     out["conv_queries"] = np.array(rows, np.int64)
+    from test_oracle_vs_ref import AXPBY_NS, axpby_inputs
+    ref = Ref(threads=1)
+    for n in AXPBY_NS:
+        a, x, b, y = axpby_inputs(n)
+        out[f"axpby_{n}"] = ref.axpby(a, x, b, y)
     save("orchestration", out)
 
 

@@ -111,3 +111,11 @@ def test_pool_and_concat(oracle):
         loops = int(np.prod(dims[0][:axis]))
         y, s = orc_concat(oracle, parts, lens, loops, g[f"cat_scales{i}"])
         assert same(y, g[f"cat_y{i}"]) and same(np.float32(s), g[f"cat_s{i}"])
+
+
+def test_axpby(oracle):
+    from test_oracle_vs_ref import AXPBY_NS, axpby_inputs
+    g = load("orchestration")
+    for n in AXPBY_NS:
+        a, x, b, y = axpby_inputs(n)
+        assert same(oracle.axpby(a, x, b, y), g[f"axpby_{n}"])

@@ -297,3 +297,25 @@ def test_requantize(oracle, ref):
     x = np.arange(-128, 128, dtype=np.int8)
     for si, so in [(1.0, 1.0), (2.0, 1.0), (1.0, 0.9), (3.0, 2.0), (7.0, 6.99)]:
         assert np.array_equal(ref.requantize(x, si, so), oracle.requantize(x, si, so)), (si, so)
+
+
+AXPBY_NS = [1, 7, 8, 9, 15, 16, 17, 1000, 1003]
+
+
+def axpby_inputs(n):
+    rng = np.random.default_rng(9000 + n)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    y = (rng.standard_normal(n) * 3).astype(np.float32)
+    return np.float32(0.37), x, np.float32(-1.7), y
+
+
+def test_axpby(oracle, ref):
+    """y = a * x + b * y in fp32: the 8-wide body and the scalar tail (cpu/x86/fp32/axpby.cpp:23-32), plus the
+    closed form fma(a, x, fl(y * b)) in float64 (exact product of two fp32 values)."""
+    for n in AXPBY_NS:
+        a, x, b, y = axpby_inputs(n)
+        want = ref.axpby(a, x, b, y)
+        assert np.array_equal(oracle.axpby(a, x, b, y).view(np.int32), want.view(np.int32)), n
+        yb = (y * b).astype(np.float32)
+        closed = (np.float64(a) * x.astype(np.float64) + yb.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(want.view(np.int32), closed.view(np.int32)), n
