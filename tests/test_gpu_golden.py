@@ -205,7 +205,8 @@ def test_encoder_fp32_neighbours_golden(torch_mod):
         return float(np.abs(a.astype(np.float64) - b.astype(np.float64)).max()) <= tol * max(1.0, float(np.abs(b).max()))
     x, ga, be, want = g["ln_x"], g["ln_g"], g["ln_b"], g["ln_y"]
     dx, out = dev(torch, x), torch.zeros(x.shape, dtype=torch.float32, device="cuda")
-    capi.check(L.bolt_gfx950_add_layernorm_f32(dx.data_ptr(), None, dev(torch, ga).data_ptr(), dev(torch, be).data_ptr(),
+    dga, dbe = dev(torch, ga), dev(torch, be)
+    capi.check(L.bolt_gfx950_add_layernorm_f32(dx.data_ptr(), None, dga.data_ptr(), dbe.data_ptr(),
                                                x.shape[0], x.shape[1], out.data_ptr()), "layernorm")
     capi.check(L.bolt_gfx950_synchronize(), "sync")
     got = out.cpu().numpy()
@@ -226,6 +227,7 @@ def test_encoder_fp32_neighbours_golden(torch_mod):
     eye = np.eye(keys, dtype=np.float32)
     qkv = np.concatenate([q, eye, eye], axis=1)
     ctx = torch.zeros((keys, 64), dtype=torch.float32, device="cuda")
-    capi.check(L.bolt_gfx950_attention_f32(dev(torch, qkv).data_ptr(), 1, keys, 64, 1, ctx.data_ptr()), "attention")
+    dqkv = dev(torch, qkv)
+    capi.check(L.bolt_gfx950_attention_f32(dqkv.data_ptr(), 1, keys, 64, 1, ctx.data_ptr()), "attention")
     capi.check(L.bolt_gfx950_synchronize(), "sync")
     assert float(np.abs(ctx.cpu().numpy()[:32] - g["softmax_small_y"]).max()) <= 2e-6
