@@ -214,6 +214,7 @@ SIGNATURES = {
     "bolt_gfx950_add_layernorm_f32": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "bolt_gfx950_gelu_f32": (C.c_int, [_vp, C.c_size_t]),
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
+    "bolt_gfx950_quantize_f32_noalloc": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_strided_batch": (C.c_int, [_u32, _u32, _u32, _vp, C.c_size_t, _u32, _vp, _vp, _vp, _vp,

@@ -17,6 +17,11 @@
 using namespace bg;
 
 namespace {
+struct Ctx;
+Ctx &ctx();
+}  // namespace
+
+namespace {
 
 struct Ctx {
     std::mutex mu;
@@ -46,7 +51,16 @@ Ctx &ctx()
     return c;
 }
 
-EE fail(EE code, const char *what, hipError_t he = hipSuccess)
+}  // namespace
+
+namespace bg {
+
+hipStream_t api_stream()
+{
+    return ctx().stream;
+}
+
+void api_set_error(const char *what, hipError_t he)
 {
     Ctx &c = ctx();
     c.err = what;
@@ -54,6 +68,15 @@ EE fail(EE code, const char *what, hipError_t he = hipSuccess)
         c.err += ": ";
         c.err += hipGetErrorString(he);
     }
+}
+
+}  // namespace bg
+
+namespace {
+
+EE fail(EE code, const char *what, hipError_t he = hipSuccess)
+{
+    bg::api_set_error(what, he);
     return code;
 }
 
@@ -113,6 +136,9 @@ EE ensure_init()
     }
     if (e != hipSuccess) {
         return fail(ALLOC_FAILED, "hipHostMalloc(scale word)", e);
+    }
+    if (noalloc_init_current_device() != SUCCESS) {
+        return UNKNOWN;  // the text is already set
     }
     c.ready = true;
     return SUCCESS;

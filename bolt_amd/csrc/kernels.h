@@ -10,6 +10,11 @@ namespace bg {
 // Every field of the argument structs below has a default (null / 0): a caller that leaves one out hands the
 // kernel a harmless value, never an indeterminate pointer.
 
+// ---- shared with the C-ABI layer (api.hip) ---------------------------------------------------------
+hipStream_t api_stream();                              // the stream every call is enqueued on (null until set)
+void api_set_error(const char *what, hipError_t he);   // text behind bolt_gfx950_last_error()
+int noalloc_init_current_device();                     // noalloc.hip: looks up the static scratch array's device address
+
 // ---- GEMV ---------------------------------------------------------------------------------------
 struct GemvBatch {
     uint32_t count = 0;      // number of independent products in the launch (0 / 1: a single one)

@@ -339,6 +339,17 @@ EE bolt_gfx950_gelu_f32(float *x, size_t n);
  *   per-output-channel weight scales scaleW[N] and optional fp32 bias[N] (both device);
  *   reduces to the per-tensor reference epilogue when every scaleW[n] is equal and bias is NULL. */
 EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode);
+
+/* No counterpart in the reference. bolt_gfx950_quantize_f32_async for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, same bytes
+ * and same scale, but the partial-maximum slots its kernels need live in a static device array of 4 KiB that each
+ * GPU holds until the process ends, and the call runs no hipMalloc / hipFree or any allocating routine (nor does
+ * it initialise the rest of the library). At most BOLT_GFX950_NOALLOC_MAX_ELEMENTS elements (NOT_SUPPORTED beyond,
+ * with the reason in bolt_gfx950_last_error()). Enqueued on the library's stream (bolt_gfx950_set_stream; the
+ * default stream if none was set). All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race. */
+#define BOLT_GFX950_NOALLOC_MAX_ELEMENTS (1u << 30)
+EE bolt_gfx950_quantize_f32_noalloc(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode);
 EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
     float *C, const float *dscaleI, const float *scaleW, const float *bias);
 EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void *x, const I32 *offsetC, float *y,
