@@ -145,6 +145,7 @@ class BoltEncoderLayerInt8(C.Structure):
 
 SIGNATURES = {
     "bolt_gfx950_init": (C.c_int, []),
+    "bolt_gfx950_get_counter": (C.c_int, [C.c_char_p, C.POINTER(C.c_ulonglong)]),
     "vector_vector_axpby_gfx950": (C.c_int, [C.c_float, TensorDesc, _vp, C.c_float, TensorDesc, _vp, C.c_int]),
     "convolution_infer_output_size_gfx950": (C.c_int, [TensorDesc, TensorDesc, ConvolutionParamSpec, _TDp, C.c_int,
                                                        C.c_int]),

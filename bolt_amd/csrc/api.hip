@@ -3,6 +3,7 @@
 // happens on the CPU here except the load-time weight pack in host-pointer mode.
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <chrono>
@@ -23,8 +24,12 @@ Ctx &ctx();
 
 namespace {
 
+// Everything a call needs besides its arguments. One context per calling thread: its stream, its scratch words, its
+// pinned scale word, its quantiser sync area and its staging pool, so that threads calling at the same time (each
+// with its own tensors, as CNN::clone() gives them) never share mutable state. Contexts come from a process-wide
+// pool: a thread takes one on its first call and returns it when it ends; device memory is never freed, so a
+// process that creates and ends threads does not leak one context per thread.
 struct Ctx {
-    std::mutex mu;
     bool ready = false;
     hipStream_t stream = nullptr;
     uint32_t *ws = nullptr;  // device scratch words for the two-pass reductions
@@ -37,6 +42,7 @@ struct Ctx {
     bool enc_ws_dirty = true;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
+    bool reused = false;  // taken over from a thread that has ended: its last work may still be running
     struct Buf {
         void *p;
         size_t bytes;
@@ -45,11 +51,49 @@ struct Ctx {
     std::vector<Buf> pool;
 };
 
+struct CtxPool {
+    std::mutex mu;
+    std::vector<Ctx *> idle;
+};
+
+CtxPool &ctx_pool()
+{
+    static CtxPool *p = new CtxPool;  // never destroyed: threads may end after static destructors have run
+    return *p;
+}
+
+struct CtxLease {
+    Ctx *c = nullptr;
+    ~CtxLease()
+    {
+        if (c) {
+            CtxPool &p = ctx_pool();
+            std::lock_guard<std::mutex> lk(p.mu);
+            c->stream = nullptr;
+            c->reused = true;
+            p.idle.push_back(c);
+        }
+    }
+};
+
 Ctx &ctx()
 {
-    static Ctx c;
-    return c;
+    thread_local CtxLease lease;
+    if (!lease.c) {
+        CtxPool &p = ctx_pool();
+        std::lock_guard<std::mutex> lk(p.mu);
+        if (!p.idle.empty()) {
+            lease.c = p.idle.back();
+            p.idle.pop_back();
+        } else {
+            lease.c = new Ctx;
+        }
+    }
+    return *lease.c;
 }
+
+// counters behind bolt_gfx950_get_counter
+std::atomic<unsigned long long> g_fused_fallbacks{0};
 
 }  // namespace
 
@@ -103,8 +147,16 @@ int g_quantize_fused = 1;
 EE ensure_init()
 {
     Ctx &c = ctx();
-    std::lock_guard<std::mutex> lk(c.mu);
     if (c.ready) {
+        if (c.reused) {
+            // this context served a thread that has ended; whatever that thread enqueued last must not overlap with
+            // this thread's use of the same scratch words (its stream may be gone: wait for the device)
+            c.reused = false;
+            hipError_t e = hipDeviceSynchronize();
+            if (e != hipSuccess) {
+                return fail(UNKNOWN, "hipDeviceSynchronize", e);
+            }
+        }
         return SUCCESS;
     }
     int n = 0;
@@ -112,12 +164,15 @@ EE ensure_init()
     if (e != hipSuccess || n == 0) {
         return fail(NOT_SUPPORTED, "no HIP device available", e);
     }
-    e = hipMalloc((void **)&c.ws, (kWsWords + 64 + 4 * kWsWords) * sizeof(uint32_t));
-    if (e != hipSuccess) {
-        return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
+    if (!c.ws) {
+        e = hipMalloc((void **)&c.ws, (kWsWords + 64 + 4 * kWsWords) * sizeof(uint32_t));
+        if (e != hipSuccess) {
+            c.ws = nullptr;
+            return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
+        }
     }
     c.enc_ws = c.ws + kWsWords + 64;
-    {
+    if (!c.fsync.slots) {
         void *p = nullptr;
         e = hipMalloc(&p, kFusedSyncBytes);
         if (e == hipSuccess) {
@@ -130,12 +185,15 @@ EE ensure_init()
         c.fsync.counter = (uint32_t *)((uint8_t *)p + 64 * 64);
         c.fsync.release = (unsigned long long *)((uint8_t *)p + 64 * 64 + 64);
     }
-    e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
-    if (e == hipSuccess) {
-        e = hipHostGetDevicePointer((void **)&c.hscale_dev, c.hscale, 0);
-    }
-    if (e != hipSuccess) {
-        return fail(ALLOC_FAILED, "hipHostMalloc(scale word)", e);
+    if (!c.hscale) {
+        e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
+        if (e == hipSuccess) {
+            e = hipHostGetDevicePointer((void **)&c.hscale_dev, c.hscale, 0);
+        }
+        if (e != hipSuccess) {
+            c.hscale = nullptr;
+            return fail(ALLOC_FAILED, "hipHostMalloc(scale word)", e);
+        }
     }
     if (noalloc_init_current_device() != SUCCESS) {
         return UNKNOWN;  // the text is already set
@@ -156,7 +214,7 @@ void arm_scale(Ctx &c)
     *(volatile uint32_t *)c.hscale = kScaleUnset;
 }
 
-EE take_scale(Ctx &c, float *dst)
+EE take_scale(Ctx &c, float *dst, bool *gave_up = nullptr)
 {
     volatile uint32_t *w = (volatile uint32_t *)c.hscale;
     const auto t0 = std::chrono::steady_clock::now();
@@ -171,20 +229,25 @@ EE take_scale(Ctx &c, float *dst)
     if (bits == kScaleUnset) {
         return fail(UNKNOWN, "the kernel did not produce a scale");
     }
-    if ((bits & 0x7fffffffu) > 0x7f800000u) {  // NaN: the one-launch quantiser gave up waiting for its grid
+    if ((bits & 0x7fffffffu) > 0x7f800000u) {
+        // NaN: the one-launch quantiser's bounded wait for its grid expired. Every workgroup of that launch then
+        // skipped its stores; the caller runs the two-pass form instead (gave_up), or reports it.
+        if (gave_up) {
+            *gave_up = true;
+            return SUCCESS;
+        }
         return fail(UNKNOWN, "the quantiser's grid barrier timed out");
     }
     memcpy(dst, &bits, 4);
     return SUCCESS;
 }
 
-// Grow-only device staging pool for the host-pointer mode.
+// Grow-only device staging pool for the host-pointer mode (per context, so per calling thread).
 struct Stage {
+    Ctx &c = ctx();
     std::vector<size_t> taken;
     ~Stage()
     {
-        Ctx &c = ctx();
-        std::lock_guard<std::mutex> lk(c.mu);
         for (size_t i : taken) {
             c.pool[i].busy = false;
         }
@@ -192,8 +255,6 @@ struct Stage {
     void *get(size_t bytes)
     {
         bytes = std::max<size_t>(bytes, 256);
-        Ctx &c = ctx();
-        std::lock_guard<std::mutex> lk(c.mu);
         for (size_t i = 0; i < c.pool.size(); ++i) {
             if (!c.pool[i].busy && c.pool[i].bytes >= bytes) {
                 c.pool[i].busy = true;
@@ -429,6 +490,15 @@ EE bolt_gfx950_set_option(const char *name, int value)
         g_lstm_gemm_rows = value;
         return SUCCESS;
     }
+    if (strcmp(name, "quantize_fused_spin") == 0) {
+        // polls of the one-launch quantiser's bounded wait before a workgroup gives up; tests set it to 1 so that the
+        // launch gives up and the two-pass form takes over. 0 restores the default (about a second). Per thread.
+        if (value < 0) {
+            return NOT_MATCH;
+        }
+        ctx().fsync.spin_limit = value ? (uint32_t)value : kFusedSpinDefault;
+        return SUCCESS;
+    }
     if (strcmp(name, "quantize_fused") == 0) {
         if (value != 0 && value != 1) {
             return NOT_MATCH;
@@ -448,6 +518,18 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         conv_force_panel(value);
+        return SUCCESS;
+    }
+    return NOT_FOUND;
+}
+
+EE bolt_gfx950_get_counter(const char *name, unsigned long long *value)
+{
+    if (!name || !value) {
+        return NULL_POINTER;
+    }
+    if (strcmp(name, "quantize_fused_fallbacks") == 0) {
+        *value = g_fused_fallbacks.load();
         return SUCCESS;
     }
     return NOT_FOUND;
@@ -1021,61 +1103,62 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     // Only a call that returns a freshly computed scale lets its kernel write the pinned word (and waits for it
     // below). A static-scale kernel that wrote it too would do so at some later time, without the host waiting,
     // and could land its value after the NEXT call has armed the word.
-    float *dscale = nullptr;
-    bool read_back = false;
-    if (f32in) {
-        const bool dynamic = (!mode || *scale <= 0);
-        if (dynamic) {
+    const bool f32dyn = f32in && (!mode || *scale <= 0);
+    const bool i32dyn = (ddt == DT_I32) && (scale[0] < 0 && scale[1] > 0);
+    const bool read_back = f32dyn || i32dyn;
+    const F32 s0 = scale ? scale[0] : 0.0f, s1 = (ddt == DT_I32) ? scale[1] : 0.0f;
+    // attempt 0 may be the one-launch form; if its bounded wait for the grid gives up (another stream held the CUs)
+    // every workgroup has skipped its stores and attempt 1 runs the two-pass form on the same stream
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        float *dscale = nullptr;
+        if (read_back) {
             arm_scale(c);
             dscale = c.hscale_dev;
         }
         bool fused = false;
-        if (dynamic && g_quantize_fused) {  // one launch, one read, where the tensor fits a resident grid's registers
-            HIP_TRY(launch_quantize_fused(dIn, n, dOut, 0, qdt == DT_U8_Q, c.fsync, *scale, dscale, c.stream, &fused));
-        }
-        if (!fused) {
-            if (dynamic) {
-                HIP_TRY(launch_absmax_f32((const float *)dIn, n, c.ws, c.stream));
+        if (f32in) {
+            if (f32dyn && g_quantize_fused && attempt == 0) {  // one launch, one read, where the tensor fits a resident grid's registers
+                HIP_TRY(launch_quantize_fused(dIn, n, dOut, 0, qdt == DT_U8_Q, c.fsync, s0, dscale, c.stream, &fused));
             }
-            HIP_TRY(launch_quantize_f32((const float *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, *scale, nullptr, mode, dscale,
-                c.stream));
-        }
-        read_back = dynamic;
-    } else if (ddt == DT_U8_Q) {
-        HIP_TRY(launch_u8_to_i8((const uint8_t *)dIn, n, (int8_t *)dOut, c.stream));
-    } else {
-        const bool dynamic = (scale[0] < 0 && scale[1] > 0);
-        bool fused = false;
-        if (dynamic) {
-            arm_scale(c);
-            dscale = c.hscale_dev;
-        }
-        if (dynamic && g_quantize_fused) {
-            HIP_TRY(launch_quantize_fused(dIn, n, dOut, 1, qdt == DT_U8_Q, c.fsync, scale[1], dscale, c.stream, &fused));
-        }
-        if (!fused) {
-            if (dynamic) {
-                HIP_TRY(launch_absmax_i32((const int32_t *)dIn, n, c.ws, c.stream));
+            if (!fused) {
+                if (f32dyn) {
+                    HIP_TRY(launch_absmax_f32((const float *)dIn, n, c.ws, c.stream));
+                }
+                HIP_TRY(launch_quantize_f32((const float *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, s0, nullptr, mode, dscale,
+                    c.stream));
             }
-            HIP_TRY(launch_requant_i32((const int32_t *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, scale[0], scale[1], dscale,
-                c.stream));
+        } else if (ddt == DT_U8_Q) {
+            HIP_TRY(launch_u8_to_i8((const uint8_t *)dIn, n, (int8_t *)dOut, c.stream));
+        } else {
+            if (i32dyn && g_quantize_fused && attempt == 0) {
+                HIP_TRY(launch_quantize_fused(dIn, n, dOut, 1, qdt == DT_U8_Q, c.fsync, s1, dscale, c.stream, &fused));
+            }
+            if (!fused) {
+                if (i32dyn) {
+                    HIP_TRY(launch_absmax_i32((const int32_t *)dIn, n, c.ws, c.stream));
+                }
+                HIP_TRY(launch_requant_i32((const int32_t *)dIn, n, dOut, qdt == DT_U8_Q, c.ws, s0, s1, dscale, c.stream));
+            }
         }
-        read_back = dynamic;
+        if (!read_back) {
+            break;
+        }
+        // the scale is a host value in this interface: the call completes before returning it
+        bool gave_up = false;
+        EE te = take_scale(c, scale, fused ? &gave_up : nullptr);
+        if (te != SUCCESS) {
+            return te;
+        }
+        if (!gave_up) {
+            break;
+        }
+        g_fused_fallbacks.fetch_add(1);
     }
     if (arch == AMD_GFX950 && n) {
         HIP_TRY(hipMemcpyAsync(qData, dOut, n, hipMemcpyDeviceToHost, c.stream));
     }
-    if (read_back) {
-        // the scale is a host value in this interface: the call completes before returning it
-        if (arch == AMD_GFX950) {
-            HIP_TRY(hipStreamSynchronize(c.stream));  // host-pointer mode: the copy of the result must have landed
-        }
-        EE te = take_scale(c, scale);
-        if (te != SUCCESS) {
-            return te;
-        }
-    } else if (arch == AMD_GFX950) {
-        HIP_TRY(hipStreamSynchronize(c.stream));
+    if (arch == AMD_GFX950) {
+        HIP_TRY(hipStreamSynchronize(c.stream));  // host-pointer mode: the copy of the result must have landed
     }
     return SUCCESS;
 }

@@ -176,7 +176,9 @@ struct FusedSync {
     uint32_t *counter = nullptr;          // arrivals, never reset
     unsigned long long *release = nullptr;  // 64 words, 8 words apart: (epoch << 32 | max) from the last arrival
     uint32_t epoch = 0, target = 0;
+    uint32_t spin_limit = 1u << 20;       // polls (about a microsecond each) before a waiting workgroup gives up
 };
+constexpr uint32_t kFusedSpinDefault = 1u << 20;
 constexpr size_t kFusedSyncBytes = 64 * 64 + 64 + 64 * 64;
 hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
     float *ds_out, hipStream_t st, bool *taken);

@@ -341,16 +341,37 @@ hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, 
 // Sync area: 64 slots of (epoch << 32 | max bits), one per 64-byte line, folded with a 64-bit atomic max -- a
 // launch's epoch beats whatever older launches left there, so nothing is ever cleared -- an arrival counter
 // that only grows (the host hands each launch the value it reaches when all of its workgroups have arrived),
-// and 64 release words, one per line. The workgroup that arrives last reads the slots and stores
-// (epoch << 32 | max) into every release word; the others poll the release word of their own line (one
-// thread per workgroup, a dozen pollers per line, sleeping between polls). The poll is bounded: a launch whose
-// bound expires publishes a NaN scale, which the host reports as an error instead of returning garbage.
-constexpr uint32_t kFusedSpinLimit = 1u << 20;  // polls of about a microsecond each: about a second
+// and 64 release words, one per line, that carry the launch's OUTCOME: (epoch << 32 | max), or
+// (epoch << 32 | 0xffffffff) when the launch is abandoned. The workgroups poll the release word of their own line
+// (one thread per workgroup, a dozen pollers per line, sleeping between polls) a bounded number of times.
+// The outcome is decided exactly once, by a compare-and-swap on release word 0: the workgroup that arrives last
+// proposes the maximum, a workgroup whose bounded wait expires proposes "abandoned"; whoever swaps first wins, copies
+// the outcome to the other 63 words, and every other workgroup -- including a loser of the swap -- acts on that one
+// outcome. So a launch either quantises everywhere with one maximum, or stores nothing anywhere and publishes a NaN
+// scale, on which the host runs the two-pass form: never a valid scale over partly written output.
+constexpr uint32_t kFusedAbandoned = 0xffffffffu;  // never a maximum: those are non-negative floats' bits, ints >= 0 or INT32_MIN
+
+// proposes `value` as this epoch's outcome on release word 0 and returns the outcome that stands
+__device__ __forceinline__ uint32_t fused_decide(unsigned long long *release, uint32_t epoch, uint32_t value, bool *won)
+{
+    const unsigned long long mine = ((unsigned long long)epoch << 32) | value;
+    unsigned long long cur = __hip_atomic_load(release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *won = false;
+    while ((uint32_t)(cur >> 32) != epoch) {
+        const unsigned long long seen = atomicCAS(release, cur, mine);
+        if (seen == cur) {
+            *won = true;
+            return value;
+        }
+        cur = seen;
+    }
+    return (uint32_t)cur;
+}
 
 template <int SRC_I32, int TO_U8, int PER>
 __global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restrict__ xin, uint32_t n, uint8_t *__restrict__ q,
     unsigned long long *slots, uint32_t *counter, unsigned long long *release, uint32_t epoch, uint32_t target, float s_in,
-    float *ds_out)
+    float *ds_out, uint32_t spin_limit)
 {
     __shared__ int red[4];
     __shared__ int bcast[2];
@@ -402,34 +423,59 @@ __global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restr
     }
     __syncthreads();
     if (bcast[1] == 2) {
-        if (wave == 0) {  // every fold is complete: take the maximum and release the others
+        if (wave == 0) {  // every fold is complete: take the maximum and propose it as the outcome
             __threadfence();
             const unsigned long long t = __hip_atomic_load(slots + lane * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             int v = ((uint32_t)(t >> 32) == epoch) ? (int)(uint32_t)t : 0;
             v = wave_reduce_max_i(v);
-            __hip_atomic_store(release + lane * 8, ((unsigned long long)epoch << 32) | (uint32_t)v, __ATOMIC_RELAXED,
-                __HIP_MEMORY_SCOPE_AGENT);
+            uint32_t outcome = 0;
+            bool won = false;
             if (lane == 0) {
-                bcast[0] = v;
+                outcome = fused_decide(release, epoch, (uint32_t)v, &won);
+            }
+            outcome = (uint32_t)__shfl((int)outcome, 0, 64);
+            won = __shfl((int)won, 0, 64) != 0;
+            if (won && lane != 0) {
+                __hip_atomic_store(release + lane * 8, ((unsigned long long)epoch << 32) | outcome, __ATOMIC_RELAXED,
+                    __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (lane == 0) {
+                bcast[0] = (int)outcome;
             }
         }
     } else if (threadIdx.x == 0) {
         uint32_t spins = 0;
         unsigned long long t;
-        while ((uint32_t)((t = __hip_atomic_load(release + (blockIdx.x & 63) * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) !=
-            epoch) {
-            __builtin_amdgcn_s_sleep(2);
-            if (++spins > kFusedSpinLimit) {
-                bcast[1] = 0;  // gave up
-                t = 0;
+        uint32_t outcome;
+        for (;;) {
+            t = __hip_atomic_load(release + (blockIdx.x & 63) * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((uint32_t)(t >> 32) == epoch) {
+                outcome = (uint32_t)t;
                 break;
             }
+            if (++spins > spin_limit) {  // give up: propose "abandoned", unless the outcome has been decided meanwhile
+                bool won = false;
+                outcome = fused_decide(release, epoch, kFusedAbandoned, &won);
+                if (won) {
+                    for (uint32_t k = 1; k < 64; ++k) {
+                        __hip_atomic_store(release + k * 8, ((unsigned long long)epoch << 32) | kFusedAbandoned, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
         }
-        bcast[0] = (int)(uint32_t)t;
+        bcast[0] = (int)outcome;
     }
     __syncthreads();
+    if ((uint32_t)bcast[0] == kFusedAbandoned) {  // the same for every workgroup of the launch: nothing is stored
+        if (tid == 0 && ds_out) {
+            *ds_out = __int_as_float(0x7fc00000);
+        }
+        return;
+    }
     const int gmax = bcast[0];
-    const bool ok = bcast[1] != 0;
     float s, published;
     if (SRC_I32) {  // avx512/quantize.cpp:315-416 with scale[0] < 0: r = 127 / max, returned scale = scale[1] * r
         s = (gmax == 0) ? 1.0f : 127.0f / (float)gmax;
@@ -441,7 +487,7 @@ __global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restr
         published = s;
     }
     if (tid == 0 && ds_out) {
-        *ds_out = ok ? published : __int_as_float(0x7fc00000);
+        *ds_out = published;
     }
 #define BG_QF(bits)                                                                                        \
     ((unsigned)(SRC_I32 ? (TO_U8 ? usat8_u(rne_i32((float)(bits)*s + 128.0f)) : ssat8(rne_i32((float)(bits)*s))) \
@@ -493,7 +539,7 @@ static hipError_t launch_fused(const void *x, uint32_t n, void *q, FusedSync &fs
     fs.epoch += 1;
     fs.target += grid;
     hipLaunchKernelGGL((quantize_fused_kernel<SRC_I32, TO_U8, PER>), dim3(grid), dim3(256), 0, st, x, n, (uint8_t *)q, fs.slots,
-        fs.counter, fs.release, fs.epoch, fs.target, s_in, ds_out);
+        fs.counter, fs.release, fs.epoch, fs.target, s_in, ds_out, fs.spin_limit);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         fs.epoch -= 1;  // nothing ran: the counter must not be waited for

@@ -15,6 +15,10 @@
  *                      quantisation, u8 results with a dynamic output scale) returns as soon as that
  *                      scale has reached the host; its tensors follow in stream order.
  * Errors come back as Bolt's EE codes; nothing here calls exit().
+ *
+ * Threads: like the reference, every function is re-entrant on disjoint buffers. Each calling thread has its own
+ * context (stream, scratch words, staging buffers, last-error text): bolt_gfx950_set_stream, _synchronize, _last_error,
+ * _timer_* and the "quantize_fused_spin" option act on the calling thread's context; the other options are process-wide.
  */
 #ifndef BOLT_GFX950_H
 #define BOLT_GFX950_H
@@ -34,8 +38,9 @@ extern "C" {
 /* ---- runtime ------------------------------------------------------------------------- */
 /* No counterpart in the reference (a CPU library needs no device context). */
 EE bolt_gfx950_init(void);
-/* stream: a hipStream_t (NULL = the default stream). The library never creates streams. Changing the
- * stream first waits for the work enqueued on the previous one (the library's scratch is shared). */
+/* stream: a hipStream_t (NULL = the default stream) for the calling thread's calls. The library never creates
+ * streams. Changing the stream first waits for the work this thread enqueued on the previous one (the thread's
+ * scratch words are shared by its calls). */
 EE bolt_gfx950_set_stream(void *stream);
 EE bolt_gfx950_synchronize(void);
 const char *bolt_gfx950_last_error(void);
@@ -59,8 +64,12 @@ const char *bolt_gfx950_last_error(void);
  * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount).
  * "lstm_gemm_rows" (>= 1, default 4): the LSTM cell sends calls with at least this many batch rows through the
  * matrix cores when its weight carries the GEMM packing (rnn_transform_filter_gfx950). Every variant
- * returns the same bytes. */
+ * returns the same bytes. "quantize_fused_spin" (calling thread only): polls of the one-launch quantiser's bounded wait
+ * before a workgroup gives up and the call falls back to two passes (0 = default, about a second; tests use 1). */
 EE bolt_gfx950_set_option(const char *name, int value);
+/* Event counters for tests and monitoring: "quantize_fused_fallbacks" = dynamic quantisations whose one-launch form
+ * gave up waiting for its grid (the CUs were held by other work) and were redone in two passes. NOT_FOUND otherwise. */
+EE bolt_gfx950_get_counter(const char *name, unsigned long long *value);
 void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);
 EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes);

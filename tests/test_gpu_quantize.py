@@ -258,3 +258,50 @@ def test_static_then_dynamic_without_sync(torch_mod, oracle):
                 assert s_static[0] == np.float32(17.5) and s_req[0] == np.float32(0.011)
         finally:
             capi.check(L.bolt_gfx950_set_option(b"quantize_fused", 1), "set_option")
+
+
+def test_one_launch_quantiser_falls_back_when_its_wait_gives_up(torch_mod, oracle):
+    """The one-launch dynamic quantiser waits for its whole grid a bounded number of polls. With the bound forced to
+    one poll from the host, launches of more than a few workgroups give up: every workgroup then skips its stores,
+    the kernel publishes a NaN scale and exits normally, and the call is redone in two passes. Bytes and scale must be
+    the oracle's either way, and the fallback counter must have moved."""
+    torch = torch_mod
+    L = capi.lib()
+    import ctypes as C
+    before = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(before)), "counter")
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 1), "set_option")
+    try:
+        rng = np.random.default_rng(31)
+        for n in (1000, 65536, 262144 + 16, 1 << 19):
+            x = (rng.standard_normal(n) * 2.5).astype(np.float32)
+            acc = rng.integers(-900000, 900000, size=n, dtype=np.int32)
+            dx, dacc = torch.from_numpy(x).cuda(), torch.from_numpy(acc).cuda()
+            for rep in range(3):
+                print("fused fallback", n, rep, flush=True)
+                for qdt in (DT_U8_Q, DT_I8):
+                    want, ws = oracle.quantize_f32(x, qdt)
+                    s = [-1.0]
+                    q = host.quantize(dx, DT_F32, qdt, s)
+                    capi.check(L.bolt_gfx950_synchronize(), "sync")
+                    assert s[0] == ws and np.array_equal(q.cpu().numpy(), want), (n, rep, qdt)
+                    want2, ws2 = oracle.quantize_i32(acc, qdt, [-1.0, 0.37])
+                    s2 = [np.float32(-1.0), np.float32(0.37)]
+                    q2 = host.quantize(dacc, DT_I32, qdt, s2)
+                    capi.check(L.bolt_gfx950_synchronize(), "sync")
+                    assert np.array_equal(np.array(s2, np.float32), ws2) and np.array_equal(q2.cpu().numpy(), want2), (n, rep, qdt)
+                    assert np.array_equal(host.quantize(x, DT_F32, qdt, [-1.0]), want)     # host-pointer mode too
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 0), "set_option")
+    after = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(after)), "counter")
+    assert after.value > before.value, "no launch gave up: the test did not exercise the fallback"
+    # and with the default bound the one-launch form completes again
+    s = [-1.0]
+    q = host.quantize(dx, DT_F32, DT_U8_Q, s)
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    want, ws = oracle.quantize_f32(x, DT_U8_Q)
+    assert s[0] == ws and np.array_equal(q.cpu().numpy(), want)
+    final = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(final)), "counter")
+    assert final.value == after.value
