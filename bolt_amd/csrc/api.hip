@@ -143,6 +143,9 @@ int g_lstm_gemm_rows = 4;
 // dynamic quantisation through the public entry points: 1 = one launch that reads the tensor once where
 // it fits (default), 0 = always the two-pass form (scratch fill, abs-max, quantise)
 int g_quantize_fused = 1;
+// encoder layer: 1 = the FullyConnected in front of the GELU also applies the GELU and quantises its result for the
+// next FullyConnected, in one launch (where the shape allows; default); 0 = separate kernels, fp32 intermediate kept
+int g_encoder_fused = 1;
 
 EE ensure_init()
 {
@@ -182,8 +185,7 @@ EE ensure_init()
             return fail(ALLOC_FAILED, "hipMalloc(quantiser sync area)", e);
         }
         c.fsync.slots = (unsigned long long *)p;
-        c.fsync.counter = (uint32_t *)((uint8_t *)p + 64 * 64);
-        c.fsync.release = (unsigned long long *)((uint8_t *)p + 64 * 64 + 64);
+        c.fsync.decide = (unsigned long long *)((uint8_t *)p + kGridSyncMaxBlocks * 8);
     }
     if (!c.hscale) {
         e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
@@ -497,6 +499,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         ctx().fsync.spin_limit = value ? (uint32_t)value : kFusedSpinDefault;
+        return SUCCESS;
+    }
+    if (strcmp(name, "encoder_fused") == 0) {
+        if (value != 0 && value != 1) {
+            return NOT_MATCH;
+        }
+        g_encoder_fused = value;
         return SUCCESS;
     }
     if (strcmp(name, "quantize_fused") == 0) {
@@ -3028,7 +3037,7 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
 // ---- BERT-style int8 encoder layer --------------------------------------------------------------------
 namespace {
 struct EncoderPlan {
-    size_t ws, scales, xq, qkv, ctx, ao, h1, f, o, total;
+    size_t ws, scales, xq, xq2, qkv, ctx, ao, h1, f, o, total;
 };
 
 EncoderPlan encoder_plan(const BoltEncoderLayerInt8 &L)
@@ -3043,7 +3052,8 @@ EncoderPlan encoder_plan(const BoltEncoderLayerInt8 &L)
     };
     p.ws = take(4 * kWsWords * sizeof(uint32_t));
     p.scales = take(64);
-    p.xq = take(T * (F > H ? F : H));  // one u8 buffer reused by the four quantised activations
+    p.xq = take(T * H);   // u8 input of the three FullyConnected layers that read [T, H]
+    p.xq2 = take(T * F);  // u8 input of the last one, [T, F] (written while the one before it still reads xq)
     p.qkv = take(T * 3 * H * 4);
     p.ctx = take(T * H * 4);
     p.ao = take(T * H * 4);
@@ -3132,7 +3142,7 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     U8 *w = (U8 *)workspace;
     const U32 T = L.batch * L.seq, H = L.hidden, F = L.ffn;
     float *sc = (float *)(w + p.scales);
-    uint8_t *xq = w + p.xq;
+    uint8_t *xq = w + p.xq, *xq2 = w + p.xq2;
     float *qkv = (float *)(w + p.qkv), *cx = (float *)(w + p.ctx), *ao = (float *)(w + p.ao), *h1 = (float *)(w + p.h1),
           *f = (float *)(w + p.f), *o = (float *)(w + p.o);
 
@@ -3175,11 +3185,46 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     HIP_TRY(gemm(xq, L.wo, H, H, sc + 1, L.so, L.bo, ao));
     HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st, ws1));
     HIP_TRY(launch_quantize_f32(h1, T * H, xq, 1, ws2, 0.0f, nullptr, 0, sc + 2, st));
-    HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
-    // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads
-    HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st, false, ws2));
-    HIP_TRY(launch_quantize_f32(f, T * F, xq, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 1));
-    HIP_TRY(gemm(xq, L.w2, H, F, sc + 3, L.s2, L.b2, o));
+    if (g_encoder_fused && gemm_gelu_dyn_fits(T, F, H)) {
+        // FullyConnected + GELU + dynamic quantisation in one launch: the accumulators stay in registers across a
+        // grid-wide agreement on max|gelu|; the [T, F] fp32 tensor is never written. Should that agreement be abandoned
+        // (the CUs were held by other work), the kernel leaves the activated values in f and sets the status word,
+        // and the two kernels behind it -- which otherwise return at once -- quantise them in two passes.
+        uint32_t *status = (uint32_t *)(sc + 8);
+        const uint32_t tiles = (T / 256) * (F / 256);
+        GemmArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = xq;
+        g.lda = H;
+        g.Bp = (const int8_t *)L.w1;
+        g.M = T;
+        g.N = F;
+        g.K = H;
+        g.comp = (const int32_t *)((const U8 *)L.w1 + packed_matrix_bytes(F, H));
+        g.ob = g.comp;
+        g.C = xq2;
+        g.epi.mode = EPI_U8_GELU_DYN;
+        g.epi.scaleI = sc + 2;
+        g.epi.scaleW = L.s1;
+        g.epi.bias = L.b1;
+        g.sync = c.fsync.next(tiles);
+        g.dscale_out = sc + 3;
+        g.status = status;
+        g.C32 = f;
+        g.clear_ws = ws2;  // consumed by the quantiser in front of this product
+        hipError_t he = launch_gemm_u8s8(g, st);
+        if (he != hipSuccess) {
+            return fail(UNKNOWN, "launch_gemm_u8s8 (GELU epilogue)", he);
+        }
+        HIP_TRY(launch_absmax_f32(f, T * F, ws3, st, true, status));
+        HIP_TRY(launch_quantize_f32(f, T * F, xq2, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 0, status));
+    } else {
+        HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
+        // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads
+        HIP_TRY(launch_gelu_f32(f, (size_t)T * F, ws3, st, false, ws2));
+        HIP_TRY(launch_quantize_f32(f, T * F, xq2, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 1));
+    }
+    HIP_TRY(gemm(xq2, L.w2, H, F, sc + 3, L.s2, L.b2, o));
     HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st, ws3));
     c.enc_ws_dirty = false;
     return SUCCESS;

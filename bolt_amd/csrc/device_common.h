@@ -41,7 +41,10 @@ enum EpiMode : int {
     EPI_F32 = 1,       // cvt(acc) * factor                      (factor = 1.0f / scale[0])
     EPI_U8 = 2,        // usat8_u(rne(cvt(acc) * factor) + 128)  (factor = scale[1])
     EPI_F32_CH = 3,    // cvt(acc) * (1.0f / (sI * sW[n])) + bias[n]   per-output-channel extension
-    EPI_U8_TRUNC = 4   // (int)(cvt(acc) * factor + 128.0f), > 255 -> 255, else low byte
+    EPI_U8_TRUNC = 4,  // (int)(cvt(acc) * factor + 128.0f), > 255 -> 255, else low byte
+    // y = gelu_tanh(cvt(acc) * (1.0f / (sI * sW[n])) + bias[n]); u8 = quantise(y) with the tensor-wide dynamic scale
+    // max(0, 127 / max|y|), the maximum agreed on by all workgroups of the launch while y is still in registers
+    EPI_U8_GELU_DYN = 5
 };
 
 struct Epilogue {
@@ -165,13 +168,37 @@ __device__ __forceinline__ int wave_reduce_max_i(int v)
     return v;
 }
 
-// tanh-form GELU: x * 0.5 * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3))), with tanh(u/2) written as 1 - 2 / (1 + e^u)
+// tanh-form GELU: x * 0.5 * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3))). With u = 2 sqrt(2/pi) (x + 0.044715 x^3),
+// 0.5 (1 + tanh(u / 2)) = 1 - 1 / (1 + e^u), so gelu(x) = x - x / (1 + e^u): eight instructions, two of them
+// transcendental (e^u as 2^(u log2 e) with the factor folded into the constant; v_exp_f32 and v_rcp_f32 are 1 ulp,
+// far inside the layer's tolerance). x -> -inf gives e^u = 0 and x - x = 0, x -> +inf gives 1 / inf = 0 and x.
 __device__ __forceinline__ float gelu_tanh(float x)
 {
-    const float c0 = 1.5957691216057308f;  // 2 * sqrt(2 / pi)
+    const float c0 = 2.3022082f;  // 2 * sqrt(2 / pi) * log2(e)
     const float u = (c0 * x) * __builtin_fmaf(0.044715f, x * x, 1.0f);
-    const float e = __expf(u);
-    return (2.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e)) * (0.5f * x);  // v_rcp_f32: 1 ulp, far inside the layer's tolerance
+    const float e = __builtin_amdgcn_exp2f(u);
+    return __builtin_fmaf(-x, __builtin_amdgcn_rcpf(1.0f + e), x);
+}
+
+// fp32 -> u8 around the zero point 128 for values known to satisfy |x * s| <= 127 (1 + 2^-22) -- a tensor quantised
+// with the dynamic scale 127 / max|x| of its own maximum: the same bytes as q_u8 in four instructions. The sum with
+// 2^23 rounds t + 128 (already rounded to fp32 once, like q_u8's) to the nearest-even integer and leaves it in the
+// low mantissa bits; clamping to [1, 255] before that rounding equals clamping after it (both are monotone).
+// Returns the word whose low byte is the result. NaN quantises to 1 as in q_u8 (v_med3_f32 drops it).
+__device__ __forceinline__ uint32_t q_u8_inrange_bits(float x, float s)
+{
+    const float t = x * s;
+    const float u = t + 128.0f;
+    const float w = __builtin_amdgcn_fmed3f(u, 1.0f, 255.0f);
+    return __float_as_uint(w + 8388608.0f);
+}
+
+// low bytes of four words -> one dword (byte 0 = a)
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
+{
+    const uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // byte 0 = a[0], byte 1 = b[0], upper bytes 0
+    const uint32_t cd = __builtin_amdgcn_perm(d, c, 0x04000c0cu);  // byte 2 = c[0], byte 3 = d[0], lower bytes 0
+    return ab | cd;
 }
 
 // ---- tensor-wide max through device scratch words --------------------------------------------------
@@ -210,6 +237,118 @@ __device__ __forceinline__ void ws_block_fold_max(uint32_t *ws, int v, int *red)
 __device__ __forceinline__ int ws_read_max(const uint32_t *ws)
 {
     return wave_reduce_max_i((int)ws[(threadIdx.x & (kWsSlots - 1)) * kWsStride]);
+}
+
+// ---- grid-wide maximum with a bounded wait ------------------------------------------------------------
+// For kernels whose workgroups are all resident at once (the launcher sizes the grid for that) and that must
+// agree on one tensor-wide maximum half way through, with their partial results still in registers.
+//
+// Sync area (device memory, zeroed once when allocated, never cleared afterwards): one 64-bit slot per workgroup
+// (at most kGridSyncMaxBlocks) and one 64-bit decision word. A launch carries an epoch that grows with every launch.
+// Every workgroup stores (epoch << 32 | its maximum) into its own slot -- one store, nothing to wait for -- and then
+// its first wave polls ALL slots of the grid (64 per load instruction) until each carries this launch's epoch; the
+// maximum over them is the same in every workgroup. That is one store and one or two rounds of loads end to end;
+// a counter that the last arrival turns into a release word costs five dependent trips to memory instead.
+//
+// The wait is bounded, and its outcome is decided exactly once through the decision word:
+//   a workgroup that has seen every slot proposes (epoch, COMMITTED) with a compare-and-swap, unless it already
+//   reads that; a workgroup whose bound expires proposes (epoch, ABANDONED). Whoever swaps first wins and every
+//   workgroup acts on the one outcome: after COMMITTED all slots are known to be present (a workgroup whose bound
+//   expired just then simply reads them), after ABANDONED nobody uses the maximum.
+// So all workgroups of a launch see the same maximum, or all see "abandoned" (kGridAbandoned).
+// Launches that share a sync area must be ordered on one stream.
+constexpr uint32_t kGridSyncMaxBlocks = 1024;
+struct GridSync {
+    unsigned long long *slots = nullptr;   // kGridSyncMaxBlocks words
+    unsigned long long *decide = nullptr;  // one word (on a cache line of its own)
+    uint32_t epoch = 0;        // this launch's tag
+    uint32_t blocks = 0;       // workgroups in the launch (gridDim.x, <= kGridSyncMaxBlocks)
+    uint32_t spin_limit = 0;   // polling rounds (a microsecond or two each) before a waiting workgroup gives up
+};
+constexpr uint32_t kGridAbandoned = 0xffffffffu;  // never a maximum: those are non-negative floats' bits, ints >= 0 or INT32_MIN
+constexpr uint32_t kGridCommitted = 1u, kGridGaveUp = 2u;
+
+// Called by every thread of every workgroup of the launch (uniform control flow) with its own candidate `m`
+// (values whose signed-integer order is the wanted order: non-negative floats' bits or ints). `lds`: 18 ints of
+// the workgroup's LDS; workgroups of whole waves, at most 16; blockIdx.x numbers the workgroups. Returns the
+// grid-wide maximum or kGridAbandoned, the same value in every thread of the grid.
+__device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int *lds)
+{
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    m = wave_reduce_max_i(m);
+    if (lane == 0) {
+        lds[wave] = m;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int mine = (lane < waves) ? lds[lane] : (int)0x80000000;
+        mine = wave_reduce_max_i(mine);
+        const unsigned long long tag = (unsigned long long)gs.epoch << 32;
+        if (lane == 0) {
+            __hip_atomic_store(gs.slots + blockIdx.x, tag | (uint32_t)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        uint32_t spins = 0, outcome = kGridAbandoned;
+        bool committed = false;  // the decision is known to be COMMITTED: every slot is (about to be) visible
+        for (;;) {
+            bool ok = true;
+            int v = (int)0x80000000;
+            for (uint32_t b = lane; b < gs.blocks; b += 64) {
+                const unsigned long long t = __hip_atomic_load(gs.slots + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = ok && ((uint32_t)(t >> 32) == gs.epoch);
+                const int tv = (int)(uint32_t)t;
+                v = tv > v ? tv : v;
+            }
+            unsigned long long d = __hip_atomic_load(gs.decide, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const bool all = __all(ok);
+            uint32_t state = ((uint32_t)(d >> 32) == gs.epoch) ? (uint32_t)d : 0u;
+            if (state == kGridGaveUp) {
+                break;
+            }
+            if (all) {
+                if (state != kGridCommitted && !committed) {
+                    if (lane == 0) {  // propose COMMITTED; a different epoch-tagged value in the word means someone decided first
+                        for (;;) {
+                            const unsigned long long seen = atomicCAS(gs.decide, d, tag | kGridCommitted);
+                            if (seen == d || (uint32_t)(seen >> 32) == gs.epoch) {
+                                state = (seen == d) ? kGridCommitted : (uint32_t)seen;
+                                break;
+                            }
+                            d = seen;
+                        }
+                    }
+                    state = (uint32_t)__shfl((int)state, 0, 64);
+                }
+                if (state != kGridGaveUp) {
+                    outcome = (uint32_t)wave_reduce_max_i(v);
+                }
+                break;
+            }
+            committed = committed || state == kGridCommitted;
+            if (!committed && ++spins > gs.spin_limit) {
+                if (lane == 0) {  // give up: propose ABANDONED, unless the outcome has been decided meanwhile
+                    for (;;) {
+                        const unsigned long long seen = atomicCAS(gs.decide, d, tag | kGridGaveUp);
+                        if (seen == d || (uint32_t)(seen >> 32) == gs.epoch) {
+                            state = (seen == d) ? kGridGaveUp : (uint32_t)seen;
+                            break;
+                        }
+                        d = seen;
+                    }
+                }
+                state = (uint32_t)__shfl((int)state, 0, 64);
+                if (state == kGridGaveUp) {
+                    break;
+                }
+                committed = true;  // someone saw every slot just now: read them
+            }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (lane == 0) {
+            lds[17] = (int)outcome;
+        }
+    }
+    __syncthreads();
+    return (uint32_t)lds[17];
 }
 
 }  // namespace bg

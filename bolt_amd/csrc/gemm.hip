@@ -472,6 +472,110 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
 #undef BG_LOAD_CIN
 }
 
+// EPI_U8_GELU_DYN: the FullyConnected in front of a GELU whose result the next FullyConnected wants quantised with a
+// tensor-wide dynamic scale. Written as separate kernels that is an fp32 matrix stored, read for max|gelu|, and read
+// again to be quantised; here the accumulators never leave the registers:
+//   y = gelu_tanh(cvt(acc + base) * (1 / (sI * sW[n])) + bias[n])     (kept in the accumulator registers)
+//   max|y| over the whole result through grid_max_sync               (every tile's workgroup is resident)
+//   u8 = q_u8(y, max(0, 127 / max|y|)), scale published through dscale_out
+// -- the arithmetic, element for element, of the per-channel fp32 epilogue, gelu_f32_kernel's maximum and
+// quantize_f32_kernel<u8, gelu>. If the grid-wide wait is abandoned nothing is quantised: every workgroup stores its
+// y as fp32 into C32 and status becomes 1, on which the two conditional kernels behind this one do the two passes.
+// Full 256 x 256 tiles only (the launcher checks).
+template <int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
+{
+    static_assert(TN == 4, "a wave's tile row must be 64 columns");
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const float sI = *a.epi.scaleI;
+    if (a.clear_ws && blockIdx.x == 0) {
+        for (uint32_t k = threadIdx.x; k < kWsWords; k += blockDim.x) {
+            a.clear_ws[k] = 0;
+        }
+    }
+    // every per-column term first, in one batch of loads (a load per use would put a trip to memory into each step)
+    uint32_t base[TN][4];
+    float qs[TN][4], bs[TN][4];
+#pragma unroll
+    for (int y = 0; y < TN; ++y) {
+        const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+        const v4i cb = *(const v4i *)(a.comp + n);
+        const v4i ob = *(const v4i *)(a.ob + n);
+        const v4f sw = *(const v4f *)(a.epi.scaleW + n);
+        const v4f bi = a.epi.bias ? *(const v4f *)(a.epi.bias + n) : (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            base[y][c] = (uint32_t)ob[c] - (uint32_t)cb[c];
+            qs[y][c] = 1.0f / (sI * sw[c]);
+            bs[y][c] = bi[c];
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float f = (float)(int)((uint32_t)acc[x][y][c] + base[y][c]) * qs[y][c];
+                if (a.epi.bias) {
+                    f = f + bs[y][c];
+                }
+                const float v = gelu_tanh(f);
+                amax = fmaxf(amax, fabsf(v));
+                acc[x][y][c] = __float_as_int(v);
+            }
+        }
+    }
+    const uint32_t outcome = grid_max_sync(a.sync, (int)__float_as_uint(amax), (int *)smem);
+    if (outcome == kGridAbandoned) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            *a.status = 1u;
+        }
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+                *(v4i *)(a.C32 + (size_t)m * a.N + n) = acc[x][y];
+            }
+        }
+        return;
+    }
+    const float mx = __uint_as_float(outcome);
+    const float s = (mx == 0.0f) ? 1.0f : 127.0f / mx;  // resolve_scale with no caller's scale: max(0, 127 / max)
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *a.status = 0u;
+        *a.dscale_out = s;
+    }
+    // u8 rows through a wave-private LDS panel of 16 rows x 64 bytes (pitch 80: the 4-byte writes of the fragment
+    // layout and the 16-byte reads of the row layout are both free of bank conflicts), so that a store instruction
+    // covers 16 rows x 64 contiguous bytes instead of 16 rows x 16 bytes. LDS operations of one wave execute in order.
+    constexpr uint32_t kPitch = 80;
+    uint8_t *pan = smem + 256 + wave * (16 * kPitch);
+    uint8_t *wr = pan + i * kPitch + g * 4;                      // + 16 * y
+    const uint8_t *rd = pan + (lane >> 2) * kPitch + (lane & 3) * 16;
+    uint8_t *out = (uint8_t *)a.C + (size_t)(m0 + wm * TM * 16 + (lane >> 2)) * a.N + n0 + wn * 64 + (lane & 3) * 16;
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const v4i v = acc[x][y];  // |v * s| <= 127: s comes from the maximum of these very values
+            *(uint32_t *)(wr + 16 * y) = pack_low_bytes(q_u8_inrange_bits(__int_as_float(v.x), s), q_u8_inrange_bits(__int_as_float(v.y), s),
+                q_u8_inrange_bits(__int_as_float(v.z), s), q_u8_inrange_bits(__int_as_float(v.w), s));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        const v4i row = *(const v4i *)rd;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        *(v4i *)(out + (size_t)x * 16 * a.N) = row;
+    }
+}
+
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
@@ -709,7 +813,9 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 // FP4 (1-bit convolution only): the operand bytes hold two E2M1 values each (+1 = 0x2, -1 = 0xA, 0 = 0x0) and the
 // products are formed by v_mfma_scale_f32_16x16x128_f8f6f4 -- twice the K per instruction at the same rate, fp32
 // accumulation that is exact for these integers; the accumulators are converted to int32 before the epilogue.
-template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false, bool FP4 = false>
+// GELU_DYN: the kernel ends in the EPI_U8_GELU_DYN epilogue and nothing else (an instantiation of its own, so that
+// the registers that epilogue needs do not burden the others).
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false, bool FP4 = false, bool GELU_DYN = false>
 // Two waves per SIMD are asked for also where a workgroup has four waves: with a budget of 512 registers per lane
 // the compiler keeps the accumulators in AGPRs and spends dozens of v_accvgpr moves per K tile on shuffling them.
 __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs a)
@@ -749,6 +855,12 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
         const uint32_t n = n0 + wn * TN * 16 + lane;
         if (lane < TN * 16 && n < a.N) {
             warm = (a.fold_bias ? __float_as_int(a.fold_bias[n]) : a.ob[n]) ^ a.comp[n];
+            if (a.epi.scaleW) {
+                warm ^= __float_as_int(a.epi.scaleW[n]);
+            }
+            if (a.epi.bias) {
+                warm ^= __float_as_int(a.epi.bias[n]);
+            }
         }
     }
 
@@ -1199,7 +1311,11 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     }
-    epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+    if constexpr (GELU_DYN) {
+        epilogue_gelu_sync<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+    } else {
+        epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
+    }
 }
 
 // Convolution with few output channels (N <= 64) and a filter panel that fits in LDS (K <= 1024).
@@ -1429,12 +1545,12 @@ __global__ __launch_bounds__(512) void gemm_u8s8_skinny_kernel(GemmArgs a)
     epilogue_panel<1, 1, 4, 1>(a, acc, nullptr, lane, 0u, m0, n0, 0);
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false, bool FP4 = false>
+template <int WM, int WN, int TM, int TN, int STAGES, int PIPE = 0, bool CONV = false, bool FP4 = false, bool GELU_DYN = false>
 static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     static bool attr_set = false;
-    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV, FP4>;
+    auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV, FP4, GELU_DYN>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
         if (e != hipSuccess) {
@@ -1564,6 +1680,22 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
 
 static int g_force_tile = -1;  // test hook: -1 = heuristic
 
+// Whether the GELU-and-quantise epilogue (EPI_U8_GELU_DYN) can run for this product: full 256 x 256 tiles of a pipelined
+// kernel, few enough of them that each gets a CU of its own at once (160 KB of LDS per workgroup: one per CU).
+bool gemm_gelu_dyn_fits(uint32_t M, uint32_t N, uint32_t K)
+{
+    static int cus = -1;
+    if (cus < 0) {
+        int dev = 0, n = 0;
+        cus = (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) ? n : 0;
+    }
+    if (M == 0 || N == 0 || M % 256 != 0 || N % 256 != 0 || K % 64 != 0 || K < 64) {
+        return false;
+    }
+    const uint64_t tiles = (uint64_t)(M / 256) * (N / 256);
+    return tiles >= 128 && tiles <= (uint64_t)cus && g_force_tile < 0;
+}
+
 void gemm_force_tile(int t)
 {
     g_force_tile = t;
@@ -1600,6 +1732,18 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     }
     if (tile == 12 && (a.K % 128 != 0 || !lds_160k())) {
         tile = 11;
+    }
+    if (a.epi.mode == EPI_U8_GELU_DYN) {
+        // every tile's workgroup must be running when the first one waits for the others: full 256 x 256 tiles, one
+        // workgroup per CU, and the sync area, status word and fallback buffer in place
+        if ((tile != 11 && tile != 12) || !gemm_gelu_dyn_fits(a.M, a.N, a.K) || !a.sync.slots || !a.status || !a.C32 || !a.dscale_out ||
+            !a.epi.scaleI || !a.epi.scaleW || a.sync.blocks == 0 || a.sync.blocks > kGridSyncMaxBlocks) {
+            return hipErrorInvalidValue;
+        }
+        if (tile == 12) {
+            return launch_dma<2, 4, 8, 4, 5, 3, false, false, true>(a, st);
+        }
+        return launch_dma<2, 4, 8, 4, 4, 2, false, false, true>(a, st);
     }
     switch (tile) {
         case 2:

@@ -80,8 +80,16 @@ struct GemmArgs {
     int fp4 = 0;             // convolution only: operand bytes are pairs of E2M1 values (1-bit convolution), K counts bytes
     Epilogue epi;
     ConvGeom conv;       // used by launch_conv_u8s8 only
+    // EPI_U8_GELU_DYN only (256 x 256 tiles, M and N multiples of 256, every workgroup resident at once):
+    GridSync sync;                 // from FusedSync::next(number of tiles)
+    float *dscale_out = nullptr;   // receives the scale the u8 result was quantised with
+    uint32_t *status = nullptr;    // receives 0; or 1 when the grid-wide wait was abandoned: then nothing was quantised and
+    float *C32 = nullptr;          //   the activated fp32 values y are in C32 [M][N] for a two-pass quantisation to pick up
+    uint32_t *clear_ws = nullptr;  // optional: an array of kWsWords max slots whose maximum has been consumed; zeroed by one workgroup
 };
 hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st);
+// whether EPI_U8_GELU_DYN can run for an M x N x K product on the current device (grid of that many tiles = M / 256 * N / 256)
+bool gemm_gelu_dyn_fits(uint32_t M, uint32_t N, uint32_t K);
 // A = padded s8 image, M = n * OH * OW output pixels, N = output channels, K = fh * fw * ICp
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
 bool conv_fp4_ok(uint32_t M, uint32_t N);
@@ -148,12 +156,14 @@ hipError_t launch_pack_mvm(const int8_t *src, uint32_t sk, uint32_t sn, uint32_t
 // ---- quantize family ----------------------------------------------------------------------------
 // Device scratch word layout used by the two-pass kernels: ws[0] = max bits / max int.
 // folds max |x| into the scratch slots ws; clears them first unless the caller just did
-hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear = false);
+// only_if (device word, optional): the kernel does nothing unless *only_if != 0
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear = false,
+    const uint32_t *only_if = nullptr);
 // Caller's scale = *ds_in (device) if given, else s_in. Dynamic when !mode or that scale <= 0:
 // the scale used is max(caller's, 127 / max|x|) with max|x| taken from ws[0]. The scale used is
 // written to *ds_out (device) when non-null.
 hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
-    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu = 0);
+    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu = 0, const uint32_t *only_if = nullptr);
 hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st);
 // s0 = output scale (< 0: dynamic from ws[0]), s1 = scale of the int32 data; the resulting output
 // scale is written to *ds_out (device) when non-null.
@@ -170,16 +180,28 @@ hipError_t launch_bias_offsetC(const float *bias, uint32_t N, const int32_t *off
 hipError_t launch_requantize_i8(const int8_t *in, uint32_t n, float rescale, int8_t *out, hipStream_t st);
 hipError_t launch_axpby_f32(uint32_t n, float a, const float *x, float b, float *y, hipStream_t st);  // y = fma(a, x, y * b)
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
-// One-launch dynamic quantisation (quantize.hip): device sync area and the host's running epoch / arrival target
+// Host side of a GridSync area (device_common.h): the device words and the running epoch. Every kernel launch that
+// synchronises through the area takes the next epoch.
 struct FusedSync {
-    unsigned long long *slots = nullptr;  // 64 slots, 8 words apart, zeroed once when allocated
-    uint32_t *counter = nullptr;          // arrivals, never reset
-    unsigned long long *release = nullptr;  // 64 words, 8 words apart: (epoch << 32 | max) from the last arrival
-    uint32_t epoch = 0, target = 0;
-    uint32_t spin_limit = 1u << 20;       // polls (about a microsecond each) before a waiting workgroup gives up
+    unsigned long long *slots = nullptr;   // kGridSyncMaxBlocks words, zeroed once when allocated
+    unsigned long long *decide = nullptr;  // the decision word, zeroed once when allocated
+    uint32_t epoch = 0;
+    uint32_t spin_limit = 1u << 19;        // polling rounds (a microsecond or two each) before a waiting workgroup gives up
+    // the device-side view for a launch of `grid` workgroups; advances the epoch
+    GridSync next(uint32_t grid)
+    {
+        epoch += 1;
+        GridSync g;
+        g.slots = slots;
+        g.decide = decide;
+        g.epoch = epoch;
+        g.blocks = grid;
+        g.spin_limit = spin_limit;
+        return g;
+    }
 };
-constexpr uint32_t kFusedSpinDefault = 1u << 20;
-constexpr size_t kFusedSyncBytes = 64 * 64 + 64 + 64 * 64;
+constexpr uint32_t kFusedSpinDefault = 1u << 19;
+constexpr size_t kFusedSyncBytes = kGridSyncMaxBlocks * 8 + 64;
 hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
     float *ds_out, hipStream_t st, bool *taken);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]

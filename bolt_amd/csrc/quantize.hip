@@ -55,8 +55,12 @@ hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStr
 // ---- |max| reductions ---------------------------------------------------------------------------
 // avx512/quantize.cpp:21-68: sign bit cleared, vmaxps (a NaN never replaces the running max).
 template <int VEC>
-__global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict__ x, uint32_t n, uint32_t *ws)
+__global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict__ x, uint32_t n, uint32_t *ws,
+    const uint32_t *only_if)
 {
+    if (only_if && *only_if == 0) {
+        return;
+    }
     __shared__ int red[4];
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -92,17 +96,18 @@ __global__ __launch_bounds__(256) void absmax_f32_kernel(const float *__restrict
     ws_block_fold_max(ws, (int)__float_as_uint(m), red);
 }
 
-hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear)
+hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream_t st, bool ws_is_clear, const uint32_t *only_if)
 {
     hipError_t e = ws_is_clear ? hipSuccess : launch_fill_u32(ws, kWsWords, 0, st);
     if (e != hipSuccess || n == 0) {
         return e;
     }
-    const uint32_t blocks = grid_for(n, 16, 256, 1024);
+    // a conditional launch nearly always returns at once: a small grid keeps that cheap (the loops stride over the grid)
+    const uint32_t blocks = grid_for(n, 16, 256, only_if ? 256 : 1024);
     if (((uintptr_t)x & 15) == 0) {
-        hipLaunchKernelGGL((absmax_f32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, ws);
+        hipLaunchKernelGGL((absmax_f32_kernel<1>), dim3(blocks), dim3(256), 0, st, x, n, ws, only_if);
     } else {
-        hipLaunchKernelGGL((absmax_f32_kernel<0>), dim3(blocks), dim3(256), 0, st, x, n, ws);
+        hipLaunchKernelGGL((absmax_f32_kernel<0>), dim3(blocks), dim3(256), 0, st, x, n, ws, only_if);
     }
     return hipGetLastError();
 }
@@ -190,8 +195,11 @@ __device__ __forceinline__ float resolve_scale(float s_in, int mode, const uint3
 template <int TO_U8, int VEC, int GELU = 0>
 __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restrict__ x, uint32_t n,
     uint8_t *__restrict__ q, const uint32_t *__restrict__ ws, float s_in, const float *ds_in, int mode,
-    float *ds_out)  // ds_in may alias ds_out: the resolved scale is a fixed point of resolve_scale
+    float *ds_out, const uint32_t *only_if)  // ds_in may alias ds_out: the resolved scale is a fixed point of resolve_scale
 {
+    if (only_if && *only_if == 0) {
+        return;
+    }
     const float s = resolve_scale(ds_in ? *ds_in : s_in, mode, ws);
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     if (tid == 0 && ds_out) {
@@ -242,21 +250,21 @@ __global__ __launch_bounds__(256) void quantize_f32_kernel(const float *__restri
 }
 
 hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
-    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu)
+    const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu, const uint32_t *only_if)
 {
     const bool vec = (((uintptr_t)x | (uintptr_t)q) & 15) == 0;
-    const uint32_t blocks = grid_for(n, vec ? 16 : 1, 256, 8192);
+    const uint32_t blocks = grid_for(n, vec ? 16 : 1, 256, only_if ? 256 : 8192);
     if (gelu) {
         if (!to_u8 || !vec) {
             return hipErrorInvalidValue;  // the fused form exists for aligned u8 output only
         }
         hipLaunchKernelGGL((quantize_f32_kernel<1, 1, 1>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s_in, ds_in,
-            mode, ds_out);
+            mode, ds_out, only_if);
         return hipGetLastError();
     }
 #define BG_LAUNCH_Q(U, V)                                                                                        \
     hipLaunchKernelGGL((quantize_f32_kernel<U, V>), dim3(blocks), dim3(256), 0, st, x, n, (uint8_t *)q, ws, s_in, \
-        ds_in, mode, ds_out)
+        ds_in, mode, ds_out, only_if)
     if (to_u8) {
         if (vec) {
             BG_LAUNCH_Q(1, 1);
@@ -338,43 +346,14 @@ hipError_t launch_requant_i32(const int32_t *x, uint32_t n, void *q, int to_u8, 
 //
 // The grid is at most two workgroups of 256 threads per CU and never more than the occupancy the runtime reports
 // for the kernel, so every workgroup is running when the first one reaches the barrier; a cooperative launch would have the runtime check that, but costs more than the launches saved.
-// Sync area: 64 slots of (epoch << 32 | max bits), one per 64-byte line, folded with a 64-bit atomic max -- a
-// launch's epoch beats whatever older launches left there, so nothing is ever cleared -- an arrival counter
-// that only grows (the host hands each launch the value it reaches when all of its workgroups have arrived),
-// and 64 release words, one per line, that carry the launch's OUTCOME: (epoch << 32 | max), or
-// (epoch << 32 | 0xffffffff) when the launch is abandoned. The workgroups poll the release word of their own line
-// (one thread per workgroup, a dozen pollers per line, sleeping between polls) a bounded number of times.
-// The outcome is decided exactly once, by a compare-and-swap on release word 0: the workgroup that arrives last
-// proposes the maximum, a workgroup whose bounded wait expires proposes "abandoned"; whoever swaps first wins, copies
-// the outcome to the other 63 words, and every other workgroup -- including a loser of the swap -- acts on that one
-// outcome. So a launch either quantises everywhere with one maximum, or stores nothing anywhere and publishes a NaN
+// The grid-wide maximum goes through grid_max_sync (device_common.h): either every workgroup quantises with one
+// maximum, or -- when the bounded wait of one of them expires -- none stores anything and the kernel publishes a NaN
 // scale, on which the host runs the two-pass form: never a valid scale over partly written output.
-constexpr uint32_t kFusedAbandoned = 0xffffffffu;  // never a maximum: those are non-negative floats' bits, ints >= 0 or INT32_MIN
-
-// proposes `value` as this epoch's outcome on release word 0 and returns the outcome that stands
-__device__ __forceinline__ uint32_t fused_decide(unsigned long long *release, uint32_t epoch, uint32_t value, bool *won)
-{
-    const unsigned long long mine = ((unsigned long long)epoch << 32) | value;
-    unsigned long long cur = __hip_atomic_load(release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *won = false;
-    while ((uint32_t)(cur >> 32) != epoch) {
-        const unsigned long long seen = atomicCAS(release, cur, mine);
-        if (seen == cur) {
-            *won = true;
-            return value;
-        }
-        cur = seen;
-    }
-    return (uint32_t)cur;
-}
-
 template <int SRC_I32, int TO_U8, int PER>
 __global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restrict__ xin, uint32_t n, uint8_t *__restrict__ q,
-    unsigned long long *slots, uint32_t *counter, unsigned long long *release, uint32_t epoch, uint32_t target, float s_in,
-    float *ds_out, uint32_t spin_limit)
+    GridSync gs, float s_in, float *ds_out)
 {
-    __shared__ int red[4];
-    __shared__ int bcast[2];
+    __shared__ int sync_lds[18];
     const uint32_t n4 = n / 4;
     const uint32_t tid = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
     const v4i *x4 = (const v4i *)xin;
@@ -406,76 +385,14 @@ __global__ __launch_bounds__(256) void quantize_fused_kernel(const void *__restr
     if (!SRC_I32) {
         m = __float_as_int(mf);  // non-negative float: integer order == float order
     }
-    m = wave_reduce_max_i(m);
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane == 0) {
-        red[wave] = m;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) {
-            m = red[w] > m ? red[w] : m;
-        }
-        const unsigned long long tag = ((unsigned long long)epoch << 32) | (uint32_t)m;
-        atomicMax(slots + (blockIdx.x & 63) * 8, tag);
-        __threadfence();
-        bcast[1] = (atomicAdd(counter, 1u) + 1u == target) ? 2 : 1;  // 2: this workgroup arrived last
-    }
-    __syncthreads();
-    if (bcast[1] == 2) {
-        if (wave == 0) {  // every fold is complete: take the maximum and propose it as the outcome
-            __threadfence();
-            const unsigned long long t = __hip_atomic_load(slots + lane * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            int v = ((uint32_t)(t >> 32) == epoch) ? (int)(uint32_t)t : 0;
-            v = wave_reduce_max_i(v);
-            uint32_t outcome = 0;
-            bool won = false;
-            if (lane == 0) {
-                outcome = fused_decide(release, epoch, (uint32_t)v, &won);
-            }
-            outcome = (uint32_t)__shfl((int)outcome, 0, 64);
-            won = __shfl((int)won, 0, 64) != 0;
-            if (won && lane != 0) {
-                __hip_atomic_store(release + lane * 8, ((unsigned long long)epoch << 32) | outcome, __ATOMIC_RELAXED,
-                    __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (lane == 0) {
-                bcast[0] = (int)outcome;
-            }
-        }
-    } else if (threadIdx.x == 0) {
-        uint32_t spins = 0;
-        unsigned long long t;
-        uint32_t outcome;
-        for (;;) {
-            t = __hip_atomic_load(release + (blockIdx.x & 63) * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((uint32_t)(t >> 32) == epoch) {
-                outcome = (uint32_t)t;
-                break;
-            }
-            if (++spins > spin_limit) {  // give up: propose "abandoned", unless the outcome has been decided meanwhile
-                bool won = false;
-                outcome = fused_decide(release, epoch, kFusedAbandoned, &won);
-                if (won) {
-                    for (uint32_t k = 1; k < 64; ++k) {
-                        __hip_atomic_store(release + k * 8, ((unsigned long long)epoch << 32) | kFusedAbandoned, __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                }
-                break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-        }
-        bcast[0] = (int)outcome;
-    }
-    __syncthreads();
-    if ((uint32_t)bcast[0] == kFusedAbandoned) {  // the same for every workgroup of the launch: nothing is stored
+    const uint32_t outcome = grid_max_sync(gs, m, sync_lds);
+    if (outcome == kGridAbandoned) {  // the same for every workgroup of the launch: nothing is stored
         if (tid == 0 && ds_out) {
             *ds_out = __int_as_float(0x7fc00000);
         }
         return;
     }
-    const int gmax = bcast[0];
+    const int gmax = (int)outcome;
     float s, published;
     if (SRC_I32) {  // avx512/quantize.cpp:315-416 with scale[0] < 0: r = 127 / max, returned scale = scale[1] * r
         s = (gmax == 0) ? 1.0f : 127.0f / (float)gmax;
@@ -521,6 +438,7 @@ static uint32_t fused_max_grid()
             cached = 0;
         } else {
             cached = cus * (per_cu >= 2 ? 2 : per_cu);
+            cached = cached > (int)kGridSyncMaxBlocks ? (int)kGridSyncMaxBlocks : cached;
         }
     }
     return (uint32_t)cached;
@@ -536,14 +454,11 @@ static hipError_t launch_fused(const void *x, uint32_t n, void *q, FusedSync &fs
     if (grid > fused_max_grid<SRC_I32, TO_U8, PER>()) {
         return hipSuccess;  // *taken stays false
     }
-    fs.epoch += 1;
-    fs.target += grid;
-    hipLaunchKernelGGL((quantize_fused_kernel<SRC_I32, TO_U8, PER>), dim3(grid), dim3(256), 0, st, x, n, (uint8_t *)q, fs.slots,
-        fs.counter, fs.release, fs.epoch, fs.target, s_in, ds_out, fs.spin_limit);
+    const GridSync gs = fs.next(grid);
+    hipLaunchKernelGGL((quantize_fused_kernel<SRC_I32, TO_U8, PER>), dim3(grid), dim3(256), 0, st, x, n, (uint8_t *)q, gs, s_in,
+        ds_out);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
-        fs.epoch -= 1;  // nothing ran: the counter must not be waited for
-        fs.target -= grid;
         return e;
     }
     *taken = true;

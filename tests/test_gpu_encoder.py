@@ -133,10 +133,34 @@ def test_encoder_layer_bert_base(torch_mod, oracle):
     P = make_params(rng, hidden, ffn, with_bias=False)
     x = rng.standard_normal((batch * seq, hidden)).astype(np.float32)
     layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
-    got = layer(dev(torch, x))
-    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
-    got = got.cpu().numpy()
+    L = capi.lib()
+    dx = dev(torch, x)
+    # separate kernels first: that form keeps every fp32 intermediate for the stage-wise checks below
+    capi.check(L.bolt_gfx950_set_option(b"encoder_fused", 0), "set_option")
+    try:
+        got = layer(dx)
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"encoder_fused", 1), "set_option")
     mid = {k: v.cpu().numpy() for k, v in layer.intermediates().items()}
+    # the default form (FullyConnected + GELU + quantisation in one launch) does the same arithmetic element for
+    # element: the layer output must be the same bytes -- also when its grid-wide wait is forced to give up from the
+    # host (a bound of one poll), which sends it through its two-pass fallback
+    fused = layer(dx)
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    assert torch.equal(fused, got), "fused FullyConnected + GELU + quantise differs from the separate kernels"
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 1), "set_option")
+    try:
+        for rep in range(3):
+            forced = layer(dx)
+            capi.check(L.bolt_gfx950_synchronize(), "sync")
+            assert torch.equal(forced, got), "fallback of the fused form differs (repetition %d)" % rep
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 0), "set_option")
+    again = layer(dx)
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    assert torch.equal(again, got)
+    got = got.cpu().numpy()
 
     def same_bits(a, b):
         return np.array_equal(a.view(np.int32), b.view(np.int32))
@@ -186,3 +210,24 @@ def test_encoder_errors(torch_mod):
     n = capi.C.c_size_t(0)
     assert L.bolt_gfx950_encoder_layer_int8_workspace_bytes(None, capi.C.byref(n)) == capi.NULL_POINTER
     assert L.bolt_gfx950_encoder_layer_int8_workspace_bytes(capi.C.byref(spec), capi.C.byref(n)) == capi.NULL_POINTER
+
+
+def test_encoder_layer_fused_ffn_other_shape(torch_mod):
+    """Another shape that takes the one-launch FullyConnected + GELU + quantise (4096 tokens x FFN 2048 = 128 tiles of
+    256 x 256, biases present): same bytes as the separate kernels."""
+    torch = torch_mod
+    batch, seq, hidden, heads, ffn = 16, 256, 256, 4, 2048
+    rng = np.random.default_rng(77)
+    P = make_params(rng, hidden, ffn, with_bias=True)
+    x = dev(torch, rng.standard_normal((batch * seq, hidden)).astype(np.float32))
+    layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_set_option(b"encoder_fused", 0), "set_option")
+    try:
+        plain = layer(x).clone()
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"encoder_fused", 1), "set_option")
+    fused = layer(x)
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    assert torch.equal(fused, plain)
