@@ -138,6 +138,9 @@ int g_bnn_mfma = 2;
 // int8 convolution through the filter-panel kernel: gather from the caller's tensor in place for int32 / fp32 results
 // (1, default) or for every result type (2); 0 = always re-lay the input as a padded s8 image first
 int g_conv_direct = 1;
+// u8 convolution through the filter-panel kernel: 1 = one pass where every workgroup fits the device at once (the
+// tensor-wide maximum is agreed on with the accumulators in registers; default), 0 = always two passes
+int g_conv_onepass = 1;
 // LSTM cell: from this many batch rows on, a weight that carries the GEMM packing goes through the matrix cores
 int g_lstm_gemm_rows = 4;
 // dynamic quantisation through the public entry points: 1 = one launch that reads the tensor once where
@@ -185,7 +188,7 @@ EE ensure_init()
             return fail(ALLOC_FAILED, "hipMalloc(quantiser sync area)", e);
         }
         c.fsync.slots = (unsigned long long *)p;
-        c.fsync.decide = (unsigned long long *)((uint8_t *)p + kGridSyncMaxBlocks * 8);
+        c.fsync.release = (unsigned long long *)((uint8_t *)p + kGridSyncMaxBlocks * 8);
     }
     if (!c.hscale) {
         e = hipHostMalloc((void **)&c.hscale, 64, hipHostMallocMapped);
@@ -520,6 +523,13 @@ EE bolt_gfx950_set_option(const char *name, int value)
             return NOT_MATCH;
         }
         g_conv_direct = value;
+        return SUCCESS;
+    }
+    if (strcmp(name, "conv_onepass") == 0) {
+        if (value != 0 && value != 1) {
+            return NOT_MATCH;
+        }
+        g_conv_onepass = value;
         return SUCCESS;
     }
     if (strcmp(name, "conv_panel") == 0) {
@@ -1644,8 +1654,14 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // in-place gather costs the kernel about as much as half a padding pass (bounds tests, and two 8-byte loads per
     // fragment from NCHWC8), so by default (1) it is taken where the convolution runs once -- int32 and fp32
     // results -- and not for u8 results, whose two passes share one padded image; 2 takes it always.
-    const bool direct = g_conv_direct && (g_conv_direct == 2 || odt != DT_U8_Q) && conv_panel_ok(s.oc, s.Kp) &&
-        s.ic % 16 == 0 && (((uintptr_t)input) & 15) == 0;
+    const bool gather_ok = conv_panel_ok(s.oc, s.Kp) && s.ic % 16 == 0 && (((uintptr_t)input) & 15) == 0;
+    // u8 result in ONE pass of the filter-panel kernel when all its workgroups are resident at once: they agree on
+    // max|acc| with the accumulators still in registers and requantise from there. The convolution then runs once,
+    // so it also gathers from the caller's tensor in place where it can.
+    const uint32_t M_pix = s.n * s.oh * s.ow;
+    bool onepass = odt == DT_U8_Q && g_conv_onepass && conv_panel_ok(s.oc, s.Kp) &&
+        conv_panel_grid(M_pix) <= conv_onepass_max_grid(s.Kp);
+    const bool direct = g_conv_direct && (g_conv_direct == 2 || odt != DT_U8_Q || onepass) && gather_ok;
     if (!direct) {
         HIP_TRY(launch_conv_pad((const uint8_t *)input, s.n, s.ic, s.ih, s.iw, idf == DF_NCHWC16 ? 16 : 8, s.pt, s.pb, s.pl,
             s.pr, (int8_t *)t, c.stream, odt == DT_U8_Q ? c.ws : nullptr));  // u8 results: also clears the max slots
@@ -1708,9 +1724,29 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     // folding max|acc| into the scratch slots without storing anything, once writing u8 with the scale
     // that maximum gives. The arithmetic per element is the same; the int32 tensor (4 bytes per output,
     // written and read back) never exists, which is worth more than the repeated matrix work.
+    if (onepass) {
+        g.C = output;
+        g.epi.mode = EPI_U8;
+        g.conv.scaleO = scaleO;
+        g.conv.dscale_out = c.hscale_dev;
+        g.sync = c.fsync.next(conv_panel_grid(M_pix));
+        arm_scale(c);
+        HIP_TRY(launch_conv_u8s8(g, c.stream));
+        bool gave_up = false;
+        EE te = take_scale(c, &scale[1], &gave_up);
+        if (te != SUCCESS || !gave_up) {
+            return te;
+        }
+        // the bounded wait of the one-pass form expired (the CUs were held by other work): nothing was stored;
+        // the two passes below redo the convolution
+        g_fused_fallbacks.fetch_add(1);
+        memset(&g.sync, 0, sizeof(g.sync));
+        g.epi.mode = EPI_I32;
+        g.conv.dscale_out = nullptr;
+    }
     g.C = nullptr;
     g.conv.absmax = c.ws;
-    if (direct) {  // otherwise the padding kernel has cleared the slots
+    if (direct || onepass) {  // otherwise the padding kernel has cleared the slots
         HIP_TRY(launch_fill_u32(c.ws, kWsWords, 0, c.stream));
     }
     HIP_TRY(launch_conv_u8s8(g, c.stream));

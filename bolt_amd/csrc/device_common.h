@@ -244,29 +244,48 @@ __device__ __forceinline__ int ws_read_max(const uint32_t *ws)
 // agree on one tensor-wide maximum half way through, with their partial results still in registers.
 //
 // Sync area (device memory, zeroed once when allocated, never cleared afterwards): one 64-bit slot per workgroup
-// (at most kGridSyncMaxBlocks) and one 64-bit decision word. A launch carries an epoch that grows with every launch.
-// Every workgroup stores (epoch << 32 | its maximum) into its own slot -- one store, nothing to wait for -- and then
-// its first wave polls ALL slots of the grid (64 per load instruction) until each carries this launch's epoch; the
-// maximum over them is the same in every workgroup. That is one store and one or two rounds of loads end to end;
-// a counter that the last arrival turns into a release word costs five dependent trips to memory instead.
+// (at most kGridSyncMaxBlocks) and 64 release words, one per 64-byte line. A launch carries an epoch that grows
+// with every launch. Every workgroup stores (epoch << 32 | its maximum) into its own slot -- one store, no atomic
+// read-modify-write, nothing to wait for. Workgroup 0 collects: its first wave polls all slots (64 per load
+// instruction) until each carries this launch's epoch, takes the maximum and publishes (epoch << 32 | max) in the
+// release words; the others poll the release word of their own line. Traffic grows with the number of workgroups,
+// not with its square (every workgroup polling every slot cost 5-10 us at 400-1000 workgroups), and no address
+// takes more than one store per workgroup (an arrival counter serialises at about 10 ns per workgroup).
 //
-// The wait is bounded, and its outcome is decided exactly once through the decision word:
-//   a workgroup that has seen every slot proposes (epoch, COMMITTED) with a compare-and-swap, unless it already
-//   reads that; a workgroup whose bound expires proposes (epoch, ABANDONED). Whoever swaps first wins and every
-//   workgroup acts on the one outcome: after COMMITTED all slots are known to be present (a workgroup whose bound
-//   expired just then simply reads them), after ABANDONED nobody uses the maximum.
-// So all workgroups of a launch see the same maximum, or all see "abandoned" (kGridAbandoned).
+// The waits are bounded, and the outcome is decided exactly once, by a compare-and-swap on release word 0: the
+// collector proposes the maximum, a workgroup whose bound expires (the collector included) proposes "abandoned"
+// (epoch << 32 | 0xffffffff); whoever swaps first wins and copies the outcome to the other 63 words; every other
+// workgroup -- a loser of the swap too -- acts on that one outcome. So all workgroups of a launch see the same
+// maximum, or all see "abandoned" (kGridAbandoned).
 // Launches that share a sync area must be ordered on one stream.
 constexpr uint32_t kGridSyncMaxBlocks = 1024;
 struct GridSync {
-    unsigned long long *slots = nullptr;   // kGridSyncMaxBlocks words
-    unsigned long long *decide = nullptr;  // one word (on a cache line of its own)
+    unsigned long long *slots = nullptr;    // kGridSyncMaxBlocks words
+    unsigned long long *release = nullptr;  // 64 words, 8 words apart
     uint32_t epoch = 0;        // this launch's tag
     uint32_t blocks = 0;       // workgroups in the launch (gridDim.x, <= kGridSyncMaxBlocks)
-    uint32_t spin_limit = 0;   // polling rounds (a microsecond or two each) before a waiting workgroup gives up
+    uint32_t spin_limit = 0;   // polling rounds (about a microsecond each) before a waiting workgroup gives up
 };
 constexpr uint32_t kGridAbandoned = 0xffffffffu;  // never a maximum: those are non-negative floats' bits, ints >= 0 or INT32_MIN
-constexpr uint32_t kGridCommitted = 1u, kGridGaveUp = 2u;
+
+// proposes `value` as this epoch's outcome on release word 0, copies it to the other words if it stands, and returns
+// the outcome that stands. Called by lane 0 of a wave.
+__device__ __forceinline__ uint32_t grid_sync_decide(unsigned long long *release, uint32_t epoch, uint32_t value)
+{
+    const unsigned long long mine = ((unsigned long long)epoch << 32) | value;
+    unsigned long long cur = __hip_atomic_load(release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while ((uint32_t)(cur >> 32) != epoch) {
+        const unsigned long long seen = atomicCAS(release, cur, mine);
+        if (seen == cur) {
+            for (uint32_t k = 1; k < 64; ++k) {
+                __hip_atomic_store(release + k * 8, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return value;
+        }
+        cur = seen;
+    }
+    return (uint32_t)cur;
+}
 
 // Called by every thread of every workgroup of the launch (uniform control flow) with its own candidate `m`
 // (values whose signed-integer order is the wanted order: non-negative floats' bits or ints). `lds`: 18 ints of
@@ -288,60 +307,47 @@ __device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int
             __hip_atomic_store(gs.slots + blockIdx.x, tag | (uint32_t)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         uint32_t spins = 0, outcome = kGridAbandoned;
-        bool committed = false;  // the decision is known to be COMMITTED: every slot is (about to be) visible
-        for (;;) {
-            bool ok = true;
-            int v = (int)0x80000000;
-            for (uint32_t b = lane; b < gs.blocks; b += 64) {
-                const unsigned long long t = __hip_atomic_load(gs.slots + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = ok && ((uint32_t)(t >> 32) == gs.epoch);
-                const int tv = (int)(uint32_t)t;
-                v = tv > v ? tv : v;
-            }
-            unsigned long long d = __hip_atomic_load(gs.decide, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const bool all = __all(ok);
-            uint32_t state = ((uint32_t)(d >> 32) == gs.epoch) ? (uint32_t)d : 0u;
-            if (state == kGridGaveUp) {
-                break;
-            }
-            if (all) {
-                if (state != kGridCommitted && !committed) {
-                    if (lane == 0) {  // propose COMMITTED; a different epoch-tagged value in the word means someone decided first
-                        for (;;) {
-                            const unsigned long long seen = atomicCAS(gs.decide, d, tag | kGridCommitted);
-                            if (seen == d || (uint32_t)(seen >> 32) == gs.epoch) {
-                                state = (seen == d) ? kGridCommitted : (uint32_t)seen;
-                                break;
-                            }
-                            d = seen;
-                        }
-                    }
-                    state = (uint32_t)__shfl((int)state, 0, 64);
-                }
-                if (state != kGridGaveUp) {
-                    outcome = (uint32_t)wave_reduce_max_i(v);
-                }
-                break;
-            }
-            committed = committed || state == kGridCommitted;
-            if (!committed && ++spins > gs.spin_limit) {
-                if (lane == 0) {  // give up: propose ABANDONED, unless the outcome has been decided meanwhile
-                    for (;;) {
-                        const unsigned long long seen = atomicCAS(gs.decide, d, tag | kGridGaveUp);
-                        if (seen == d || (uint32_t)(seen >> 32) == gs.epoch) {
-                            state = (seen == d) ? kGridGaveUp : (uint32_t)seen;
-                            break;
-                        }
-                        d = seen;
+        if (blockIdx.x == 0) {  // the collector
+            for (;;) {
+                bool ok = true;
+                int v = mine;
+                for (uint32_t b = lane; b < gs.blocks; b += 64) {
+                    if (b != 0) {  // its own slot needs no trip to memory
+                        const unsigned long long t = __hip_atomic_load(gs.slots + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        ok = ok && ((uint32_t)(t >> 32) == gs.epoch);
+                        const int tv = (int)(uint32_t)t;
+                        v = tv > v ? tv : v;
                     }
                 }
-                state = (uint32_t)__shfl((int)state, 0, 64);
-                if (state == kGridGaveUp) {
+                if (__all(ok)) {
+                    v = wave_reduce_max_i(v);
+                    if (lane == 0) {
+                        outcome = grid_sync_decide(gs.release, gs.epoch, (uint32_t)v);
+                    }
                     break;
                 }
-                committed = true;  // someone saw every slot just now: read them
+                if (++spins > gs.spin_limit) {
+                    if (lane == 0) {
+                        outcome = grid_sync_decide(gs.release, gs.epoch, kGridAbandoned);
+                    }
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
             }
-            __builtin_amdgcn_s_sleep(4);
+        } else if (lane == 0) {
+            for (;;) {
+                const unsigned long long t =
+                    __hip_atomic_load(gs.release + (blockIdx.x & 63) * 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((uint32_t)(t >> 32) == gs.epoch) {
+                    outcome = (uint32_t)t;
+                    break;
+                }
+                if (++spins > gs.spin_limit) {  // give up, unless the outcome has been decided meanwhile
+                    outcome = grid_sync_decide(gs.release, gs.epoch, kGridAbandoned);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
         }
         if (lane == 0) {
             lds[17] = (int)outcome;

@@ -179,7 +179,6 @@ template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CI
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
-    (void)smem;
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const bool use_cin = (CIN == 2) ? (!CONV && a.add_cin && MODE != EPI_U8) : (CIN == 1);
@@ -189,9 +188,12 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     float factor = 0.0f, sI = 0.0f;
     if (CONV && MODE == EPI_U8) {
         // tensor-wide dynamic requantisation (avx512/quantize.cpp:364-416 after the abs-max of :70-119)
-        const int mx = ws_read_max(a.conv.absmax);
+        int mx = 0;
+        if (!a.sync.slots) {
+            mx = ws_read_max(a.conv.absmax);
+        }
         factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
-        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out && !a.sync.slots) {
             *a.conv.dscale_out = a.conv.scaleO * factor;
         }
     } else if (MODE == EPI_F32 || MODE == EPI_U8) {
@@ -232,6 +234,39 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             const uint32_t xc = a.conv.out_c, blk = n / xc;
             cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
             cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+        }
+    }
+
+    if (CONV && MODE == EPI_U8 && a.sync.slots) {
+        // one pass: the maximum is agreed on by all workgroups of the launch while the accumulators are still in
+        // registers (smem: 18 ints of LDS that no wave of the workgroup is still reading tiles from)
+        int lm = 0;
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (n + c < a.N) {
+#pragma unroll
+                    for (int x = 0; x < TM; ++x) {
+                        int t = (int)((uint32_t)acc[x][y][c] + base[y][c]);
+                        t = (a.conv.relu && t < 0) ? 0 : t;
+                        const int av = (t == (int)0x80000000) ? t : (t < 0 ? -t : t);
+                        lm = av > lm ? av : lm;
+                    }
+                }
+            }
+        }
+        const uint32_t outcome = grid_max_sync(a.sync, lm, (int *)smem);
+        if (outcome == kGridAbandoned) {  // nothing is stored; the host sees a NaN scale and runs the two passes
+            if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+                *a.conv.dscale_out = __int_as_float(0x7fc00000);
+            }
+            return;
+        }
+        factor = ((int)outcome == 0) ? 1.0f : 127.0f / (float)(int)outcome;
+        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+            *a.conv.dscale_out = a.conv.scaleO * factor;
         }
     }
 
@@ -777,7 +812,7 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_tiled_kernel(GemmArg
 // the same factor for its own arithmetic) does not store it a second time.
 __device__ __forceinline__ void conv_publish_scale(GemmArgs &a, uint32_t wave)
 {
-    if (a.epi.mode == EPI_U8 && a.conv.dscale_out) {
+    if (a.epi.mode == EPI_U8 && a.conv.dscale_out && !a.sync.slots) {
         if (blockIdx.x == 0 && wave == 0) {
             const int mx = ws_read_max(a.conv.absmax);
             const float factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
@@ -1338,6 +1373,7 @@ template <int TM, bool DIRECT>
 __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ int sync_lds[18];  // the one-pass u8 form's grid-wide maximum (the waves read the panel at their own pace)
     constexpr int P = 3;  // K tiles of A in flight per wave
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1464,7 +1500,7 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
             }
         }
     }
-    epilogue_panel<4, 1, TM, 4, true>(a, acc, nullptr, lane, wave, m0, 0u, 0);
+    epilogue_panel<4, 1, TM, 4, true>(a, acc, (uint8_t *)sync_lds, lane, wave, m0, 0u, 0);
 }
 
 // Skinny kernel for few rows (FullyConnected at small batch: M <= 64 per block, any N, K % 64 == 0).
@@ -1617,6 +1653,33 @@ bool conv_panel_ok(uint32_t N, uint32_t K)
     return N <= 64 && K % 64 == 0 && K <= 1024 && g_conv_panel != 0;
 }
 
+// Workgroups of the filter-panel kernel that are resident at once: two per CU where the kernel's registers and its
+// K x 64 bytes of LDS allow (0 if the device cannot be asked), never more than a grid sync spans.
+uint32_t conv_onepass_max_grid(uint32_t K)
+{
+    static int cus = -1, per_cu_regs = 0;
+    if (cus < 0) {
+        int dev = 0, n = 0, occ = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, conv_u8s8_panel_kernel<4, true>, 256, 65536) == hipSuccess) {
+            cus = n;
+            per_cu_regs = occ;  // with the largest panel (64 KB): a lower bound for smaller ones
+        } else {
+            cus = 0;
+        }
+    }
+    (void)K;
+    const uint32_t per_cu = per_cu_regs >= 2 ? 2u : (uint32_t)per_cu_regs;
+    const uint32_t g = (uint32_t)cus * per_cu;
+    return g > kGridSyncMaxBlocks ? kGridSyncMaxBlocks : g;
+}
+
+// the grid launch_conv_u8s8 gives the filter-panel kernel for M output pixels
+uint32_t conv_panel_grid(uint32_t M)
+{
+    return (g_conv_panel == 2) ? (M + 127) / 128 : (M + 255) / 256;
+}
+
 // Implicit-GEMM convolution: same pipeline, A rows are output pixels gathered from the padded image.
 hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
 {
@@ -1639,16 +1702,20 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
         }
         const uint32_t lds = a.K * 64;
         const bool direct = a.conv.in_c != 0;
+        const uint32_t grid = (g_conv_panel == 2) ? (a.M + 127) / 128 : (a.M + 255) / 256;
+        if (a.sync.slots && (a.sync.blocks != grid || grid > conv_onepass_max_grid(a.K))) {
+            return hipErrorInvalidValue;  // the one-pass form needs every workgroup resident at once
+        }
         if (g_conv_panel == 2) {
             if (direct) {
-                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, true>), dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, true>), dim3(grid), dim3(256), lds, st, a);
             } else {
-                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, false>), dim3((a.M + 127) / 128), dim3(256), lds, st, a);
+                hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, false>), dim3(grid), dim3(256), lds, st, a);
             }
         } else if (direct) {
-            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, true>), dim3((a.M + 255) / 256), dim3(256), lds, st, a);
+            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, true>), dim3(grid), dim3(256), lds, st, a);
         } else {
-            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, false>), dim3((a.M + 255) / 256), dim3(256), lds, st, a);
+            hipLaunchKernelGGL((conv_u8s8_panel_kernel<4, false>), dim3(grid), dim3(256), lds, st, a);
         }
         return hipGetLastError();
     }

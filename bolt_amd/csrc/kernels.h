@@ -80,8 +80,9 @@ struct GemmArgs {
     int fp4 = 0;             // convolution only: operand bytes are pairs of E2M1 values (1-bit convolution), K counts bytes
     Epilogue epi;
     ConvGeom conv;       // used by launch_conv_u8s8 only
-    // EPI_U8_GELU_DYN only (256 x 256 tiles, M and N multiples of 256, every workgroup resident at once):
-    GridSync sync;                 // from FusedSync::next(number of tiles)
+    // EPI_U8_GELU_DYN (256 x 256 tiles, M and N multiples of 256), and the filter-panel convolution with a u8 result in
+    // ONE pass (launch_conv_u8s8, conv.absmax null): every workgroup resident at once
+    GridSync sync;                 // from FusedSync::next(number of workgroups)
     float *dscale_out = nullptr;   // receives the scale the u8 result was quantised with
     uint32_t *status = nullptr;    // receives 0; or 1 when the grid-wide wait was abandoned: then nothing was quantised and
     float *C32 = nullptr;          //   the activated fp32 values y are in C32 [M][N] for a two-pass quantisation to pick up
@@ -95,6 +96,8 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st);
 bool conv_fp4_ok(uint32_t M, uint32_t N);
 // whether launch_conv_u8s8 would run the filter-panel kernel for this shape (the one that can gather from the caller's tensor)
 bool conv_panel_ok(uint32_t N, uint32_t K);  // whether launch_conv_u8s8 has an fp4 kernel for this shape
+uint32_t conv_onepass_max_grid(uint32_t K);  // most workgroups of the filter-panel kernel that a one-pass u8 convolution may span
+uint32_t conv_panel_grid(uint32_t M);        // the grid the filter-panel kernel gets for M output pixels
 void conv_force_panel(int v);  // 0: shared-pipeline kernel only; 2 / 4: panel kernel with 32 / 64 pixels per wave
 // tuning / test hook: -1 = shape heuristic, 0 = general kernel, 1 = 256x256 tiles, 2 = 128x128 tiles
 void gemm_force_tile(int tile);
@@ -184,7 +187,7 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t st);
 // synchronises through the area takes the next epoch.
 struct FusedSync {
     unsigned long long *slots = nullptr;   // kGridSyncMaxBlocks words, zeroed once when allocated
-    unsigned long long *decide = nullptr;  // the decision word, zeroed once when allocated
+    unsigned long long *release = nullptr; // 64 release words, 8 words apart, zeroed once when allocated
     uint32_t epoch = 0;
     uint32_t spin_limit = 1u << 19;        // polling rounds (a microsecond or two each) before a waiting workgroup gives up
     // the device-side view for a launch of `grid` workgroups; advances the epoch
@@ -193,7 +196,7 @@ struct FusedSync {
         epoch += 1;
         GridSync g;
         g.slots = slots;
-        g.decide = decide;
+        g.release = release;
         g.epoch = epoch;
         g.blocks = grid;
         g.spin_limit = spin_limit;
@@ -201,7 +204,7 @@ struct FusedSync {
     }
 };
 constexpr uint32_t kFusedSpinDefault = 1u << 19;
-constexpr size_t kFusedSyncBytes = kGridSyncMaxBlocks * 8 + 64;
+constexpr size_t kFusedSyncBytes = kGridSyncMaxBlocks * 8 + 64 * 64;
 hipError_t launch_quantize_fused(const void *x, uint32_t n, void *q, int src_i32, int to_u8, FusedSync &fs, float s_in,
     float *ds_out, hipStream_t st, bool *taken);
 hipError_t launch_mul_scalars(float *out, const float *a, const float *b, hipStream_t st);  // out[0] = a[0] * b[0]

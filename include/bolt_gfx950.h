@@ -64,8 +64,12 @@ const char *bolt_gfx950_last_error(void);
  * matrix cores with one byte per value; 0 on the vector ALU (xor + popcount).
  * "lstm_gemm_rows" (>= 1, default 4): the LSTM cell sends calls with at least this many batch rows through the
  * matrix cores when its weight carries the GEMM packing (rnn_transform_filter_gfx950). Every variant
- * returns the same bytes. "quantize_fused_spin" (calling thread only): polls of the one-launch quantiser's bounded wait
- * before a workgroup gives up and the call falls back to two passes (0 = default, about a second; tests use 1). */
+ * returns the same bytes. "conv_onepass" (default 1): a u8 convolution through the filter-panel kernel runs once, its
+ * workgroups agreeing on the tensor-wide maximum with the accumulators in registers, where all of them fit the device
+ * at once; 0 = two passes (maximum only, then the stores). "encoder_fused" (default 1): the encoder layer's
+ * FullyConnected in front of the GELU also applies the GELU and quantises, in one launch; 0 = separate kernels, which
+ * keep the fp32 intermediate. "quantize_fused_spin" (calling thread only): polling rounds of the bounded grid-wide wait (one-launch quantiser,
+ * one-pass convolution, fused encoder FullyConnected) before a workgroup gives up and the call falls back to two passes (0 = default, about a second; tests use 1). */
 EE bolt_gfx950_set_option(const char *name, int value);
 /* Event counters for tests and monitoring: "quantize_fused_fallbacks" = dynamic quantisations whose one-launch form
  * gave up waiting for its grid (the CUs were held by other work) and were redone in two passes. NOT_FOUND otherwise. */

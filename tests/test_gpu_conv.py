@@ -61,15 +61,19 @@ def test_conv_int8(torch_mod, oracle, co, device_mode, case, relu):
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (case, odt, out_c)
 
 
+@pytest.mark.parametrize("onepass", [1, 0], ids=["one_pass", "two_pass"])
 @pytest.mark.parametrize("panel,direct", [(0, 0), (2, 0), (2, 2), (4, 0), (4, 2)])
-def test_conv_int8_every_kernel(torch_mod, oracle, co, panel, direct):
+def test_conv_int8_every_kernel(torch_mod, oracle, co, panel, direct, onepass):
     """Convolutions with up to 64 output channels and K <= 1024 have three kernels to choose from: the shared
     LDS pipeline (0) and the filter-panel kernel with 32 (2) or 64 (4) pixels per wave; the filter-panel kernel
     either reads the padded s8 image (direct = 0) or, when the channel count is a multiple of 16, gathers from
     the caller's u8 tensor in place (direct = 2: for every result type). Each is forced in turn on shapes with ragged pixel counts,
-    channel tails, strides, a 5 x 5 filter, no padding, and a K that is padded up to 64."""
+    channel tails, strides, a 5 x 5 filter, no padding, and a K that is padded up to 64. u8 results through the
+    filter-panel kernel come in one pass (the workgroups agree on the tensor-wide maximum with their accumulators in
+    registers; default) or two (maximum only, then the stores)."""
     L = capi.lib()
     try:
+        capi.check(L.bolt_gfx950_set_option(b"conv_onepass", onepass), "set_option")
         capi.check(L.bolt_gfx950_set_option(b"conv_panel", panel), "set_option")
         capi.check(L.bolt_gfx950_set_option(b"conv_direct", direct), "set_option")
         for case in [(2, 24, 6, 5, 24, 5, 5, 1, 2), (3, 16, 10, 9, 40, 3, 3, 1, 1), (1, 64, 56, 56, 64, 3, 3, 1, 1),
@@ -88,6 +92,46 @@ def test_conv_int8_every_kernel(torch_mod, oracle, co, panel, direct):
     finally:
         capi.check(L.bolt_gfx950_set_option(b"conv_panel", 4), "set_option")
         capi.check(L.bolt_gfx950_set_option(b"conv_direct", 1), "set_option")
+        capi.check(L.bolt_gfx950_set_option(b"conv_onepass", 1), "set_option")
+
+
+def test_conv_u8_one_pass_falls_back_when_its_wait_gives_up(torch_mod, oracle, co):
+    """The one-pass u8 convolution waits a bounded number of polls for all its workgroups. With the bound forced to one
+    poll from the host, launches of more than a few workgroups give up: nothing is stored, the kernel publishes a NaN
+    scale and exits normally, and the call redoes the convolution in two passes. Same bytes and scale either way."""
+    import ctypes as C
+    L = capi.lib()
+    before = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(before)), "counter")
+    cases = [(8, 64, 56, 56, 64, 3, 3, 1, 1), (3, 16, 10, 9, 40, 3, 3, 1, 1), (5, 32, 13, 13, 64, 1, 1, 1, 0)]
+    want = {}
+    for case in cases:
+        n, ic, ih, iw, oc, fh, fw, stride, pad = case
+        xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, sum(case))
+        d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, True, DT_U8_Q, 16)
+        want[case] = (xq, sI, W, sF, bias) + co.conv(d, xq, W, bias, [sI, -1.0, sF])
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 1), "set_option")
+    try:
+        for rep in range(3):
+            for case in cases:
+                print("conv one-pass fallback", rep, case, flush=True)
+                xq, sI, W, sF, bias, out, ws = want[case]
+                sc = [sI, -1.0, sF]
+                got = run_conv(torch_mod, True, xq, DF_NCHWC8, W, bias, sc, case, True, DT_U8_Q, DF_NCHWC16)
+                assert np.array_equal(np.array(sc, np.float32), ws) and np.array_equal(got, out), (rep, case)
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 0), "set_option")
+    after = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(after)), "counter")
+    assert after.value > before.value, "no launch gave up: the test did not exercise the fallback"
+    for case in cases:      # and with the default bound the one-pass form completes
+        xq, sI, W, sF, bias, out, ws = want[case]
+        sc = [sI, -1.0, sF]
+        got = run_conv(torch_mod, True, xq, DF_NCHWC8, W, bias, sc, case, True, DT_U8_Q, DF_NCHWC16)
+        assert np.array_equal(np.array(sc, np.float32), ws) and np.array_equal(got, out), case
+    final = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(final)), "counter")
+    assert final.value == after.value
 
 
 @pytest.mark.parametrize("direct", [2, 0])
