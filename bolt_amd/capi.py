@@ -81,6 +81,7 @@ class ActivationParamSpec(C.Structure):
 assert C.sizeof(ConvolutionParamSpec) == 108 and C.sizeof(ActivationParamSpec) == 20
 ACTIVATION_NULL, ACTIVATION_RELU = 0, 1
 CONVOLUTION_ALGORITHM_POINTWISE, CONVOLUTION_ALGORITHM_DIRECT, CONVOLUTION_ALGORITHM_BNN = 0, 1, 6
+CONVOLUTION_ALGORITHM_IM2COL_GEMM, CONVOLUTION_ALGORITHM_GROUP_DECONV, CONVOLUTION_ALGORITHM_NULL = 2, 8, 9
 
 
 def conv_param_spec(oc, fh, fw, stride, pad, dilation=1, group=1):
@@ -192,6 +193,17 @@ SIGNATURES = {
                                                              C.c_int, _u32p, C.c_int]),
     "convolution_gfx950": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, C.c_int, TensorDesc,
                                      _vp, _u32, _vp, TensorDesc, _vp, _f32p, ActivationParamSpec, C.c_int]),
+    "deconvolution_infer_output_size_gfx950": (C.c_int, [TensorDesc, TensorDesc, ConvolutionParamSpec, _TDp, C.c_int,
+                                                         C.c_int]),
+    "deconvolution_infer_forward_algorithm_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, ConvolutionParamSpec,
+                                                               C.c_int, C.POINTER(C.c_int), C.c_int, C.c_int]),
+    "deconvolution_transform_filter_bytes_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, C.c_int, _u32p, C.c_int]),
+    "deconvolution_transform_filter_gfx950": (C.c_int, [TensorDesc, _vp, ConvolutionParamSpec, C.c_int, _TDp, _vp,
+                                                        C.c_int]),
+    "deconvolution_infer_forward_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, ConvolutionParamSpec,
+                                                               C.c_int, _u32p, C.c_int]),
+    "deconvolution_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, ConvolutionParamSpec, C.c_int, TensorDesc, _vp,
+                                       TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, ActivationParamSpec, C.c_int]),
     "convolution_transform_filter_bytes_bnn_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
     "convolution_transform_filter_bnn_gfx950": (C.c_int, [TensorDesc, _vp, C.POINTER(TensorDesc), _vp, C.c_int]),
     "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),

@@ -11,45 +11,12 @@
 #include <string>
 #include <vector>
 
-#include "../../include/bolt_gfx950.h"
-#include "kernels.h"
-#include "layout.h"
+#include "api_internal.h"
 
 using namespace bg;
+using namespace bgapi;
 
 namespace {
-struct Ctx;
-Ctx &ctx();
-}  // namespace
-
-namespace {
-
-// Everything a call needs besides its arguments. One context per calling thread: its stream, its scratch words, its
-// pinned scale word, its quantiser sync area and its staging pool, so that threads calling at the same time (each
-// with its own tensors, as CNN::clone() gives them) never share mutable state. Contexts come from a process-wide
-// pool: a thread takes one on its first call and returns it when it ends; device memory is never freed, so a
-// process that creates and ends threads does not leak one context per thread.
-struct Ctx {
-    bool ready = false;
-    hipStream_t stream = nullptr;
-    uint32_t *ws = nullptr;  // device scratch words for the two-pass reductions
-    // One pinned host word that kernels write a freshly computed scale into (the interfaces that return a
-    // scale through a host pointer read it after the stream has drained: no copy command in between), and
-    // the address the device uses for it.
-    float *hscale = nullptr, *hscale_dev = nullptr;
-    FusedSync fsync;  // sync area of the one-launch dynamic quantiser
-    uint32_t *enc_ws = nullptr;  // the encoder layer's four arrays of max slots (behind ws), kept clear between calls
-    bool enc_ws_dirty = true;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    std::string err;
-    bool reused = false;  // taken over from a thread that has ended: its last work may still be running
-    struct Buf {
-        void *p;
-        size_t bytes;
-        bool busy;
-    };
-    std::vector<Buf> pool;
-};
 
 struct CtxPool {
     std::mutex mu;
@@ -76,6 +43,10 @@ struct CtxLease {
     }
 };
 
+}  // namespace
+
+namespace bgapi {
+
 Ctx &ctx()
 {
     thread_local CtxLease lease;
@@ -95,7 +66,7 @@ Ctx &ctx()
 // counters behind bolt_gfx950_get_counter
 std::atomic<unsigned long long> g_fused_fallbacks{0};
 
-}  // namespace
+}  // namespace bgapi
 
 namespace bg {
 
@@ -116,21 +87,17 @@ void api_set_error(const char *what, hipError_t he)
 
 }  // namespace bg
 
-namespace {
+namespace bgapi {
 
-EE fail(EE code, const char *what, hipError_t he = hipSuccess)
+EE fail(EE code, const char *what, hipError_t he)
 {
     bg::api_set_error(what, he);
     return code;
 }
 
-#define HIP_TRY(expr)                                   \
-    do {                                                \
-        hipError_t e__ = (expr);                        \
-        if (e__ != hipSuccess) {                        \
-            return fail(UNKNOWN, #expr, e__);           \
-        }                                               \
-    } while (0)
+}  // namespace bgapi
+
+namespace {
 
 // 1-bit convolution: 2 = matrix cores with E2M1 operands where the shape has that kernel, else int8 (default);
 // 1 = matrix cores with int8 operands; 0 = vector-ALU xor / popcount route
@@ -149,6 +116,10 @@ int g_quantize_fused = 1;
 // encoder layer: 1 = the FullyConnected in front of the GELU also applies the GELU and quantises its result for the
 // next FullyConnected, in one launch (where the shape allows; default); 0 = separate kernels, fp32 intermediate kept
 int g_encoder_fused = 1;
+
+}  // namespace
+
+namespace bgapi {
 
 EE ensure_init()
 {
@@ -219,7 +190,7 @@ void arm_scale(Ctx &c)
     *(volatile uint32_t *)c.hscale = kScaleUnset;
 }
 
-EE take_scale(Ctx &c, float *dst, bool *gave_up = nullptr)
+EE take_scale(Ctx &c, float *dst, bool *gave_up)
 {
     volatile uint32_t *w = (volatile uint32_t *)c.hscale;
     const auto t0 = std::chrono::steady_clock::now();
@@ -247,35 +218,9 @@ EE take_scale(Ctx &c, float *dst, bool *gave_up = nullptr)
     return SUCCESS;
 }
 
-// Grow-only device staging pool for the host-pointer mode (per context, so per calling thread).
-struct Stage {
-    Ctx &c = ctx();
-    std::vector<size_t> taken;
-    ~Stage()
-    {
-        for (size_t i : taken) {
-            c.pool[i].busy = false;
-        }
-    }
-    void *get(size_t bytes)
-    {
-        bytes = std::max<size_t>(bytes, 256);
-        for (size_t i = 0; i < c.pool.size(); ++i) {
-            if (!c.pool[i].busy && c.pool[i].bytes >= bytes) {
-                c.pool[i].busy = true;
-                taken.push_back(i);
-                return c.pool[i].p;
-            }
-        }
-        void *p = nullptr;
-        if (hipMalloc(&p, bytes) != hipSuccess) {
-            return nullptr;
-        }
-        c.pool.push_back({p, bytes, true});
-        taken.push_back(c.pool.size() - 1);
-        return p;
-    }
-};
+}  // namespace bgapi
+
+namespace {
 
 EE get2d(TensorDesc d, DataType *dt, DataFormat *df, U32 *rows, U32 *cols)
 {
@@ -1551,13 +1496,8 @@ EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScal
 }
 
 // ---- int8 convolution (compute/tensor/src/cpu/x86/int8/convolution.cpp:97-150) ---------------------
-namespace {
-
-struct ConvShape {
-    U32 n, ic, ih, iw, oc, fh, fw, oh, ow;
-    U32 sh, sw, pt, pb, pl, pr, dh, dw;
-    U32 Hp, Wp, ICp, Kp, N16;
-};
+extern "C++" {
+namespace bgapi {
 
 EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w)
 {
@@ -1759,7 +1699,8 @@ EE conv_device(const ConvShape &s, DataFormat idf, const void *input, const void
     return take_scale(c, &scale[1]);
 }
 
-}  // namespace
+}  // namespace bgapi
+}  // extern "C++"
 
 EE convolution_infer_output_size_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, ConvolutionParamSpec p,
     TensorDesc *outputDesc, DataType targetDataType, Arch arch)

@@ -110,6 +110,33 @@ hipError_t launch_conv_pad(const uint8_t *in, uint32_t N, uint32_t C, uint32_t H
 hipError_t launch_conv_pack_filter(const int8_t *src, uint32_t OC, uint32_t IC, uint32_t fh, uint32_t fw, int32_t *offsetC,
     int8_t *dst, hipStream_t st);
 
+// ---- int8 deconvolution (deconv.hip) ------------------------------------------------------------------
+// filter s8 [ic][oc][taps] -> offsetC[taps * oc] and the convolution's packed matrix with rows tap * oc + o over K = ic
+hipError_t launch_deconv_pack_filter(const int8_t *src, uint32_t IC, uint32_t OC, uint32_t taps, int32_t *offsetC, int8_t *dst,
+    hipStream_t st);
+hipError_t launch_nchw_to_c8_u8(const uint8_t *in, uint32_t N, uint32_t C, uint32_t HW, uint8_t *out, hipStream_t st);  // C % 8 == 0
+hipError_t launch_repeat_f32(const float *src, uint32_t period, uint32_t n, float *out, hipStream_t st);  // out[i] = src[i % period]
+hipError_t launch_relu_u8(uint8_t *q, uint32_t n, hipStream_t st);  // in place max(q, 128)
+enum DeconvMode {
+    DECONV_I32 = 0,          // int32 sums + round(scaleO * bias), optional integer ReLU; stored, max|.| folded into absmax
+    DECONV_F32_DEQ = 1,      // the same sums, then cvt(acc) * factor
+    DECONV_F32_SUM = 2,      // bias + sum of cvt(col) * factor in ascending (kh, kw) order, optional fp32 ReLU
+    DECONV_U8 = 3,           // kernel == stride: the one u8 column byte per output, optional max(q, 128)
+    DECONV_F32_FROM_U8 = 4   // kernel == stride: cvt(q - 128) * factor, optional fp32 ReLU
+};
+struct DeconvArgs {
+    const void *col = nullptr;   // [n][fh * fw * oc / 16][ih][iw][16], int32 (u8 for the kernel == stride modes)
+    void *out = nullptr;         // [n][oc / 16][oh][ow][16]
+    uint32_t n = 0, oc = 0, ih = 0, iw = 0, oh = 0, ow = 0, fh = 0, fw = 0, sh = 0, sw = 0, pt = 0, pl = 0;
+    const float *bias = nullptr; // [oc], 16-byte aligned
+    float scaleO = 0;            // input scale * filter scale
+    float factor = 0;            // 1 / scaleO, or 1 / (scale of the u8 columns)
+    int relu = 0;
+    int mode = 0;
+    uint32_t *absmax = nullptr;  // DECONV_I32: cleared scratch slots
+};
+hipError_t launch_deconv_gather(const DeconvArgs &a, hipStream_t st);
+
 // ---- 1-bit convolution (bnn.hip) ----------------------------------------------------------------
 struct BnnArgs {
     const uint32_t *x = nullptr;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded

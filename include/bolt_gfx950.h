@@ -205,6 +205,45 @@ EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwi
     const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, F32 *scale,
     ActivationParamSpec activationDesc, Arch arch);
 
+/* ---- tensor_computing: int8 deconvolution (transposed convolution) ------------------------ */
+/* The (TensorDesc + pointer) forms behind the reference's deconvolution*() on x86:
+ *   deconvolution_infer_output_size_cpu        compute/tensor/src/deconvolution.cpp:23-65
+ *   deconvolution_infer_forward_algorithm_cpu  compute/tensor/src/cpu/deconvolution.cpp:23-55
+ *   deconvolution_transform_filter_bytes_cpu   compute/tensor/src/cpu/deconvolution.cpp:128-156
+ *   deconvolution_transform_filter_cpu         compute/tensor/src/cpu/deconvolution.cpp:158-186
+ *   deconvolution_infer_forward_tmp_bytes_cpu  compute/tensor/src/cpu/deconvolution.cpp:188-250
+ *   deconvolution_cpu                          compute/tensor/src/cpu/deconvolution.cpp:487-538
+ * Input DT_U8_Q: DF_NCHW runs the reference's IM2COL_GEMM route (deconvolution_gemm, :252-365), DF_NCHWC16 its
+ * POINTWISE route (deconvolution_pointwise_x86, cpu/x86/deconvolution.cpp:130-257); both multiply every input pixel
+ * with the [ic] x [fh * fw * oc] filter matrix and add the columns onto the output pixels they land on, and differ in
+ * where bias, ReLU and the change of type sit -- each is reproduced bit for bit, including what the call leaves in
+ * the caller's scale array: scale[3] = {input, output (in / out), filter}, host memory;
+ *   IM2COL_GEMM: DT_F32 leaves it alone; DT_U8_Q sets scale[2] = scale[0] * scale[2] and, when scale[1] <= 0 on entry,
+ *                scale[1] = the dynamic output scale (scale[1] > 0: quantised with that scale);
+ *   POINTWISE:   scale[1] = the output scale (DT_U8_Q; always dynamic), or what the inner convolution left there
+ *                (DT_F32: input * filter scale; with kernel == stride the scale of its u8 columns); DT_U8_Q with
+ *                overlapping taps also sets scale[2] = scale[0] * scale[2].
+ * Filter: DT_I8 DF_NCHW [ic, oc, fh, fw] -> blob of deconvolution_transform_filter_bytes_gfx950 bytes; ftmDesc is what
+ * the reference returns for the algorithm (DF_NKNxKx 2-D for IM2COL_GEMM, DF_NCHWC2NxC4 for POINTWISE).
+ * Output: DF_NCHWC16, DT_U8_Q or DT_F32. ic % 8 == 0 (DF_NCHWC16 input: ic % 16 == 0), oc % 16 == 0, group 1, no
+ * dilation; ACTIVATION_NULL or ACTIVATION_RELU. GROUP_DECONV (depthwise) and DF_NCHWC8 inputs return NOT_SUPPORTED:
+ * for the latter the reference lays its bias rows out in blocks of 8 under a 16-channel output. */
+EE deconvolution_infer_output_size_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, ConvolutionParamSpec convParamSpec,
+    TensorDesc *outputDesc, DataType targetDataType, Arch arch);
+EE deconvolution_infer_forward_algorithm_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec convParamSpec, ConvolutionPolicy policy, ConvolutionForwardAlgorithm *algorithm,
+    DataType targetDataType, Arch arch);
+EE deconvolution_transform_filter_bytes_gfx950(TensorDesc filterDesc, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch);
+EE deconvolution_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, TensorDesc *ftmDesc, void *filterTransformed, Arch arch);
+EE deconvolution_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec convParamSpec, ConvolutionForwardAlgorithm algorithm, U32 *bytes, Arch arch);
+EE deconvolution_gfx950(TensorDesc inputDesc, void *input, TensorDesc filterDesc, const void *filter,
+    ConvolutionParamSpec convParamSpec, ConvolutionForwardAlgorithm algorithm, TensorDesc scaleDesc, void *scale,
+    TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output,
+    ActivationParamSpec activationDesc, Arch arch);
+
 /* ---- 1-bit (XNOR / DoReFa) convolution ---------------------------------------------- */
 /* compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72 (convolution_bnn), filter transform
  * compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86, tmp bytes

@@ -74,6 +74,20 @@ void orc_conv_int8_acc(const orc_conv_desc *d, const uint8_t *in, const int8_t *
 void orc_conv_int8(const orc_conv_desc *d, const uint8_t *in, const int8_t *filter, const float *bias,
     const float *eltwise, float *scale /* [in, out, filter] */, void *out);
 
+/* ---- int8 deconvolution (oracle_deconv.c) ---------------------------------------------- */
+typedef struct {
+    uint32_t n, ic, ih, iw;      /* input u8: in_c = 0 plain NCHW, 8 / 16 = NCHWC8 / NCHWC16 */
+    uint32_t oc, fh, fw;         /* filter s8 [ic][oc][fh][fw] */
+    uint32_t sh, sw, pt, pb, pl, pr;
+    uint32_t oh, ow;
+    int in_c;
+    int out_c;                   /* channel block of the output layout: 16, or 8 when oc == 8 */
+    int relu;
+    int odt;                     /* ORC_F32 / ORC_U8Q (ORC_I32: raw sums of the gemm form) */
+} orc_deconv_desc;
+void orc_deconv_int8(const orc_deconv_desc *d, const uint8_t *in, const int8_t *filter, const float *bias,
+    float *scale /* [in, out, filter]; left as the reference leaves the caller's array */, void *out);
+
 /* ---- 1-bit convolution ------------------------------------------------------------- */
 typedef struct {
     uint32_t n, ic, ih, iw, oc, fh, fw, sh, sw, pt, pb, pl, pr, oh, ow;

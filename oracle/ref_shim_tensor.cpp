@@ -185,6 +185,70 @@ int ref_conv_queries(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32
     return 0;
 }
 
+// int8 deconvolution through the public Tensor API in the engine's order (inference/engine/include/cpu/deconvolution_cpu.hpp:
+// infer_output_size -> infer_forward_algorithm -> transform_filter_bytes -> transform_filter -> infer_forward_tmp_bytes ->
+// deconvolution). Input u8 (DT_U8_Q) in `idf` (DF_NCHW = 0 -> IM2COL_GEMM, DF_NCHWC8 = 2 / DF_NCHWC16 = 41 -> POINTWISE),
+// filter s8 [ic][oc][fh][fw], fp32 bias [oc]. scale[3] = {input, output (in/out), filter} is the caller's array and comes
+// back as the reference leaves it. q[0..8] = output desc, q[9] = algorithm, q[10] = filter bytes, q[11..19] = ftm desc,
+// q[20] = tmp bytes. `out` must hold n * oc * oh * ow elements of odt.
+int ref_deconv_int8(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 fw, U32 sh, U32 sw, U32 pt, U32 pb, U32 pl,
+    U32 pr, const uint8_t *in, const int8_t *filter, const float *bias, float *scale, int relu, int odt, void *out, U32 *q)
+{
+    ConvolutionParamSpec p = createConvolutionParamSpec(
+        1, 1, fh, fw, 1, sh, sw, 0, 0, pt, pb, pl, pr, 1, 1, 1, oc, CONVOLUTION_DECONVOLUTION);
+    TensorDesc id = tensor4df(DT_U8_Q, (DataFormat)idf, n, ic, ih, iw);
+    Tensor input = make(id, in);
+    TensorDesc fd = tensor4df(DT_I8, DF_NCHW, ic, oc, fh, fw);
+    Tensor filt = make(fd, filter);
+    Tensor output;
+    EE e = deconvolution_infer_output_size(&input, filt, p, &output, (DataType)odt, &g_arch);
+    if (e != SUCCESS) {
+        return 1000 + e;
+    }
+    put_desc(output.get_desc(), q);
+    ActivationParamSpec act;
+    act.mode = relu ? ACTIVATION_RELU : ACTIVATION_NULL;
+    ConvolutionForwardAlgorithm alg = CONVOLUTION_ALGORITHM_NULL;
+    e = deconvolution_infer_forward_algorithm(input, filt, output, p, CONVOLUTION_FASTEST, &alg, (DataType)odt, act, &g_arch);
+    if (e != SUCCESS) {
+        return 2000 + e;
+    }
+    q[9] = alg;
+    U32 fb = 0;
+    e = deconvolution_transform_filter_bytes(filt, p, alg, &fb, &g_arch);
+    if (e != SUCCESS) {
+        return 3000 + e;
+    }
+    q[10] = fb;
+    Tensor ftm = Tensor::alloc_sized<CPUMem>(tensor1d(DT_U8, fb + 64)), none;
+    e = deconvolution_transform_filter(filt, p, alg, none, &ftm, &g_arch);
+    if (e != SUCCESS) {
+        return 4000 + e;
+    }
+    put_desc(ftm.get_desc(), q + 11);
+    U32 tb = 0;
+    e = deconvolution_infer_forward_tmp_bytes(input, ftm, output, p, alg, &tb, &g_arch);
+    if (e != SUCCESS) {
+        return 5000 + e;
+    }
+    q[20] = tb;
+    // The POINTWISE route runs a 1x1 convolution inside whose own tmp needs (the int32 results ahead of its
+    // requantisation, x86/int8/convolution.cpp:40-93) are not part of deconvolution_infer_forward_tmp_bytes
+    // (cpu/deconvolution.cpp:195-222); the engine hides that by sizing one tmp as the maximum over all operators.
+    // Here the buffer gets that much slack so the reference does not write past it.
+    const size_t slack = (size_t)n * ih * iw * oc * fh * fw * 8 + (1u << 20);
+    Tensor tmp = Tensor::alloc_sized<CPUMem>(tensor1d(DT_U8, tb + slack));
+    memset(get_ptr_from_tensor(tmp, CPU_GENERAL), 0, tb + slack);
+    Tensor biasT = make(tensor1d(DT_F32, oc), bias);
+    output.alloc();
+    e = deconvolution(input, ftm, p, alg, scale, biasT, tmp, output, act, &g_arch);
+    if (e != SUCCESS) {
+        return 6000 + e;
+    }
+    memcpy(out, get_ptr_from_tensor(output, CPU_GENERAL), tensorNumBytes(output.get_desc()));
+    return 0;
+}
+
 // fp32 neighbours of the int8 GEMMs inside an encoder layer
 int ref_layer_norm_f32(U32 rows, U32 H, const float *in, const float *gamma, const float *beta, float *out)
 {

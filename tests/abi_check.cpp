@@ -59,6 +59,11 @@ SAME(requantize_cpu, requantize_gfx950);                             // cpu/tens
 SAME_PLUS_ARCH(convolution_transform_filter_bytes_x86, convolution_transform_filter_bytes_gfx950);
 SAME_PLUS_ARCH(convolution_transform_filter_x86, convolution_transform_filter_gfx950);
 SAME_PLUS_ARCH(convolution_infer_forward_tmp_bytes_x86, convolution_infer_forward_tmp_bytes_gfx950);
+SAME(deconvolution_infer_forward_algorithm_cpu, deconvolution_infer_forward_algorithm_gfx950);  // cpu/tensor_computing_cpu.h:200-246
+SAME(deconvolution_transform_filter_bytes_cpu, deconvolution_transform_filter_bytes_gfx950);
+SAME(deconvolution_transform_filter_cpu, deconvolution_transform_filter_gfx950);
+SAME(deconvolution_infer_forward_tmp_bytes_cpu, deconvolution_infer_forward_tmp_bytes_gfx950);
+SAME(deconvolution_cpu, deconvolution_gfx950);
 
 // ---- plain-data types ---------------------------------------------------------------------------------------------
 #define SIZE(T) static_assert(sizeof(ours::T) == sizeof(::T), "sizeof " #T)
