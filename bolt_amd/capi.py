@@ -204,6 +204,12 @@ SIGNATURES = {
                                                                C.c_int, _u32p, C.c_int]),
     "deconvolution_gfx950": (C.c_int, [TensorDesc, _vp, TensorDesc, _vp, ConvolutionParamSpec, C.c_int, TensorDesc, _vp,
                                        TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, ActivationParamSpec, C.c_int]),
+    "depthwise_convolution_transform_filter_bytes_int8_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
+    "depthwise_convolution_transform_filter_int8_gfx950": (C.c_int, [TensorDesc, _vp, _TDp, _vp, C.c_int]),
+    "depthwise_pointwise_convolution_int8_gfx950": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, TensorDesc, _vp,
+                                                              ConvolutionParamSpec, TensorDesc, _vp, TensorDesc, _vp, _u32,
+                                                              _vp, TensorDesc, _vp, _f32p, ActivationParamSpec,
+                                                              ActivationParamSpec, C.c_int]),
     "convolution_transform_filter_bytes_bnn_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
     "convolution_transform_filter_bnn_gfx950": (C.c_int, [TensorDesc, _vp, C.POINTER(TensorDesc), _vp, C.c_int]),
     "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),

@@ -137,6 +137,19 @@ struct DeconvArgs {
 };
 hipError_t launch_deconv_gather(const DeconvArgs &a, hipStream_t st);
 
+// ---- int8 depthwise convolution (depthwise.hip) ---------------------------------------------------------
+struct DepthwiseArgs {
+    const uint8_t *in = nullptr;     // u8 [n][c/16][ih][iw][16]
+    const int8_t *filter = nullptr;  // per 16-channel block: [(fh*fw+3)/4][16][4]
+    const int32_t *offsetC = nullptr;  // [c], -128 * sum of the channel's taps
+    const float *bias = nullptr;     // [c] or null
+    float scaleO = 0;                // input scale * filter scale
+    int32_t *out = nullptr;          // [n][c/16][oh][ow][16]
+    uint32_t n = 0, c = 0, ih = 0, iw = 0, oh = 0, ow = 0, fh = 0, fw = 0, sh = 0, sw = 0;
+    int relu = 0;
+};
+hipError_t launch_depthwise_u8s8_i32(const DepthwiseArgs &a, hipStream_t st);
+
 // ---- 1-bit convolution (bnn.hip) ----------------------------------------------------------------
 struct BnnArgs {
     const uint32_t *x = nullptr;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded

@@ -121,3 +121,43 @@ def convolution_bnn(x, idt, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, s
                                      tensor1d(DT_F32, oc), ptr(bias), b.value, ptr(tmp), odesc, ptr(out), act, arch)
     check(e, "convolution_bnn")
     return out
+
+
+def depthwise_transform_filter(filt_chw, c, fh, fw):
+    """filt_chw: s8 [c][fh][fw] (the reference's [1, c, fh, fw] DF_NCHW). Returns (blob, ftm desc)."""
+    arch = arch_of(filt_chw)
+    fdesc = tensor4df(DT_I8, DF_NCHW, 1, c, fh, fw)
+    b = C.c_uint32(0)
+    check(lib().depthwise_convolution_transform_filter_bytes_int8_gfx950(fdesc, C.byref(b), arch), "dw_filter_bytes")
+    blob = _empty_like_mode(filt_chw, b.value)
+    ftm = TensorDesc()
+    check(lib().depthwise_convolution_transform_filter_int8_gfx950(fdesc, ptr(filt_chw), C.byref(ftm), ptr(blob), arch),
+          "dw_transform_filter")
+    return blob, ftm
+
+
+def depthwise_convolution_i32(x, n, c, ih, iw, blob, ftm, fh, fw, stride, bias, scale, relu, pad=0):
+    """x: u8 NCHWC16. Returns int32 NCHWC16; scale = [sI, sO, sF] (sO written)."""
+    arch = arch_of(x)
+    p = conv_param_spec(c, fh, fw, stride, pad, 1, group=c)
+    oh, ow = conv_out_hw(ih, iw, fh, fw, stride, pad)
+    idesc = tensor4df(DT_U8_Q, DF_NCHWC16, n, c, ih, iw)
+    odesc = tensor4df(DT_I32, DF_NCHWC16, n, c, oh, ow)
+    count = n * c * oh * ow
+    if _is_torch(x):
+        import torch
+        out = torch.zeros(count, dtype=torch.int32, device=x.device)
+    else:
+        out = np.zeros(count, np.int32)
+    sarr = (C.c_float * 3)(*[float(np.float32(v)) for v in scale])
+    act, none = ActivationParamSpec(), ActivationParamSpec()
+    act.mode = ACTIVATION_RELU if relu else ACTIVATION_NULL
+    none.mode = ACTIVATION_NULL
+    blank = TensorDesc()
+    e = lib().depthwise_pointwise_convolution_int8_gfx950(idesc, ptr(x), None, ftm, ptr(blob), blank, None, p,
+                                                          tensor1d(DT_F32, c), ptr(bias), blank, None, 0, None, odesc,
+                                                          ptr(out), sarr, act, none, arch)
+    check(e, "depthwise_convolution")
+    for i in range(3):
+        scale[i] = np.float32(sarr[i])
+    return out

@@ -244,6 +244,26 @@ EE deconvolution_gfx950(TensorDesc inputDesc, void *input, TensorDesc filterDesc
     TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output,
     ActivationParamSpec activationDesc, Arch arch);
 
+/* ---- tensor_computing: int8 depthwise convolution ------------------------------------------ */
+/* depthwise_convolution_transform_filter_int8 (compute/tensor/src/cpu/x86/int8/depthwise_convolution_transform.cpp:17-69,
+ * bytes: compute/tensor/src/depthwise_pointwise_convolution.cpp:197-205) and depthwise_pointwise_convolution_int8
+ * (compute/tensor/src/cpu/x86/int8/avx512/depthwise_convolution_direct.cpp:441-599), each + Arch.
+ * The filter blob is byte for byte the reference's: [offsetC c*4 | per 16 channels: [tap / 4][channel][tap % 4]],
+ * tagged DF_NCHWN8HW4 as the reference tags it. The convolution reproduces the one result that function defines:
+ * DT_I32 output (DF_NCHWC16) of the depthwise stage alone, from a DT_U8_Q DF_NCHWC16 input, ReLU or no activation,
+ * acc = offsetC + round(bias * sI * sF) + sum in_u8 * w, scale[1] = sI * sF on return. Paddings and dilation must be
+ * 0 / 1 (the reference's gather ignores them), c % 16 == 0; a pointwise filter, an eltwise input and DT_F32 / DT_U8_Q
+ * outputs return NOT_SUPPORTED (the reference's fp32 epilogue converts the wrong register, its quantised result never
+ * reaches the output tensor, its pointwise stage is not run). tmp is not used. */
+EE depthwise_convolution_transform_filter_bytes_int8_gfx950(TensorDesc filterDesc, U32 *bytes, Arch arch);
+EE depthwise_convolution_transform_filter_int8_gfx950(TensorDesc filterDesc, const INT8 *filter, TensorDesc *ftmDesc,
+    INT8 *filterTransformed, Arch arch);
+EE depthwise_pointwise_convolution_int8_gfx950(TensorDesc inputDesc, UINT8 *inArray, F32 *eltwiseInput,
+    TensorDesc dwFilterDesc, const INT8 *dwFilterArray, TensorDesc pwFilterDesc, const INT8 *pwFilterArray,
+    ConvolutionParamSpec convParamSpec, TensorDesc dwBiasDesc, const F32 *dwBiasArray, TensorDesc pwBiasDesc,
+    const F32 *pwBiasArray, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *outArray, F32 *scale,
+    ActivationParamSpec depthwiseActivationParamSpec, ActivationParamSpec pointwiseActivationParamSpec, Arch arch);
+
 /* ---- 1-bit (XNOR / DoReFa) convolution ---------------------------------------------- */
 /* compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72 (convolution_bnn), filter transform
  * compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86, tmp bytes

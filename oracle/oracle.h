@@ -88,6 +88,11 @@ typedef struct {
 void orc_deconv_int8(const orc_deconv_desc *d, const uint8_t *in, const int8_t *filter, const float *bias,
     float *scale /* [in, out, filter]; left as the reference leaves the caller's array */, void *out);
 
+/* int8 depthwise convolution, int32 result, no padding (oracle_deconv.c) */
+void orc_depthwise_int8_i32(uint32_t n, uint32_t c, uint32_t ih, uint32_t iw, uint32_t fh, uint32_t fw, uint32_t sh,
+    uint32_t sw, uint32_t oh, uint32_t ow, const uint8_t *in, const int8_t *filter /* [c][fh][fw] */, const float *bias,
+    float *scale /* [in, out, filter] */, int relu, int32_t *out);
+
 /* ---- 1-bit convolution ------------------------------------------------------------- */
 typedef struct {
     uint32_t n, ic, ih, iw, oc, fh, fw, sh, sw, pt, pb, pl, pr, oh, ow;

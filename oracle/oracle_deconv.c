@@ -227,3 +227,47 @@ void orc_deconv_int8(const orc_deconv_desc *d, const uint8_t *in, const int8_t *
     }
     free(acc);
 }
+
+/* ------------------------------------------------------------------------------------
+ * int8 depthwise convolution as the reference's x86 kernel computes it
+ * (compute/tensor/src/cpu/x86/int8/avx512/depthwise_convolution_direct.cpp:441-599): u8 NCHWC16 input,
+ * one s8 fh x fw filter per channel, int32 result in NCHWC16:
+ *   acc[n, c, y, x] = round(bias[c] * sI * sF) + sum_{kh, kw} (in_u8[n, c, y*sh + kh, x*sw + kw] - 128) * w[c][kh][kw]
+ * with ReLU in the integer domain (:125-145). The window is taken from the UNPADDED image at (y*sh, x*sw) (:560-566):
+ * paddings and dilation do not enter the gather, so only pad 0 / dilation 1 is a convolution; the restatement covers
+ * exactly that. The int32 result is the only defined one: the fp32 epilogue converts the bits of the scale factor
+ * instead of the accumulators (:148-166), and a quantised result is left in tmp, never written to the output (:521-525).
+ * scale = {input, output (written: sI * sF), filter}.
+ * ---------------------------------------------------------------------------------- */
+void orc_depthwise_int8_i32(uint32_t n, uint32_t c, uint32_t ih, uint32_t iw, uint32_t fh, uint32_t fw, uint32_t sh,
+    uint32_t sw, uint32_t oh, uint32_t ow, const uint8_t *in, const int8_t *filter, const float *bias, float *scale, int relu,
+    int32_t *out)
+{
+    const float s = scale[0] * scale[2];
+    scale[1] = s;
+    for (uint32_t b = 0; b < n; ++b) {
+        for (uint32_t ch = 0; ch < c; ++ch) {
+            int32_t bq = 0;
+            if (bias) {
+                const float p = bias[ch] * s;
+                bq = (int32_t)round((double)p); /* avx512/quantize.cpp:236-269 */
+            }
+            for (uint32_t y = 0; y < oh; ++y) {
+                for (uint32_t x = 0; x < ow; ++x) {
+                    uint32_t a = (uint32_t)bq;
+                    for (uint32_t kh = 0; kh < fh; ++kh) {
+                        for (uint32_t kw = 0; kw < fw; ++kw) {
+                            const size_t ii = ((((size_t)b * (c / 16) + ch / 16) * ih + (y * sh + kh)) * iw + (x * sw + kw)) * 16 + ch % 16;
+                            a += (uint32_t)(((int32_t)in[ii] - 128) * (int32_t)filter[((size_t)ch * fh + kh) * fw + kw]);
+                        }
+                    }
+                    int32_t v = (int32_t)a;
+                    if (relu && v < 0) {
+                        v = 0;
+                    }
+                    out[((((size_t)b * (c / 16) + ch / 16) * oh + y) * ow + x) * 16 + ch % 16] = v;
+                }
+            }
+        }
+    }
+}

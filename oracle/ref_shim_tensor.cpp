@@ -14,6 +14,7 @@
 #include "tensor_computing.h"
 #include "blas_enhance.h"
 #include "cpu/x86/fp32/tensor_computing_fp32.h"
+#include "cpu/x86/int8/tensor_computing_int8.h"
 #include "cpu/x86/fp32/x86_functions_fp32.h"
 
 static ArchInfo g_arch = {X86_AVX512, nullptr};
@@ -247,6 +248,46 @@ int ref_deconv_int8(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 
     }
     memcpy(out, get_ptr_from_tensor(output, CPU_GENERAL), tensorNumBytes(output.get_desc()));
     return 0;
+}
+
+// int8 depthwise convolution, inner form (compute/tensor/src/cpu/x86/int8/avx512/depthwise_convolution_direct.cpp:441-599)
+// with no pointwise stage: depthwise_convolution_transform_filter_int8 then depthwise_pointwise_convolution_int8.
+// Input u8 NCHWC16, filter s8 [1][c][fh][fw] (DF_NCHW), fp32 bias [c]; odt DT_I32 or DT_F32; output NCHWC16.
+// The public depthwise_convolution() route hands this function a null scale array (cpu/x86/depthwise_convolution.cpp:
+// 107-113), which it dereferences; so it is only callable directly.
+int ref_depthwise_int8(U32 n, U32 c, U32 ih, U32 iw, U32 fh, U32 fw, U32 sh, U32 sw, U32 pt, U32 pb, U32 pl, U32 pr, U32 oh,
+    U32 ow, const uint8_t *in, const int8_t *filter, const float *bias, float *scale, int relu, int odt, void *out)
+{
+    ConvolutionParamSpec p = createConvolutionParamSpec(
+        c, 1, fh, fw, 1, sh, sw, 0, 0, pt, pb, pl, pr, c, 1, 1, c, CONVOLUTION_DEPTHWISE);
+    TensorDesc id = tensor4df(DT_U8_Q, DF_NCHWC16, n, c, ih, iw);
+    TensorDesc fd = tensor4df(DT_I8, DF_NCHW, 1, c, fh, fw);
+    TensorDesc od = tensor4df((DataType)odt, DF_NCHWC16, n, c, oh, ow);
+    U32 fsz = (fh * fw + 3) / 4 * 4;
+    std::vector<INT8> ftm((size_t)fsz * c + c * 4 + 4096, 0);
+    TensorDesc ftmDesc;
+    EE e = depthwise_convolution_transform_filter_int8(fd, filter, &ftmDesc, ftm.data());
+    if (e != SUCCESS) {
+        return 1000 + e;
+    }
+    std::vector<uint8_t> tmp((size_t)n * c * oh * ow * 4 + (size_t)c * 4 + (size_t)fsz * 16 * 16 + (1u << 20), 0);
+    ActivationParamSpec act, none;
+    act.mode = relu ? ACTIVATION_RELU : ACTIVATION_NULL;
+    none.mode = ACTIVATION_NULL;
+    TensorDesc blank;
+    e = depthwise_pointwise_convolution_int8(id, (UINT8 *)in, nullptr, ftmDesc, ftm.data(), blank, nullptr, p,
+        tensor1d(DT_F32, c), bias, blank, nullptr, (U32)tmp.size(), tmp.data(), od, out, scale, act, none);
+    return e;
+}
+
+// The reference's transformed depthwise filter (x86/int8/depthwise_convolution_transform.cpp:17-69): blob must hold
+// ALIGN(fh * fw, 4) * c + c * 4 bytes; desc9 = its desc.
+int ref_depthwise_transform_filter(U32 c, U32 fh, U32 fw, const int8_t *filter, int8_t *blob, U32 *desc9)
+{
+    TensorDesc fd = tensor4df(DT_I8, DF_NCHW, 1, c, fh, fw), ftm;
+    EE e = depthwise_convolution_transform_filter_int8(fd, filter, &ftm, blob);
+    put_desc(ftm, desc9);
+    return e;
 }
 
 // fp32 neighbours of the int8 GEMMs inside an encoder layer

@@ -64,6 +64,8 @@ SAME(deconvolution_transform_filter_bytes_cpu, deconvolution_transform_filter_by
 SAME(deconvolution_transform_filter_cpu, deconvolution_transform_filter_gfx950);
 SAME(deconvolution_infer_forward_tmp_bytes_cpu, deconvolution_infer_forward_tmp_bytes_gfx950);
 SAME(deconvolution_cpu, deconvolution_gfx950);
+SAME_PLUS_ARCH(depthwise_convolution_transform_filter_int8, depthwise_convolution_transform_filter_int8_gfx950);
+SAME_PLUS_ARCH(depthwise_pointwise_convolution_int8, depthwise_pointwise_convolution_int8_gfx950);
 
 // ---- plain-data types ---------------------------------------------------------------------------------------------
 #define SIZE(T) static_assert(sizeof(ours::T) == sizeof(::T), "sizeof " #T)
