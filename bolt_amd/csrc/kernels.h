@@ -150,6 +150,16 @@ struct DepthwiseArgs {
 };
 hipError_t launch_depthwise_u8s8_i32(const DepthwiseArgs &a, hipStream_t st);
 
+// ---- weight storage of the post-training quantisation tool (ptq.hip) ---------------------------------------
+// ws: kWsWords scratch words (overwritten). floor_: the caller's scale; the scale used, max(127 or 7 / max|w|, floor_),
+// goes to *ds_out. n even for the 4-bit form, a multiple of 8 for the 1-bit form.
+hipError_t launch_ws_int8(const float *w, uint32_t n, int8_t *q, uint32_t *ws, float floor_, float *ds_out, hipStream_t st);
+hipError_t launch_ws_int4(const float *w, uint32_t n, int8_t *q, uint32_t *ws, float floor_, float *ds_out, hipStream_t st);
+hipError_t launch_ws_bnn(const float *w, uint32_t n, uint8_t *bits, uint32_t *ws, float *ds_out, hipStream_t st);
+// src4: q holds two 4-bit values per byte (value = nibble - 7), else one s8 per byte; dst 0: fp32 = (1 / scale) * value,
+// 1: s8 = value, 2: u8 = value + 128 (dst 1 / 2 only from 4-bit storage)
+hipError_t launch_ws_expand(const int8_t *q, uint32_t n, int src4, int dst, float scale, void *d, hipStream_t st);
+
 // ---- 1-bit convolution (bnn.hip) ----------------------------------------------------------------
 struct BnnArgs {
     const uint32_t *x = nullptr;     // [n][Hp][Wp][IC/32] dwords, zero-bit padded

@@ -264,6 +264,37 @@ EE depthwise_pointwise_convolution_int8_gfx950(TensorDesc inputDesc, UINT8 *inAr
     const F32 *pwBiasArray, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *outArray, F32 *scale,
     ActivationParamSpec depthwiseActivationParamSpec, ActivationParamSpec pointwiseActivationParamSpec, Arch arch);
 
+/* ---- offline quantisation: weight storage, load-time expansion, stored scales -------------------- */
+/* The data-parallel part of the post-training quantisation tool (model_tools/tools/quantization/
+ * post_training_quantization.cpp -> ms_datatype_converter): the three weight-storage converters of
+ * model_tools/src/model_data_type_converter.cpp:22-103, same arguments + Arch, EE instead of void / F32:
+ *   ws_datatype_converter_int8  q = rne(w * scale), scale = max(127.0 / max|w|, *scale) (in: floor, out: used)
+ *   ws_datatype_converter_int4  two values per byte, nibble = rne(w * 7.0 / max|w|) + 7, low nibble first;
+ *                               scale = max(7.0 / max|w|, *scale). paramNum must be even (the reference misplaces
+ *                               an odd trailing element, :99-101).
+ *   ws_datatype_converter_bnn   one bit per weight (w > 0), first weight in the top bit; *scale = the first positive
+ *                               weight (the reference returns it). paramNum % 8 == 0.
+ * and the expansion a model loader applies to such weights (common/model_spec/src/model_deserialize.cpp:162-222):
+ *   dequantize_int8_weight / dequantize_int4_weight  d = (1 / scale) * value (the DT_F32 instantiations)
+ *   dequantize_int4_int8 / dequantize_int4_u8_q      value = nibble - 7 as s8, or + 128 as u8
+ * originalPtr / q are fp32 / packed inputs, targetPtr / d outputs; host or device pointers by Arch. */
+EE ws_datatype_converter_int8_gfx950(U8 *originalPtr, U8 *targetPtr, int paramNum, F32 *scale, Arch arch);
+EE ws_datatype_converter_int4_gfx950(U8 *originalPtr, U8 *targetPtr, int paramNum, F32 *scale, Arch arch);
+EE ws_datatype_converter_bnn_gfx950(U8 *originalPtr, U8 *targetPtr, int paramNum, F32 *scale, Arch arch);
+EE dequantize_int8_weight_gfx950(int num, F32 scale, INT8 *q, F32 *d, Arch arch);
+EE dequantize_int4_weight_gfx950(int num, F32 scale, INT8 *q, F32 *d, Arch arch);
+EE dequantize_int4_int8_gfx950(int num, INT8 *q, INT8 *d, Arch arch);
+EE dequantize_int4_u8_q_gfx950(int num, INT8 *q, UINT8 *d, Arch arch);
+/* The rule by which the engine's int8 operators turn the QuantSpec records a .bolt model stores for them
+ * (OperatorSpec::feature_scale, common/uni/include/parameter_spec.h:753-756; copied by Operator::init_feature_scale,
+ * inference/engine/include/operator.hpp:139-150) into the scales[3] = {input, output, filter} they pass down
+ * (inference/engine/include/cpu/convolution_cpu.hpp:143-157, deconvolution_cpu.hpp:65-84): a calibrated input scale
+ * is used only while the input is not yet quantised; the last record is the output scale, -2 there (or no record)
+ * leaves it dynamic (-1); *labelledNoQuant (optional) = 1 when the first record is 0 (operator.hpp:164-169).
+ * Pure host logic: no GPU is touched, no Arch. A clip value c from the tool's scale table is stored as 127 / c. */
+EE bolt_gfx950_operator_scales(const QuantSpec *featureScale, U32 numQuantFeature, DataType inputDataType,
+    F32 inputTensorScale, F32 filterScale, F32 scales[3], int *labelledNoQuant);
+
 /* ---- 1-bit (XNOR / DoReFa) convolution ---------------------------------------------- */
 /* compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72 (convolution_bnn), filter transform
  * compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86, tmp bytes

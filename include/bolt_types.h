@@ -383,4 +383,11 @@ static_assert(sizeof(RNNParamSpec) == 36, "RNNParamSpec must match Bolt's record
 static_assert(sizeof(DataType) == 4 && sizeof(DataFormat) == 4, "enums are 32-bit in Bolt");
 #endif
 
+/* common/uni/include/parameter_spec.h:753-756 (inside #pragma pack(8)): one record of per-tensor quantisation scales
+ * as a .bolt model stores them per operator (OperatorSpec::feature_scale) and per weight (WeightSpec::weight_scale) */
+typedef struct {
+    I32 num_scale;
+    F32 *scale;
+} QuantSpec;
+
 #endif

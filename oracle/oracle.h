@@ -93,6 +93,15 @@ void orc_depthwise_int8_i32(uint32_t n, uint32_t c, uint32_t ih, uint32_t iw, ui
     uint32_t sw, uint32_t oh, uint32_t ow, const uint8_t *in, const int8_t *filter /* [c][fh][fw] */, const float *bias,
     float *scale /* [in, out, filter] */, int relu, int32_t *out);
 
+/* ---- weight storage of the post-training quantisation tool (oracle_ptq.c) ----------------- */
+void orc_ws_convert_int8(const float *w, int n, int8_t *q, float *scale /* in: floor, out: scale used */);
+void orc_ws_convert_int4(const float *w, int n /* even */, int8_t *q, float *scale);
+float orc_ws_convert_bnn(const float *w, int n /* multiple of 8 */, uint8_t *bits);
+void orc_dequantize_int8_weight(int n, float scale, const int8_t *q, float *d);
+void orc_dequantize_int4_weight(int n, float scale, const int8_t *q, float *d);
+void orc_dequantize_int4_int8(int n, const int8_t *q, int8_t *d);
+void orc_dequantize_int4_u8q(int n, const int8_t *q, uint8_t *d);
+
 /* ---- 1-bit convolution ------------------------------------------------------------- */
 typedef struct {
     uint32_t n, ic, ih, iw, oc, fh, fw, sh, sw, pt, pb, pl, pr, oh, ow;

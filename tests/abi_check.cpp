@@ -18,6 +18,7 @@
 #include "cpu/tensor_computing_cpu.h"
 #include "cpu/x86/tensor_computing_x86.h"
 #include "cpu/x86/int8/tensor_computing_int8.h"
+#include "parameter_spec.h"
 
 #define BOLT_GFX950_NO_TYPES
 #include "bolt_gfx950.h"
@@ -90,6 +91,7 @@ FIELD(ConvolutionParamSpec, pad_right);
 FIELD(ConvolutionParamSpec, group);
 FIELD(ConvolutionParamSpec, dilatedRate_h);
 FIELD(ConvolutionParamSpec, convolution_type);
+static_assert(sizeof(ours::QuantSpec) == sizeof(QuantSpec) && offsetof(ours::QuantSpec, scale) == offsetof(QuantSpec, scale), "QuantSpec");
 FIELD(ConvolutionParamSpec, round_mode);
 SIZE(PoolingParamSpec);
 FIELD(PoolingParamSpec, mode);
