@@ -1042,6 +1042,155 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
 #undef BG3_STEP
 #undef BG3_ISSUE_A
 #undef BG3_ISSUE_B
+    } else if constexpr (PIPE == 4) {
+        // Ping-pong schedule as PIPE == 3 (A in whole 128-byte lines, pairs of K tiles, three pair slots of 32 KB), with
+        // the B fragments NOT staged through LDS: the packed right-hand side already holds every 16-column x 64-byte
+        // fragment as 1 KB in lane order, so each wave loads the TN fragments of its own columns straight into registers
+        // three tiles ahead (a ring of three register sets). The two waves that share a column block load the same
+        // bytes (the second is served by the CU's cache), which doubles the B requests; in exchange the LDS carries A
+        // only -- per K tile and CU 64 KB of fragment reads + 16 KB of arriving A instead of 96 + 32 KB, which at
+        // 128 bytes per cycle was as long as the 1024 cycles the tile's MFMAs take.
+        static_assert(PIPE != 4 || (!CONV && !FP4 && WM * WN == 8 && STAGES == 3 && T::kAFrags == 16 && T::kBFrags == 16 && TN == 4),
+            "the register-B loop is written for 256 x 256 matrix tiles");
+        constexpr uint32_t kASlot = T::kAFrags * 2048;
+        constexpr int kQA2 = 2 * T::kAFrags / T::kWaves;  // A requests per wave and tile pair
+        static_assert(3 * kASlot == (uint32_t)T::kLdsBytes, "LDS layout");
+        uint32_t offA[kQA2], offB[TN];
+#pragma unroll
+        for (int q = 0; q < kQA2; ++q) {
+            const uint32_t b = wave + q * T::kWaves;  // block of 8 rows
+            uint32_t row = m0 + b * 8 + (lane >> 3);
+            row = row < a.M ? row : a.M - 1;
+            const uint32_t row16 = (b & 1) * 8 + (lane >> 3);
+            offA[q] = row * a.lda + (((lane & 7) ^ ((row16 >> 1) & 7)) * 16);
+        }
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            uint32_t nb = (n0 >> 4) + wn * TN + y;
+            nb = nb < nblocks ? nb : nblocks - 1;
+            offB[y] = nb * 16 * K + lane * 16;
+        }
+        const uint32_t ksteps = K / 64, kpairs = ksteps / 2;  // the launcher checks K % 128 == 0
+        const uint32_t rdA = (i >> 3) * 1024 + ((i & 7) * 8 + (g ^ ((i >> 1) & 7))) * 16;
+#define BG4_ISSUE_A(aslot, pair)                                                                                  \
+    {                                                                                                             \
+        const uint8_t *base_ = a.A + (size_t)((pair) < kpairs ? (pair) : kpairs - 1) * 128;                       \
+        _Pragma("unroll") for (int q = 0; q < kQA2; ++q)                                                          \
+        {                                                                                                         \
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_ + offA[q]),                                           \
+                (lptr_t)(smem + (aslot)*kASlot + (wave + q * T::kWaves) * 1024), 16, 0, 0);                       \
+        }                                                                                                         \
+    }
+#define BG4_LOAD_B(FB, tile)                                                                                      \
+    {                                                                                                             \
+        const uint8_t *base_ = (const uint8_t *)a.Bp + (size_t)((tile) < ksteps ? (tile) : ksteps - 1) * 1024;    \
+        _Pragma("unroll") for (int y = 0; y < TN; ++y)                                                            \
+        {                                                                                                         \
+            /* issued as text, so that the compiler's own wait insertion does not see these loads: next to the */ \
+            /* LDS-bound requests it would wait for ALL outstanding memory operations before the first use.   */ \
+            /* The waits are the explicit vmcnt counts below; nothing reads FB between a load and its wait.    */ \
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(FB[y]) : "v"(base_ + offB[y]) : "memory");     \
+        }                                                                                                         \
+    }
+        // Request order: A0 B0 A1 B1 B2 | tile 0: A2 .. B3 | tile 1: .. B4 | tile 2: A3 .. B5 | ... : the even tile t
+        // requests pair t / 2 + 2 in its memory phase, every tile t loads B(t + 3) after its MFMAs into the register
+        // set it has just consumed. Behind the request of a pair come B, B, the next pair and one more B before the
+        // odd tile that first needs it starts: 2 * kQA2... = kQA2 + 3 * TN requests may then still be outstanding.
+        v4i fb0[TN], fb1[TN], fb2[TN], fa[TM];
+        BG4_ISSUE_A(0u, 0u);
+        BG4_LOAD_B(fb0, 0u);
+        BG4_ISSUE_A(1u, 1u);
+        BG4_LOAD_B(fb1, 1u);
+        BG4_LOAD_B(fb2, 2u);
+        const bool late = wave >= 4;
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kQA2 + 2 * TN));  // pair 0 (and B0) landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (late) {
+            __builtin_amdgcn_s_barrier();
+        }
+#define BG4_STEP(HALF, FB)                                                                                        \
+    {                                                                                                             \
+        if (HALF) {                                                                                               \
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(kQA2 + 3 * TN)); /* the pair of tile t + 1 has landed */          \
+            asm volatile("" ::: "memory");                                                                        \
+        } else {                                                                                                  \
+            BG4_ISSUE_A(aslot_req, t / 2 + 2);                                                                    \
+        }                                                                                                         \
+        {                                                                                                         \
+            const uint8_t *sA_ = smem + aslot * kASlot + (rdA ^ ((HALF)*64));                                     \
+            _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                        \
+            {                                                                                                     \
+                fa[x] = *(const v4i *)(sA_ + (wm * TM + x) * 2048);                                               \
+            }                                                                                                     \
+        }                                                                                                         \
+        __builtin_amdgcn_s_waitcnt(0xc07f);                                                                       \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                            \
+        {                                                                                                         \
+            fa[x] ^= flip;                                                                                        \
+        }                                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_s_barrier();                                                                             \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        /* B(t), loaded three tiles ago, is in its registers: behind it came B, a pair and B (in some order) */  \
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kQA2 + 2 * TN));                                                     \
+        asm volatile("" : "+v"(FB[0]), "+v"(FB[1]), "+v"(FB[2]), "+v"(FB[3]));                                    \
+        __builtin_amdgcn_s_setprio(1);                                                                            \
+        _Pragma("unroll") for (int x = 0; x < TM; ++x)                                                            \
+        {                                                                                                         \
+            _Pragma("unroll") for (int y = 0; y < TN; ++y)                                                        \
+            {                                                                                                     \
+                acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(FB[y], fa[x], acc[x][y], 0, 0, 0);              \
+            }                                                                                                     \
+        }                                                                                                         \
+        __builtin_amdgcn_s_setprio(0);                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        BG4_LOAD_B(FB, t + 3);                                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                                        \
+        asm volatile("" ::: "memory");                                                                            \
+        __builtin_amdgcn_s_barrier();                                                                             \
+        asm volatile("" ::: "memory");                                                                            \
+    }
+#define BG4_PAIR(FBE, FBO)                                                                                        \
+    {                                                                                                             \
+        BG4_STEP(0, FBE);                                                                                         \
+        ++t;                                                                                                      \
+        BG4_STEP(1, FBO);                                                                                         \
+        ++t;                                                                                                      \
+        aslot = aslot == 2 ? 0 : aslot + 1;                                                                       \
+        aslot_req = aslot_req == 2 ? 0 : aslot_req + 1;                                                           \
+    }
+        uint32_t aslot = 0, aslot_req = 2;  // slot of the pair being read / of the pair requested at the even tile
+        uint32_t t = 0;
+        while (t + 6 <= ksteps) {  // the register ring comes round every three tiles, the A halves every two
+            BG4_PAIR(fb0, fb1);
+            BG4_PAIR(fb2, fb0);
+            BG4_PAIR(fb1, fb2);
+        }
+        if (t + 2 <= ksteps) {
+            BG4_PAIR(fb0, fb1);
+        }
+        if (t + 2 <= ksteps) {
+            BG4_PAIR(fb2, fb0);
+        }
+        if (!late) {
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches
+        // The last loads of every register set are never consumed. Their destinations must stay allocated until the
+        // data has landed (the drain above): a register the compiler handed to something else in between -- an
+        // address, an accumulator -- would be overwritten when the load returns.
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            asm volatile("" ::"v"(fb0[y]), "v"(fb1[y]), "v"(fb2[y]));
+        }
+#undef BG4_PAIR
+#undef BG4_STEP
+#undef BG4_LOAD_B
+#undef BG4_ISSUE_A
     } else {
     // This wave's fragments per K tile: kQA A fragments (16 rows x 64 K-bytes), then B fragments.
     // Addresses are split into a wave-uniform 64-bit base that advances with the tile (scalar
@@ -1786,6 +1935,11 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             // ping-pong: 12 % faster than the fragment-prefetch loop at 8192^3, level elsewhere; with A requested in
             // whole lines another 4 % at 8192^3 and level at 4096^3 (needs K % 128 == 0 and 160 KB of LDS)
             tile = (a.K % 128 == 0) ? 12 : 11;
+            // up to two rounds of tiles the register-B form is 6-18 % faster (4096^3, the encoder's FFN shapes); long
+            // multi-round launches run at the clock the power limit allows either way and measure level
+            if (tile == 12 && b256 <= 512) {
+                tile = 13;
+            }
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
             tile = k64 ? 10 : 2;
         }
@@ -1797,15 +1951,21 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     if (tile >= 3 && !dma_ok) {
         tile = tiled_ok ? 2 : 0;
     }
+    if (tile == 13 && a.K % 128 != 0) {
+        tile = 11;
+    }
     if (tile == 12 && (a.K % 128 != 0 || !lds_160k())) {
         tile = 11;
     }
     if (a.epi.mode == EPI_U8_GELU_DYN) {
         // every tile's workgroup must be running when the first one waits for the others: full 256 x 256 tiles, one
         // workgroup per CU, and the sync area, status word and fallback buffer in place
-        if ((tile != 11 && tile != 12) || !gemm_gelu_dyn_fits(a.M, a.N, a.K) || !a.sync.slots || !a.status || !a.C32 || !a.dscale_out ||
+        if ((tile != 11 && tile != 12 && tile != 13) || !gemm_gelu_dyn_fits(a.M, a.N, a.K) || !a.sync.slots || !a.status || !a.C32 || !a.dscale_out ||
             !a.epi.scaleI || !a.epi.scaleW || a.sync.blocks == 0 || a.sync.blocks > kGridSyncMaxBlocks) {
             return hipErrorInvalidValue;
+        }
+        if (tile == 13) {
+            return launch_dma<2, 4, 8, 4, 3, 4, false, false, true>(a, st);
         }
         if (tile == 12) {
             return launch_dma<2, 4, 8, 4, 5, 3, false, false, true>(a, st);
@@ -1823,6 +1983,8 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 4, 8, 4, 4, 2>(a, st);  // 256 x 256, 8 waves, ping-pong memory / matrix phases
         case 12:
             return launch_dma<2, 4, 8, 4, 5, 3>(a, st);  // the same with A requested in whole 128-byte lines (160 KB of LDS)
+        case 13:
+            return launch_dma<2, 4, 8, 4, 3, 4>(a, st);  // as 12 with the B fragments loaded straight into registers (96 KB of LDS)
         default:
             break;
     }

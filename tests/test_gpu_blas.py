@@ -118,7 +118,7 @@ def test_mmm_all_outputs_device(torch_mod, oracle, M, K, N):
     assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
 
 
-@pytest.mark.parametrize("tile", [0, 2, 7, 10, 11, 12, 14])
+@pytest.mark.parametrize("tile", [0, 2, 7, 10, 11, 12, 13, 14])
 def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
     """Each GEMM kernel (general, register-staged tiles, LDS-DMA pipelines) is forced in turn on
     shapes with ragged M / N edges, one and many K tiles, and all four epilogues."""
@@ -127,7 +127,8 @@ def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
     try:
         capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
         for M, K, N in [(1, 64, 16), (130, 128, 70), (256, 64, 256), (300, 256, 200), (257, 192, 513),
-                        (512, 1024, 384), (100, 1040, 48), (260, 384, 300), (40, 896, 272)]:
+                        (512, 1024, 384), (100, 1040, 48), (260, 384, 300), (40, 896, 272), (512, 1536, 512),
+                        (300, 768, 600)]:
             say("variant", tile, M, K, N)
             A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
             W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
