@@ -3166,7 +3166,7 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
         // FullyConnected + GELU + dynamic quantisation in one launch: the accumulators stay in registers across a
         // grid-wide agreement on max|gelu|; the [T, F] fp32 tensor is never written. Should that agreement be abandoned
         // (the CUs were held by other work), the kernel leaves the activated values in f and sets the status word,
-        // and the two kernels behind it -- which otherwise return at once -- quantise them in two passes.
+        // and the one-workgroup kernel behind it -- which otherwise returns at once -- quantises them.
         uint32_t *status = (uint32_t *)(sc + 8);
         const uint32_t tiles = (T / 256) * (F / 256);
         GemmArgs g;
@@ -3193,8 +3193,7 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
         if (he != hipSuccess) {
             return fail(UNKNOWN, "launch_gemm_u8s8 (GELU epilogue)", he);
         }
-        HIP_TRY(launch_absmax_f32(f, T * F, ws3, st, true, status));
-        HIP_TRY(launch_quantize_f32(f, T * F, xq2, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 0, status));
+        HIP_TRY(launch_quantize_f32_standby(f, T * F, xq2, sc + 3, status, st));
     } else {
         HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
         // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads
