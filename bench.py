@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool", "lstm"],
+    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool", "lstm", "deconv", "depthwise", "ptq"],
                     help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
@@ -452,6 +452,54 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         both("concat_i8_rescale_channels", 4 * half,
              lambda i: host_pool.concat([xs[i][:half], xs[i][half:]], [d_in, d_in], 1, d_out, [9.0, 6.5], out=cat[i]),
              "2 x (32 x 128 x 56 x 56) -> 32 x 256 x 56 x 56, one input rescaled by 6.5 / 9, the other copied")
+    # -- int8 deconvolution (decoder-style upsampling layer), depthwise convolution, weight-storage converters
+    if want("deconv"):
+        from bolt_amd import host_deconv
+        n, ic, ih, iw, oc, fh, st_, pd = 16, 64, 28, 28, 64, 4, 2, 1
+        xq = torch.randint(1, 256, (n * ic * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
+        Wd = torch.randint(-127, 128, (ic, oc, fh, fh), dtype=torch.int8, device=dev, generator=g)
+        bd_ = torch.randn(oc, device=dev, generator=g) * 0.1
+        pd_ = host_deconv.deconv_param_spec(oc, fh, fh, st_, st_, pd, pd, pd, pd)
+        dtmp = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        for odt, nm, tdt in ((DT_U8_Q, "u8_dynamic_scale", torch.uint8), (DT_F32, "f32", torch.float32)):
+            idesc, fdesc, odesc, alg = host_deconv.plan(xq, DF_NCHWC16, n, ic, ih, iw, oc, fh, fh, pd_, odt)
+            dblob, dftm, _ = host_deconv.transform_filter(Wd, fdesc, pd_, alg)
+            oh = fh + st_ * (ih - 1) - 2 * pd
+            dout = torch.empty(n * oc * oh * oh, dtype=tdt, device=dev)
+            t = timed(lambda: host_deconv.deconvolution(xq, idesc, dblob, dftm, pd_, alg, bd_, [40.0, -1.0, 80.0], True, odesc,
+                                                        tmp=dtmp, out=dout), 20)
+            ops = 2.0 * n * ih * iw * ic * oc * fh * fh
+            res["deconv_4x4_s2_" + nm] = {"config": "16 x 64 x 28 x 28 -> 64 channels, 56 x 56, 4 x 4 kernel, stride 2, pad 1, ReLU (POINTWISE route)",
+                                           "ms": t, "tops": ops / t / 1e9,
+                                           "algorithmic_bytes": n * ic * ih * iw + ic * oc * fh * fh + n * oc * oh * oh * (1 if odt == DT_U8_Q else 4)}
+    if want("depthwise"):
+        n, c, ih, iw = 32, 256, 58, 58
+        xq = torch.randint(1, 256, (n * c * ih * iw,), dtype=torch.uint8, device=dev, generator=g)
+        Ww = torch.randint(-127, 128, (c, 3, 3), dtype=torch.int8, device=dev, generator=g)
+        bw = torch.randn(c, device=dev, generator=g) * 0.1
+        wblob, wftm = host_conv.depthwise_transform_filter(Ww, c, 3, 3)
+        wout = torch.empty(n * c * 56 * 56, dtype=torch.int32, device=dev)
+        t = timed(lambda: host_conv.depthwise_convolution_i32(xq, n, c, ih, iw, wblob, wftm, 3, 3, 1, bw, [40.0, -1.0, 80.0], True,
+                                                              out=wout), 20)
+        byt = n * c * (ih * iw + 4 * 56 * 56)
+        res["depthwise_3x3_i32"] = {"config": "32 x 256 x 58 x 58 -> 56 x 56, 3 x 3, stride 1, no padding, ReLU, int32 result",
+                                    "ms": t, "algorithmic_bytes": byt, "gbps": byt / t / 1e6, "frac_hbm_peak": byt / t / 1e6 / 8000.0}
+    if want("ptq"):
+        nW = 3072 * 768
+        Wf = torch.randn(nW, device=dev, generator=g) * 0.02
+        q8 = torch.empty(nW, dtype=torch.int8, device=dev)
+        back = torch.empty(nW, dtype=torch.float32, device=dev)
+        sc = (C.c_float * 1)(-1.0)
+
+        def conv8():
+            sc[0] = -1.0
+            capi.check(L.ws_datatype_converter_int8_gfx950(Wf.data_ptr(), q8.data_ptr(), nW, sc, capi.AMD_GFX950_DEVICE), "ws8")
+        t = timed(conv8, 20)
+        t2 = timed(lambda: capi.check(L.dequantize_int8_weight_gfx950(nW, sc[0], q8.data_ptr(), back.data_ptr(),
+                                                                      capi.AMD_GFX950_DEVICE), "dq8"), 20)
+        res["ws_convert_int8_3072x768"] = {"ms": t, "algorithmic_bytes": nW * 9, "gbps": nW * 9 / t / 1e6,
+                                           "note": "fp32 -> s8 weight storage with the tensor's own scale returned to the host (two reads, one write)"}
+        res["dequantize_int8_weight_3072x768"] = {"ms": t2, "algorithmic_bytes": nW * 5, "gbps": nW * 5 / t2 / 1e6}
     # -- int8 LSTM cell at the decode shape: 256 rows, x 2048 + h 2048 -> 4 x 2048 gates (the headline GEMV, N = 8192,
     #    K = 4096, inside its caller: per-row quantisation, one batched GEMV launch, gates and state update)
     if want("lstm"):

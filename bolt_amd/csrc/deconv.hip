@@ -119,18 +119,18 @@ template <int MODE>
 __global__ __launch_bounds__(256) void deconv_gather_kernel(DeconvArgs a)
 {
     __shared__ int red[4];
+    // blockIdx.x = plane * chunks + chunk: the plane (image, 16-channel block) comes from one scalar division per
+    // workgroup, the pixel from one 32-bit division per thread
     const uint32_t OB = a.oc / 16;
-    const uint64_t total = (uint64_t)a.n * OB * a.oh * a.ow * 4;
-    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint32_t opix = a.oh * a.ow, chunks = (opix + 63) / 64;
+    const uint32_t plane = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+    const uint32_t pix = chunk * 64 + (threadIdx.x >> 2);
     int m = 0;
-    if (id < total) {
-        const uint32_t q = (uint32_t)(id & 3);
-        uint64_t t = id >> 2;
-        const uint32_t ow = (uint32_t)(t % a.ow);
-        t /= a.ow;
-        const uint32_t oh = (uint32_t)(t % a.oh);
-        t /= a.oh;
-        const uint32_t ob = (uint32_t)(t % OB), n = (uint32_t)(t / OB);
+    if (pix < opix) {
+        const uint32_t q = threadIdx.x & 3;
+        const uint32_t oh = pix / a.ow, ow = pix % a.ow;
+        const uint32_t ob = plane % OB, n = plane / OB;
+        const size_t id = ((size_t)plane * opix + pix) * 4 + q;  // the output is [plane][pixel][16]
         const uint32_t o0 = ob * 16 + q * 4;
         const uint32_t planes = a.fh * a.fw * OB;
         // kh with 0 <= oh + pt - kh * sh < fh, inside the image
@@ -239,14 +239,15 @@ __global__ __launch_bounds__(256) void deconv_gather_kernel(DeconvArgs a)
 
 hipError_t launch_deconv_gather(const DeconvArgs &a, hipStream_t st)
 {
-    const uint64_t threads = (uint64_t)a.n * (a.oc / 16) * a.oh * a.ow * 4;
-    if (threads == 0) {
+    const uint64_t planes = (uint64_t)a.n * (a.oc / 16), chunks = ((uint64_t)a.oh * a.ow + 63) / 64;
+    if (planes == 0 || chunks == 0) {
         return hipSuccess;
     }
-    if (a.oc % 16 || a.ih == 0 || a.iw == 0 || a.sh == 0 || a.sw == 0 || (threads + 255) / 256 > 0x7fffffffull) {
+    if (a.oc % 16 || a.ih == 0 || a.iw == 0 || a.sh == 0 || a.sw == 0 || planes * chunks > 0x7fffffffull ||
+        (uint64_t)a.oh * a.ow > 0x3fffffffull) {
         return hipErrorInvalidValue;
     }
-    const dim3 grid((uint32_t)((threads + 255) / 256)), block(256);
+    const dim3 grid((uint32_t)(planes * chunks)), block(256);
     switch (a.mode) {
         case DECONV_I32:
             hipLaunchKernelGGL((deconv_gather_kernel<DECONV_I32>), grid, block, 0, st, a);

@@ -136,7 +136,7 @@ def depthwise_transform_filter(filt_chw, c, fh, fw):
     return blob, ftm
 
 
-def depthwise_convolution_i32(x, n, c, ih, iw, blob, ftm, fh, fw, stride, bias, scale, relu, pad=0):
+def depthwise_convolution_i32(x, n, c, ih, iw, blob, ftm, fh, fw, stride, bias, scale, relu, pad=0, out=None):
     """x: u8 NCHWC16. Returns int32 NCHWC16; scale = [sI, sO, sF] (sO written)."""
     arch = arch_of(x)
     p = conv_param_spec(c, fh, fw, stride, pad, 1, group=c)
@@ -144,7 +144,9 @@ def depthwise_convolution_i32(x, n, c, ih, iw, blob, ftm, fh, fw, stride, bias, 
     idesc = tensor4df(DT_U8_Q, DF_NCHWC16, n, c, ih, iw)
     odesc = tensor4df(DT_I32, DF_NCHWC16, n, c, oh, ow)
     count = n * c * oh * ow
-    if _is_torch(x):
+    if out is not None:
+        pass
+    elif _is_torch(x):
         import torch
         out = torch.zeros(count, dtype=torch.int32, device=x.device)
     else:
