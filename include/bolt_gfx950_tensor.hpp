@@ -5,7 +5,7 @@
 // compute/tensor/include/tensor_computing.h and unwraps its Tensors exactly as that function does
 // (get_ptr_from_tensor, common/memory/include/tensor_auxiliary.h:26-37; compute/tensor/src/quantize.cpp:19-34,
 // dequantize.cpp:25-49, fully_connected.cpp:107-159,307-498, matmul.cpp:203-300,302-576,
-// convolution.cpp:28-470), then calls the `_gfx950` twin. A dispatcher branch
+// convolution.cpp:28-470, deconvolution.cpp:23-279), then calls the `_gfx950` twin. A dispatcher branch
 //     } else if (IS_GFX950(arch)) { ret = bolt_gfx950::fully_connected(in, filter, bias, tmp, out, archInfo); }
 // in those reference functions is all the operator classes (FullyConnectedCPU, ConvolutionCPU, MatMulCPU,
 // QuantizeLinearCPU) need: they keep their call order bytes -> transform -> tmp bytes -> run.
@@ -206,6 +206,67 @@ inline EE convolution(std::vector<Tensor> inputTensors, Tensor filterTensor, Con
     return convolution_gfx950(inputTensors[0].get_desc(), ptr_of(inputTensors[0]), eltwiseInput, filterTensor.get_desc(),
         ptr_of(filterTensor), convParamSpec, algorithm, biasTensor.get_desc(), ptr_of(biasTensor), tmpTensors[0].bytes(),
         ptr_of(tmpTensors[0]), outputTensor.get_desc(), ptr_of(outputTensor), (F32 *)scale, activationDesc, archInfo->arch);
+}
+
+// ---- int8 deconvolution (deconvolution.cpp:23-279) ---------------------------------------------------------------
+inline EE deconvolution_infer_output_size(Tensor *inputTensor, Tensor filterTensor, ConvolutionParamSpec convParamSpec,
+    Tensor *outputTensor, DataType targetDataType, ArchInfo_t archInfo)
+{
+    TensorDesc outputDesc = outputTensor->get_desc();
+    EE ret = deconvolution_infer_output_size_gfx950(
+        inputTensor->get_desc(), filterTensor.get_desc(), convParamSpec, &outputDesc, targetDataType, archInfo->arch);
+    if (ret == SUCCESS) {
+        outputTensor->resize(outputDesc);
+    }
+    return ret;
+}
+
+// activationDesc does not take part in the choice on x86 either (cpu/deconvolution.cpp:23-55)
+inline EE deconvolution_infer_forward_algorithm(Tensor inputTensor, Tensor filterTensor, Tensor outputTensor,
+    ConvolutionParamSpec convParamSpec, ConvolutionPolicy policy, ConvolutionForwardAlgorithm *algorithm,
+    DataType targetDataType, ActivationParamSpec activationDesc, ArchInfo_t archInfo)
+{
+    (void)activationDesc;
+    return deconvolution_infer_forward_algorithm_gfx950(inputTensor.get_desc(), filterTensor.get_desc(),
+        outputTensor.get_desc(), convParamSpec, policy, algorithm, targetDataType, archInfo->arch);
+}
+
+inline EE deconvolution_transform_filter_bytes(Tensor filterTensor, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, void *bytes, ArchInfo_t archInfo)
+{
+    return deconvolution_transform_filter_bytes_gfx950(
+        filterTensor.get_desc(), convParamSpec, algorithm, (U32 *)bytes, archInfo->arch);
+}
+
+inline EE deconvolution_transform_filter(Tensor filterTensor, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, Tensor tmpTensor, Tensor *ftmTensor, ArchInfo_t archInfo)
+{
+    (void)tmpTensor;
+    TensorDesc ftmDesc = ftmTensor->get_desc();
+    EE ret = deconvolution_transform_filter_gfx950(filterTensor.get_desc(), ptr_of(filterTensor), convParamSpec, algorithm,
+        &ftmDesc, ptr_of(*ftmTensor), archInfo->arch);
+    if (ret == SUCCESS) {
+        ftmTensor->resize(ftmDesc);
+    }
+    return ret;
+}
+
+inline EE deconvolution_infer_forward_tmp_bytes(Tensor inputTensor, Tensor filterTensor, Tensor outputTensor,
+    ConvolutionParamSpec convParamSpec, ConvolutionForwardAlgorithm algorithm, U32 *bytes, ArchInfo_t archInfo)
+{
+    return deconvolution_infer_forward_tmp_bytes_gfx950(inputTensor.get_desc(), filterTensor.get_desc(),
+        outputTensor.get_desc(), convParamSpec, algorithm, bytes, archInfo->arch);
+}
+
+// scale: host F32[3] = {input scale, filter scale, output scale}, read and rewritten as on x86 (DeconvolutionCPU::run,
+// deconvolution_cpu.hpp:65-84); the scale descriptor is the filter's, as deconvolution.cpp:255 passes it
+inline EE deconvolution(Tensor inputTensor, Tensor filterTensor, ConvolutionParamSpec convParamSpec,
+    ConvolutionForwardAlgorithm algorithm, void *scale, Tensor biasTensor, Tensor tmpTensor, Tensor outputTensor,
+    ActivationParamSpec activationDesc, ArchInfo_t archInfo)
+{
+    return deconvolution_gfx950(inputTensor.get_desc(), ptr_of(inputTensor), filterTensor.get_desc(), ptr_of(filterTensor),
+        convParamSpec, algorithm, filterTensor.get_desc(), scale, biasTensor.get_desc(), ptr_of(biasTensor), tmpTensor.bytes(),
+        ptr_of(tmpTensor), outputTensor.get_desc(), ptr_of(outputTensor), activationDesc, archInfo->arch);
 }
 
 }  // namespace bolt_gfx950

@@ -4,7 +4,8 @@
 //      DEVICE memory between the three operators (Arch AMD_GFX950_DEVICE: only the layer input goes up and only the final
 //      output comes down), and the same chain with host pointers (AMD_GFX950);
 //   2. an int8 3x3 convolution with ReLU and a u8 result through the six convolution_* calls;
-//   3. a batched int8 matmul.
+//   3. an int8 4x4 stride-2 deconvolution with ReLU and a u8 result through the six deconvolution_* calls;
+//   4. a batched int8 matmul.
 // Built by `make -C oracle glue` where the reference checkout is present (this file includes Bolt's headers); the
 // binary lands in oracle/_ref/ and tests/test_gpu_glue.py runs it on the GPU box. Exit code 0 = everything equal.
 #include <cmath>
@@ -219,6 +220,78 @@ static int conv_u8()
     return bad | same("int8 3x3 convolution, ReLU, u8 out, through the six convolution_* calls", outs[1], outs[0]);
 }
 
+static int deconv_u8()
+{
+    const U32 n = 2, ic = 32, ih = 9, iw = 7, oc = 32, fh = 4, fw = 4;
+    ConvolutionParamSpec p = createConvolutionParamSpec(1, 1, fh, fw, 1, 2, 2, 0, 0, 1, 1, 1, 1, 1, 1, 1, oc, CONVOLUTION_DECONVOLUTION);
+    ActivationParamSpec act;
+    act.mode = ACTIVATION_RELU;
+    Tensor in = host_tensor(tensor4df(DT_U8_Q, DF_NCHW, n, ic, ih, iw));
+    for (U32 i = 0; i < in.bytes(); ++i) {
+        ((U8 *)hp(in))[i] = (U8)(128 + (int)(rnd() % 200) - 100);
+    }
+    Tensor filter = host_tensor(tensor4df(DT_I8, DF_NCHW, ic, oc, fh, fw));
+    for (U32 i = 0; i < filter.bytes(); ++i) {
+        ((INT8 *)hp(filter))[i] = (INT8)((int)(rnd() % 255) - 127);
+    }
+    Tensor bias = host_tensor(tensor1d(DT_F32, oc));
+    for (U32 i = 0; i < oc; ++i) {
+        ((F32 *)hp(bias))[i] = 0.1f * gauss();
+    }
+    Tensor outs[2];
+    F32 got[2][3];
+    for (int which = 0; which < 2; ++which) {
+        const bool gpu = which == 1;
+        ArchInfo_t a = gpu ? &g_host : &g_x86;
+        Tensor out, tmp0;
+        ConvolutionForwardAlgorithm alg = CONVOLUTION_ALGORITHM_NULL;
+        U32 fb = 0, tb = 0;
+        if (gpu) {
+            CHECK_STATUS(bolt_gfx950::deconvolution_infer_output_size(&in, filter, p, &out, DT_U8_Q, a));
+            CHECK_STATUS(bolt_gfx950::deconvolution_infer_forward_algorithm(in, filter, out, p, CONVOLUTION_FASTEST, &alg, DT_U8_Q, act, a));
+            CHECK_STATUS(bolt_gfx950::deconvolution_transform_filter_bytes(filter, p, alg, &fb, a));
+        } else {
+            CHECK_STATUS(deconvolution_infer_output_size(&in, filter, p, &out, DT_U8_Q, a));
+            CHECK_STATUS(deconvolution_infer_forward_algorithm(in, filter, out, p, CONVOLUTION_FASTEST, &alg, DT_U8_Q, act, a));
+            CHECK_STATUS(deconvolution_transform_filter_bytes(filter, p, alg, &fb, a));
+        }
+        out.alloc();
+        Tensor ftm = host_tensor(tensor1d(DT_U8, fb + 64));
+        if (gpu) {
+            CHECK_STATUS(bolt_gfx950::deconvolution_transform_filter(filter, p, alg, tmp0, &ftm, a));
+            CHECK_STATUS(bolt_gfx950::deconvolution_infer_forward_tmp_bytes(in, ftm, out, p, alg, &tb, a));
+        } else {
+            CHECK_STATUS(deconvolution_transform_filter(filter, p, alg, tmp0, &ftm, a));
+            CHECK_STATUS(deconvolution_infer_forward_tmp_bytes(in, ftm, out, p, alg, &tb, a));
+            // the reference's figure leaves out what the product inside needs (cpu/deconvolution.cpp:188-250); the engine
+            // covers that by sharing one tmp sized as the maximum over all operators
+            tb += n * ih * iw * oc * fh * fw * 8 + (1u << 20);
+        }
+        Tensor tmp = host_tensor(tensor1d(DT_U8, tb));
+        memset(hp(tmp), 0, tb);
+        F32 scales[3] = {31.5f, 80.0f, -1.0f};
+        if (gpu) {
+            CHECK_STATUS(bolt_gfx950::deconvolution(in, ftm, p, alg, scales, bias, tmp, out, act, a));
+        } else {
+            CHECK_STATUS(deconvolution(in, ftm, p, alg, scales, bias, tmp, out, act, a));
+        }
+        outs[which] = out;
+        memcpy(got[which], scales, sizeof(scales));
+    }
+    int bad = 0;
+    TensorDesc d0 = outs[0].get_desc(), d1 = outs[1].get_desc();
+    if (d0.dt != d1.dt || d0.df != d1.df || d0.nDims != d1.nDims || memcmp(d0.dims, d1.dims, d0.nDims * sizeof(U32)) != 0) {
+        printf("MISMATCH: deconvolution output descs\n");
+        bad = 1;
+    }
+    if (memcmp(got[0], got[1], sizeof(got[0])) != 0) {
+        printf("MISMATCH: deconvolution scales %g %g %g / %g %g %g\n", got[1][0], got[1][1], got[1][2], got[0][0], got[0][1],
+            got[0][2]);
+        bad = 1;
+    }
+    return bad | same("int8 4x4 stride-2 deconvolution, ReLU, u8 out, through the six deconvolution_* calls", outs[1], outs[0]);
+}
+
 static int batched_matmul()
 {
     TensorDesc ad = tensor4df(DT_F32, DF_NCHW, 2, 3, 16, 64), bd = tensor4df(DT_F32, DF_NCHW, 2, 3, 24, 64),
@@ -261,6 +334,7 @@ int main()
     }
     int bad = chain_quantize_fc_fc();
     bad |= conv_u8();
+    bad |= deconv_u8();
     bad |= batched_matmul();
     printf(bad ? "glue FAILED\n" : "glue OK\n");
     return bad;
