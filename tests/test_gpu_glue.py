@@ -20,7 +20,7 @@ def test_tensor_glue_matches_the_reference_operators():
     r = subprocess.run([EXE], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "glue OK" in r.stdout and r.stdout.count("equal:") == 4
+    assert "glue OK" in r.stdout and r.stdout.count("equal:") == 5
 
 
 @pytest.mark.skipif(not os.path.isdir("/root/reference/compute/tensor"), reason="no reference checkout here")
