@@ -14,6 +14,7 @@
 // so only the lane <-> row/column association matters; the packed B layout (layout.h) hands every
 // lane its 16 bytes with one 128-bit load.
 #include "device_common.h"
+#include <type_traits>
 #include "kernels.h"
 #include "layout.h"
 
@@ -177,7 +178,7 @@ __device__ __forceinline__ void store_c16(V *p, V v)
 
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0)
+    uint32_t wave, uint32_t m0, uint32_t n0, const uint32_t (*pre_base)[4] = nullptr)
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -211,7 +212,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const bool ok = FULL || (n + c < a.N);
-            base[y][c] = ok ? column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c) : 0u;
+            // pre_base: the caller formed these terms ahead of its K loop, while it was waiting for memory anyway
+            base[y][c] = pre_base ? pre_base[y][c] : (ok ? column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c) : 0u);
             qs[y][c] = 1.0f;
             bs[y][c] = 0.0f;
             if (MODE == EPI_F32_CH && ok) {
@@ -613,7 +615,7 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
 
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0)
+    uint32_t wave, uint32_t m0, uint32_t n0, const uint32_t (*pre_base)[4] = nullptr)
 {
     const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
     const bool cin = !CONV && a.add_cin && MODE != EPI_U8;
@@ -635,28 +637,28 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
         }
     }
     if (full && !cin) {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0, pre_base);
     } else if (full && MODE != EPI_U8 && !CONV) {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1>(a, acc, smem, lane, wave, m0, n0);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1>(a, acc, smem, lane, wave, m0, n0, pre_base);
     } else {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2>(a, acc, smem, lane, wave, m0, n0);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2>(a, acc, smem, lane, wave, m0, n0, pre_base);
     }
 }
 
 template <int WM, int WN, int TM, int TN, bool CONV = false>
 __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes)
+    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes, const uint32_t (*pre_base)[4] = nullptr)
 {
     (void)lds_bytes;
     if (CONV) {
         if (a.epi.mode == EPI_I32) {
-            epilogue_mode<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_U8) {
-            epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_F32_CH) {
-            epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else {
-            epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         }
         return;
     }
@@ -1516,14 +1518,14 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
 // neighbouring channel blocks (NCHWC8); taps that fall outside the image, and the chunks that pad K to 64, read a
 // constant block of 0x80 instead, and every fragment is re-biased (^ 0x80) before use, which turns those into the
 // zeros the padded image holds.
-__device__ const uint8_t kConvPad128[16] = {128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128};
+__device__ __attribute__((aligned(16))) const uint8_t kConvPad128[16] = {128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128, 128};
 
 template <int TM, bool DIRECT>
 __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ int sync_lds[18];  // the one-pass u8 form's grid-wide maximum (the waves read the panel at their own pace)
-    constexpr int P = 3;  // K tiles of A in flight per wave
+    constexpr int P = 5;  // K tiles of A in flight per wave
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t i = lane & 15, g = lane >> 4;
@@ -1540,26 +1542,73 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(smem + f * 1024), 16, 0, 0);
     }
 
+    // The loads below name the global address space: a pointer chosen between the image and the constant block would
+    // otherwise be loaded from as a flat pointer, and flat loads cannot be counted in order, so every K tile would
+    // wait for all the tiles requested after it as well.
+    typedef const __attribute__((address_space(1))) uint8_t *gbytes_t;
+    typedef const __attribute__((address_space(1))) v4i *gv4i_t;
+    typedef const __attribute__((address_space(1))) v2i *gv2i_t;
+    const gbytes_t gA = (gbytes_t)a.A, gPad = (gbytes_t)kConvPad128;
     const uint32_t cpc = a.conv.ICp / 16;  // 16-channel planes of the image
     const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+    const uint32_t ic_bytes = DIRECT ? a.conv.in_c : 16;  // bytes per pixel inside a channel block
+    const uint32_t plane8 = a.conv.H * a.conv.W * 8;
+    // ---- per-pixel terms ----------------------------------------------------------------------------------
     uint32_t off[TM];   // padded image: byte offset of the pixel's receptive field; DIRECT: of pixel (iy0, ix0), may be "negative"
     int32_t iy0[TM], ix0[TM];  // DIRECT: input row / column of tap (0, 0)
-    const uint32_t ic_bytes = DIRECT ? a.conv.in_c : 16;  // bytes per pixel inside a channel block
+    auto pixel_terms = [&]() {
 #pragma unroll
-    for (int x = 0; x < TM; ++x) {
-        uint32_t row = m0 + (wave * TM + x) * 16 + i;
-        row = row < a.M ? row : a.M - 1;
-        const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
-        const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
-        if (DIRECT) {
-            iy0[x] = (int32_t)(oy * a.conv.sh) - (int32_t)a.conv.pt;
-            ix0[x] = (int32_t)(ox * a.conv.sw) - (int32_t)a.conv.pl;
-            off[x] = img * a.conv.IC * a.conv.H * a.conv.W +
-                (uint32_t)(iy0[x] * (int32_t)a.conv.W + ix0[x]) * ic_bytes;  // wraps for border pixels; used only when in range
-        } else {
-            off[x] = ((img * cpc * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
+        for (int x = 0; x < TM; ++x) {
+            uint32_t row = m0 + (wave * TM + x) * 16 + i;
+            row = row < a.M ? row : a.M - 1;
+            const uint32_t img = row / a.conv.OHW, r = row % a.conv.OHW;
+            const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
+            if (DIRECT) {
+                iy0[x] = (int32_t)(oy * a.conv.sh) - (int32_t)a.conv.pt;
+                ix0[x] = (int32_t)(ox * a.conv.sw) - (int32_t)a.conv.pl;
+                off[x] = img * a.conv.IC * a.conv.H * a.conv.W +
+                    (uint32_t)(iy0[x] * (int32_t)a.conv.W + ix0[x]) * ic_bytes;  // wraps for border pixels; used only when in range
+            } else {
+                off[x] = ((img * cpc * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
+            }
         }
-    }
+    };
+
+    // ---- per-column terms of the epilogue (offsetC - compensation, with the bias folded in) -------------------
+    // Formed ahead of the K loop, while the first loads are on their way, instead of on the critical path behind it.
+    // All loads first, none behind a branch (columns past N read column N - 1 and are dropped; the vector that the
+    // mode does not use is read from the other one's address), so that they are in flight together.
+    uint32_t pre_base[4][4];
+    int32_t pb_c[4][4], pb_o[4][4];
+    float pb_f[4][4];
+    const bool fold = a.fold_bias != nullptr;
+    auto pre_base_request = [&]() {
+        const int32_t *obp = fold ? a.comp : a.ob;
+        const float *fbp = fold ? a.fold_bias : (const float *)a.comp;
+#pragma unroll
+        for (int y = 0; y < 4; ++y) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t n = y * 16 + 4 * g + c, nc = n < a.N ? n : a.N - 1;
+                pb_c[y][c] = a.comp[nc];
+                pb_o[y][c] = obp[nc];
+                pb_f[y][c] = fbp[nc];
+            }
+        }
+    };
+    auto pre_base_form = [&]() {
+#pragma unroll
+        for (int y = 0; y < 4; ++y) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t n = y * 16 + 4 * g + c;
+                const float p_ = pb_f[y][c] * a.fold_scale;  // as column_base() forms it
+                const int32_t o_ = fold ? (int32_t)(round((double)p_) + (double)pb_c[y][c]) : pb_o[y][c];
+                pre_base[y][c] = (n < a.N) ? (uint32_t)o_ - (uint32_t)pb_c[y][c] : 0u;
+            }
+        }
+    };
+
     // this lane's K-group g covers 16-channel chunk 4 * tile + g; its (kh, kw, c16) is stepped in registers
     uint32_t c16 = g % cpc, kw = (g / cpc) % a.conv.fw, kh = (g / cpc) / a.conv.fw, at = 0;  // at: tile the walk points to
     auto tap_offset = [&]() -> uint32_t {
@@ -1568,78 +1617,93 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
         }
         return (kh < a.conv.fh) ? ((c16 * a.conv.Hp + kh * a.conv.dh) * a.conv.Wp + kw * a.conv.dw) * 16 : 0u;
     };
-    // one fragment: the lane's 16 channels of pixel x at the current tap
-    auto gather = [&](int x, uint32_t o) -> v4i {
-        if (!DIRECT) {
-            return *(const v4i *)(a.A + off[x] + o);
-        }
-        const uint32_t iy = (uint32_t)(iy0[x] + (int32_t)(kh * a.conv.dh)), ix = (uint32_t)(ix0[x] + (int32_t)(kw * a.conv.dw));
-        const bool ok = kh < a.conv.fh && iy < a.conv.H && ix < a.conv.W;
-        const uint8_t *p = ok ? a.A + (uint32_t)(off[x] + o) : kConvPad128;
-        if (a.conv.in_c == 16) {
-            return *(const v4i *)p;
-        }
-        const uint8_t *p2 = ok ? p + a.conv.H * a.conv.W * 8 : kConvPad128;  // the next block of 8 channels
-        const v2i lo = *(const v2i *)p, hi = *(const v2i *)p2;
-        return (v4i){lo.x, lo.y, hi.x, hi.y};
-    };
     auto advance = [&]() {
-        if (at + 1 < ksteps) {  // past the last tile the walk stays put: the refetch is never used
-            ++at;
-            c16 += 4;
+        const uint32_t mv = (at + 1 < ksteps) ? 1u : 0u;  // past the last tile the walk stays put: the refetch is never used
+        at += mv;
+        c16 += 4 * mv;
 #pragma unroll
-            for (int w_ = 0; w_ < 4; ++w_) {
-                const bool wr_ = c16 >= cpc;
-                c16 -= wr_ ? cpc : 0u;
-                kw += wr_ ? 1u : 0u;
-                const bool w2_ = kw >= a.conv.fw;
-                kw = w2_ ? 0u : kw;
-                kh += w2_ ? 1u : 0u;
-            }
+        for (int w_ = 0; w_ < 4; ++w_) {
+            const bool wr_ = c16 >= cpc;
+            c16 -= wr_ ? cpc : 0u;
+            kw += wr_ ? 1u : 0u;
+            const bool w2_ = kw >= a.conv.fw;
+            kw = w2_ ? 0u : kw;
+            kh += w2_ ? 1u : 0u;
         }
     };
 
-    v4i fa[P][TM];
-#pragma unroll
-    for (int s = 0; s < P; ++s) {
-        const uint32_t o = tap_offset();
-#pragma unroll
-        for (int x = 0; x < TM; ++x) {
-            fa[s][x] = gather(x, o);
-        }
-        advance();
-    }
     v4i acc[TM][4];
+    // The rest once per input layout (IN16: a pixel's 16 channels are one 16-byte access; else two 8-byte accesses to
+    // neighbouring channel blocks) so that no branch separates the loads of a tile from each other. The main loop takes
+    // P tiles per round with no condition inside: then the compiler counts the loads still in flight behind a tile's
+    // own instead of waiting for all of them. Tiles past the end are requested again from the last tap and dropped.
+    auto k_loop = [&](auto in16_tag) {
+        constexpr bool IN16 = decltype(in16_tag)::value;
+        // one fragment: the lane's 16 channels of pixel x at the current tap
+        auto gather = [&](int x, uint32_t o) -> v4i {
+            if (!DIRECT) {
+                return *(gv4i_t)(gA + off[x] + o);
+            }
+            const uint32_t iy = (uint32_t)(iy0[x] + (int32_t)(kh * a.conv.dh)), ix = (uint32_t)(ix0[x] + (int32_t)(kw * a.conv.dw));
+            const bool ok = kh < a.conv.fh && iy < a.conv.H && ix < a.conv.W;
+            const gbytes_t p = ok ? gA + (uint32_t)(off[x] + o) : gPad;
+            if (IN16) {
+                return *(gv4i_t)p;
+            }
+            const gbytes_t p2 = ok ? p + plane8 : gPad;  // the next block of 8 channels
+            const v2i lo = *(gv2i_t)p, hi = *(gv2i_t)p2;
+            return (v4i){lo.x, lo.y, hi.x, hi.y};
+        };
+        v4i fa[P][TM];
+        auto first_tiles = [&]() {
 #pragma unroll
-    for (int x = 0; x < TM; ++x) {
-#pragma unroll
-        for (int y = 0; y < 4; ++y) {
-            acc[x][y] = (v4i){0, 0, 0, 0};
-        }
-    }
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the panel (and the first A tiles) have landed
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-
-    for (uint32_t t = 0; t < ksteps; t += P) {
-#pragma unroll
-        for (int u = 0; u < P; ++u) {
-            if (t + u < ksteps) {
-                const uint8_t *sB = smem + (size_t)(t + u) * 4096 + lane * 16;
-                v4i fb[4];
-#pragma unroll
-                for (int y = 0; y < 4; ++y) {
-                    fb[y] = *(const v4i *)(sB + y * 1024);
-                }
+            for (int s_ = 0; s_ < P; ++s_) {
+                const uint32_t o = tap_offset();
 #pragma unroll
                 for (int x = 0; x < TM; ++x) {
-                    const v4i fx = DIRECT ? (fa[u][x] ^ flip) : fa[u][x];
-#pragma unroll
-                    for (int y = 0; y < 4; ++y) {
-                        acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fx, acc[x][y], 0, 0, 0);
-                    }
+                    fa[s_][x] = gather(x, o);
                 }
+                advance();
+            }
+        };
+        // order: the A tiles first (the long pole), the epilogue's column terms behind them, their arithmetic while
+        // all of it is on its way
+        pixel_terms();
+        first_tiles();
+        pre_base_request();
+        pre_base_form();
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the panel (and the first A tiles) have landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+                acc[x][y] = (v4i){0, 0, 0, 0};
+            }
+        }
+        auto tile = [&](uint32_t t, int u) {
+            const uint8_t *sB = smem + (size_t)t * 4096 + lane * 16;
+            v4i fb[4];
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+                fb[y] = *(const v4i *)(sB + y * 1024);
+            }
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+                const v4i fx = DIRECT ? (fa[u][x] ^ flip) : fa[u][x];
+#pragma unroll
+                for (int y = 0; y < 4; ++y) {
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[y], fx, acc[x][y], 0, 0, 0);
+                }
+            }
+        };
+        uint32_t t = 0;
+        for (; t + P <= ksteps; t += P) {
+#pragma unroll
+            for (int u = 0; u < P; ++u) {
+                tile(t + u, u);
                 const uint32_t o = tap_offset();
 #pragma unroll
                 for (int x = 0; x < TM; ++x) {
@@ -1648,8 +1712,19 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
                 advance();
             }
         }
+#pragma unroll
+        for (int u = 0; u < P - 1; ++u) {  // what is left of K: its tiles were requested by the last full round
+            if (t + u < ksteps) {
+                tile(t + u, u);
+            }
+        }
+    };
+    if (a.conv.in_c == 16) {
+        k_loop(std::true_type{});
+    } else {
+        k_loop(std::false_type{});
     }
-    epilogue_panel<4, 1, TM, 4, true>(a, acc, (uint8_t *)sync_lds, lane, wave, m0, 0u, 0);
+    epilogue_panel<4, 1, TM, 4, true>(a, acc, (uint8_t *)sync_lds, lane, wave, m0, 0u, 0, pre_base);
 }
 
 // Skinny kernel for few rows (FullyConnected at small batch: M <= 64 per block, any N, K % 64 == 0).
@@ -1849,12 +1924,12 @@ hipError_t launch_conv_u8s8(const GemmArgs &a, hipStream_t st)
             }
             attr_set = true;
         }
-        const uint32_t lds = a.K * 64;
         const bool direct = a.conv.in_c != 0;
         const uint32_t grid = (g_conv_panel == 2) ? (a.M + 127) / 128 : (a.M + 255) / 256;
         if (a.sync.slots && (a.sync.blocks != grid || grid > conv_onepass_max_grid(a.K))) {
             return hipErrorInvalidValue;  // the one-pass form needs every workgroup resident at once
         }
+        const uint32_t lds = a.K * 64;
         if (g_conv_panel == 2) {
             if (direct) {
                 hipLaunchKernelGGL((conv_u8s8_panel_kernel<2, true>), dim3(grid), dim3(256), lds, st, a);
