@@ -149,6 +149,32 @@ __device__ __forceinline__ uint32_t column_base(const int32_t *ob, const int32_t
     return (uint32_t)ob[n] - (uint32_t)c;
 }
 
+// column_base() for NC columns n[0..NC-1] at once: every load first and none behind a branch (the vector that the
+// mode does not use is read from the other one's address), so that all of them are in flight together instead of each
+// costing its own trip to memory. Columns whose n is past N must be clamped by the caller (n < N always).
+template <int NC>
+__device__ __forceinline__ void column_bases(const int32_t *ob, const int32_t *comp, const float *fold_bias, float fold_scale,
+    const uint32_t (&n)[NC], uint32_t (&base)[NC])
+{
+    const bool fold = fold_bias != nullptr;
+    const int32_t *obp = fold ? comp : ob;
+    const float *fbp = fold ? fold_bias : (const float *)comp;
+    int32_t c[NC], o[NC];
+    float f[NC];
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+        c[k] = comp[n[k]];
+        o[k] = obp[n[k]];
+        f[k] = fbp[n[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+        const float p = f[k] * fold_scale;
+        const int32_t v = fold ? (int32_t)(round((double)p) + (double)c[k]) : o[k];
+        base[k] = (uint32_t)v - (uint32_t)c[k];
+    }
+}
+
 __device__ __forceinline__ float wave_reduce_sum(float v)
 {
 #pragma unroll

@@ -206,36 +206,56 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     uint32_t base[TN][4];
     float qs[TN][4], bs[TN][4];
     uint32_t cblk_off[TN], cblk_w[TN];
+    {
+        // every per-column term in one batch of loads, none behind a branch (a load per use would put a trip to memory
+        // into each column); columns past N read column N - 1 and are dropped. pre_base: the caller formed the
+        // offsets ahead of its K loop, while it was waiting for memory anyway.
+        uint32_t nn[TN * 4], flat[TN * 4];
+        float sw[TN * 4], bi[TN * 4];
+        const float *swp = (MODE == EPI_F32_CH) ? a.epi.scaleW : (const float *)a.comp;
+        const float *bip = (MODE == EPI_F32_CH && a.epi.bias) ? a.epi.bias : (const float *)a.comp;
 #pragma unroll
-    for (int y = 0; y < TN; ++y) {
-        const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+        for (int y = 0; y < TN; ++y) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const bool ok = FULL || (n + c < a.N);
-            // pre_base: the caller formed these terms ahead of its K loop, while it was waiting for memory anyway
-            base[y][c] = pre_base ? pre_base[y][c] : (ok ? column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c) : 0u);
-            qs[y][c] = 1.0f;
-            bs[y][c] = 0.0f;
-            if (MODE == EPI_F32_CH && ok) {
-                if (CONV) {
-                    // 1-bit convolution on the matrix cores: fma(S, scale[oc], bias[oc]), scale used as it is
-                    qs[y][c] = a.epi.scaleW[n + c];
-                    bs[y][c] = a.epi.bias[n + c];
-                } else {
-                    const float s = sI * a.epi.scaleW[n + c];
-                    qs[y][c] = 1.0f / s;
-                    bs[y][c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
-                }
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g + c;
+                nn[y * 4 + c] = (FULL || n < a.N) ? n : a.N - 1;
+                sw[y * 4 + c] = swp[nn[y * 4 + c]];
+                bi[y * 4 + c] = bip[nn[y * 4 + c]];
             }
         }
-        cblk_off[y] = 0;
-        cblk_w[y] = 1;
-        if (CONV) {
-            // output blocks of out_c channels per pixel (a trailing block may be narrower); 4 channels
-            // starting at a multiple of 4 never straddle a block
-            const uint32_t xc = a.conv.out_c, blk = n / xc;
-            cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
-            cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+        if (!pre_base) {
+            column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, a.fold_scale, nn, flat);
+        }
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const bool ok = FULL || (n + c < a.N);
+                base[y][c] = pre_base ? pre_base[y][c] : (ok ? flat[y * 4 + c] : 0u);
+                qs[y][c] = 1.0f;
+                bs[y][c] = 0.0f;
+                if (MODE == EPI_F32_CH && ok) {
+                    if (CONV) {
+                        // 1-bit convolution on the matrix cores: fma(S, scale[oc], bias[oc]), scale used as it is
+                        qs[y][c] = sw[y * 4 + c];
+                        bs[y][c] = bi[y * 4 + c];
+                    } else {
+                        qs[y][c] = 1.0f / (sI * sw[y * 4 + c]);
+                        bs[y][c] = a.epi.bias ? bi[y * 4 + c] : 0.0f;
+                    }
+                }
+            }
+            cblk_off[y] = 0;
+            cblk_w[y] = 1;
+            if (CONV) {
+                // output blocks of out_c channels per pixel (a trailing block may be narrower); 4 channels
+                // starting at a multiple of 4 never straddle a block
+                const uint32_t xc = a.conv.out_c, blk = n / xc;
+                cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
+                cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+            }
         }
     }
 
@@ -441,15 +461,21 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
     uint32_t base[4];
     float qs[4], bs[4];
     {
+        // every per-column term in one batch of loads (a load per use would put a trip to memory into each column)
+        const uint32_t nn[4] = {n, n + 1, n + 2, n + 3};
+        const float *swp = (MODE == EPI_F32_CH) ? a.epi.scaleW : (const float *)a.comp;
+        const float *bip = (MODE == EPI_F32_CH && a.epi.bias) ? a.epi.bias : (const float *)a.comp;
+        float sw[4], bi[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            base[c] = column_base(a.ob, a.comp, a.fold_bias, a.fold_scale, n + c);
-            qs[c] = 1.0f;
-            bs[c] = 0.0f;
-            if (MODE == EPI_F32_CH) {
-                qs[c] = 1.0f / (sI * a.epi.scaleW[n + c]);
-                bs[c] = a.epi.bias ? a.epi.bias[n + c] : 0.0f;
-            }
+            sw[c] = swp[nn[c]];
+            bi[c] = bip[nn[c]];
+        }
+        column_bases<4>(a.ob, a.comp, a.fold_bias, a.fold_scale, nn, base);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            qs[c] = (MODE == EPI_F32_CH) ? 1.0f / (sI * sw[c]) : 1.0f;
+            bs[c] = (MODE == EPI_F32_CH && a.epi.bias) ? bi[c] : 0.0f;
         }
     }
     v4i cin[2][4];
