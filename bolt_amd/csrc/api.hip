@@ -3165,8 +3165,8 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     if (g_encoder_fused && gemm_gelu_dyn_fits(T, F, H)) {
         // FullyConnected + GELU + dynamic quantisation in one launch: the accumulators stay in registers across a
         // grid-wide agreement on max|gelu|; the [T, F] fp32 tensor is never written. Should that agreement be abandoned
-        // (the CUs were held by other work), the kernel leaves the activated values in f and sets the status word,
-        // and the one-workgroup kernel behind it -- which otherwise returns at once -- quantises them.
+        // (the CUs were held by other work), the kernel leaves the activated values in f, sets the status word, and
+        // its last workgroup quantises them alone.
         uint32_t *status = (uint32_t *)(sc + 8);
         const uint32_t tiles = (T / 256) * (F / 256);
         GemmArgs g;
@@ -3193,7 +3193,6 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
         if (he != hipSuccess) {
             return fail(UNKNOWN, "launch_gemm_u8s8 (GELU epilogue)", he);
         }
-        HIP_TRY(launch_quantize_f32_standby(f, T * F, xq2, sc + 3, status, st));
     } else {
         HIP_TRY(gemm(xq, L.w1, F, H, sc + 2, L.s1, L.b1, f));
         // GELU: one pass takes max|gelu(f)| without writing anything, the quantiser applies the same gelu to what it reads

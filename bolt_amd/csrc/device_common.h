@@ -291,6 +291,7 @@ struct GridSync {
     uint32_t epoch = 0;        // this launch's tag
     uint32_t blocks = 0;       // workgroups in the launch (gridDim.x, <= kGridSyncMaxBlocks)
     uint32_t spin_limit = 0;   // polling rounds (about a microsecond each) before a waiting workgroup gives up
+    unsigned *done = nullptr;  // arrival counter for grid_last_arrival (a spare word of the area; zero between launches)
 };
 constexpr uint32_t kGridAbandoned = 0xffffffffu;  // never a maximum: those are non-negative floats' bits, ints >= 0 or INT32_MIN
 
@@ -381,6 +382,61 @@ __device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int
     }
     __syncthreads();
     return (uint32_t)lds[17];
+}
+
+
+// What a kernel does when grid_max_sync() was abandoned and it cannot leave the job to the host: every workgroup
+// first stores its partial result where a second pass can read it, then calls this (all threads); exactly one
+// workgroup -- the last to arrive -- gets true and does that second pass alone, the others return. No workgroup
+// waits for another, so it works whatever part of the grid is resident. The fences make the others' stores visible
+// to the one that continues. `lds`: the 18 ints grid_max_sync used.
+__device__ __forceinline__ bool grid_last_arrival(const GridSync &gs, int *lds)
+{
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned prev = __hip_atomic_fetch_add(gs.done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev + 1 == gs.blocks;
+        if (last) {
+            __hip_atomic_store(gs.done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch on the stream
+        }
+        lds[16] = last ? 1 : 0;
+    }
+    __syncthreads();
+    const bool last = lds[16] != 0;
+    if (last) {
+        __threadfence();
+    }
+    return last;
+}
+
+// Both passes of a dynamic fp32 -> u8 quantisation (scale 127 / max|x|, 1 for an all-zero tensor) by ONE workgroup of
+// whole waves (at most 16): the second pass of grid_last_arrival()'s survivor. `red`: 16 floats of LDS.
+__device__ __forceinline__ void quantize_f32_u8_alone(const float *x, uint32_t n, uint8_t *q, float *ds_out, float *red)
+{
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    float m = 0.0f;
+    for (uint32_t k = tid; k < n; k += nt) {
+        const float a_ = fabsf(x[k]);
+        m = (a_ > m) ? a_ : m;  // a NaN never replaces the running max (avx512/quantize.cpp:21-68)
+    }
+    m = wave_reduce_max(m);
+    __syncthreads();
+    if ((tid & 63) == 0) {
+        red[tid >> 6] = m;
+    }
+    __syncthreads();
+    m = red[0];
+    for (uint32_t w = 1; w < (nt >> 6); ++w) {
+        m = red[w] > m ? red[w] : m;
+    }
+    const float s = (m == 0.0f) ? 1.0f : 127.0f / m;
+    if (tid == 0 && ds_out) {
+        *ds_out = s;
+    }
+    for (uint32_t k = tid; k < n; k += nt) {
+        q[k] = (uint8_t)q_u8(x[k], s);
+    }
 }
 
 }  // namespace bg

@@ -542,8 +542,9 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
 //   max|y| over the whole result through grid_max_sync               (every tile's workgroup is resident)
 //   u8 = q_u8(y, max(0, 127 / max|y|)), scale published through dscale_out
 // -- the arithmetic, element for element, of the per-channel fp32 epilogue, gelu_f32_kernel's maximum and
-// quantize_f32_kernel<u8, gelu>. If the grid-wide wait is abandoned nothing is quantised: every workgroup stores its
-// y as fp32 into C32 and status becomes 1, on which the two conditional kernels behind this one do the two passes.
+// quantize_f32_kernel<u8, gelu>. If the grid-wide wait is abandoned every workgroup stores its y as fp32 into C32,
+// status becomes 1, and the last workgroup to finish quantises all of C32 by itself (grid_last_arrival): slow, but it
+// needs neither another launch nor the host, and the wait only expires when the CUs were held by other work.
 // Full 256 x 256 tiles only (the launcher checks).
 template <int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
@@ -605,6 +606,10 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
                 const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
                 *(v4i *)(a.C32 + (size_t)m * a.N + n) = acc[x][y];
             }
+        }
+        // no workgroup can wait for the others now; the last one to get here quantises the whole result alone
+        if (grid_last_arrival(a.sync, (int *)smem)) {
+            quantize_f32_u8_alone(a.C32, a.M * a.N, (uint8_t *)a.C, a.dscale_out, (float *)smem);
         }
         return;
     }

@@ -217,10 +217,6 @@ hipError_t launch_absmax_f32(const float *x, uint32_t n, uint32_t *ws, hipStream
 // written to *ds_out (device) when non-null.
 hipError_t launch_quantize_f32(const float *x, uint32_t n, void *q, int to_u8, const uint32_t *ws, float s_in,
     const float *ds_in, int mode, float *ds_out, hipStream_t st, int gelu = 0, const uint32_t *only_if = nullptr);
-// One workgroup that quantises x (dynamic scale, u8) only if *only_if != 0, writing the scale to *ds_out: the stand-by
-// behind a producer that normally quantises its own result
-hipError_t launch_quantize_f32_standby(const float *x, uint32_t n, void *q, float *ds_out, const uint32_t *only_if,
-    hipStream_t st);
 hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st);
 // s0 = output scale (< 0: dynamic from ws[0]), s1 = scale of the int32 data; the resulting output
 // scale is written to *ds_out (device) when non-null.
@@ -254,6 +250,7 @@ struct FusedSync {
         g.epoch = epoch;
         g.blocks = grid;
         g.spin_limit = spin_limit;
+        g.done = (unsigned *)(release + 1);  // a spare word beside release word 0
         return g;
     }
 };

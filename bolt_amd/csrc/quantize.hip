@@ -150,49 +150,6 @@ __global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t *__restri
     ws_block_fold_max(ws, m, red);
 }
 
-// Both passes of a dynamic fp32 -> u8 quantisation in ONE workgroup, run only when *only_if != 0: the stand-by behind a
-// producer that normally quantises its own result (and then leaves *only_if at 0, so that this launch costs one
-// near-empty dispatch). When the producer had to give up -- its workgroups could not all be resident within their
-// bounded wait, which takes the better part of a second to expire -- one workgroup's pace is no concern.
-__global__ __launch_bounds__(1024) void quantize_f32_standby_kernel(const float *__restrict__ x, uint32_t n,
-    uint8_t *__restrict__ q, float *__restrict__ ds_out, const uint32_t *__restrict__ only_if)
-{
-    if (*only_if == 0) {
-        return;
-    }
-    __shared__ float red[16];
-    const uint32_t tid = threadIdx.x;
-    float m = 0.0f;
-    for (uint32_t i = tid; i < n; i += 1024) {
-        const float a_ = fabsf(x[i]);
-        m = (a_ > m) ? a_ : m;  // a NaN never replaces the running max (avx512/quantize.cpp:21-68)
-    }
-    m = wave_reduce_max(m);
-    if ((tid & 63) == 0) {
-        red[tid >> 6] = m;
-    }
-    __syncthreads();
-    m = red[0];
-#pragma unroll
-    for (int w = 1; w < 16; ++w) {
-        m = red[w] > m ? red[w] : m;
-    }
-    const float s = (m == 0.0f) ? 1.0f : 127.0f / m;
-    if (tid == 0) {
-        *ds_out = s;
-    }
-    for (uint32_t i = tid; i < n; i += 1024) {
-        q[i] = (uint8_t)q_u8(x[i], s);
-    }
-}
-
-hipError_t launch_quantize_f32_standby(const float *x, uint32_t n, void *q, float *ds_out, const uint32_t *only_if,
-    hipStream_t st)
-{
-    hipLaunchKernelGGL(quantize_f32_standby_kernel, dim3(1), dim3(1024), 0, st, x, n, (uint8_t *)q, ds_out, only_if);
-    return hipGetLastError();
-}
-
 hipError_t launch_absmax_i32(const int32_t *x, uint32_t n, uint32_t *ws, hipStream_t st)
 {
     hipError_t e = launch_fill_u32(ws, kWsWords, 0, st);
