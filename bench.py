@@ -410,6 +410,11 @@ def other_kernels(L, capi, host, torch, dev, only=None):
             res[name] = {"n": cnt, "ms": t_h, "algorithmic_bytes": nbytes, "gbps": nbytes / t_h / 1e6,
                          "frac_hbm_peak": nbytes / t_h / 1e6 / HBM_PEAK_GBS, "ms_cache_resident": t_c,
                          "gbps_cache_resident": nbytes / t_c / 1e6}
+        # the practical ceiling for this kind of kernel: a plain device-to-device copy of the same tensors (50 MB read,
+        # 50 MB written per call, rotating like the others), done by the runtime's own copy
+        both("device_copy_f32_reference", 8 * cnt, lambda i: fo[i].copy_(xs[i]))
+        res["device_copy_f32_reference"]["note"] = ("torch's tensor copy of 4096 x 3072 fp32 (hipMemcpy-class kernel), not a kernel of "
+                                                    "this library: what HBM delivers to a read-and-write stream of this size")
         both("quantize_f32_u8_dynamic", 9 * cnt,
              lambda i: capi.check(L.bolt_gfx950_quantize_f32_async(xs[i].data_ptr(), cnt, DT_U8_Q, q8[i].data_ptr(),
                                                                    dsc.data_ptr(), 0), "q"))
