@@ -14,6 +14,9 @@ namespace bg {
 
 constexpr uint32_t kPixPerWg = 512;
 
+// F3: the filter is 3 x 3 (known when the kernel is compiled): the nine loads of a pixel are issued together and nothing
+// walks the taps; otherwise the tap position is carried along at run time.
+template <bool F3>
 __global__ __launch_bounds__(256) void depthwise_u8s8_i32_kernel(DepthwiseArgs a)
 {
     // blockIdx.x = plane * chunks + chunk: the plane (image, 16-channel block) comes from one scalar division per
@@ -63,28 +66,9 @@ __global__ __launch_bounds__(256) void depthwise_u8s8_i32_kernel(DepthwiseArgs a
         const uint32_t y = pix / a.ow, x = pix % a.ow;
         const size_t id = ((size_t)plane * opix + pix) * 4 + q;  // the output is [plane][pixel][16]
         int acc[4] = {base[0], base[1], base[2], base[3]};
-        // tap position carried along (kh, kw wrap at fw): no division inside the loop; everything here is wave-uniform
-        uint32_t kh = 0, kw = 0, left = taps;
         const uint8_t *row = in + ((size_t)(y * a.sh) * a.iw + x * a.sw) * 16;  // tap (0, 0) of this pixel
-        for (uint32_t g = 0; g < groups; ++g) {
-            // channel i: its four taps of this group, one byte each
-            const v4i wv = held ? (g == 0 ? wreg[0] : (g == 1 ? wreg[1] : wreg[2])) : *(const v4i *)(w + (size_t)g * 64);
-            // the same four taps of the input: one dword (4 channels) per tap; taps past the end repeat the last one
-            // (their weights are zero)
-            uint32_t px[4];
-#pragma unroll
-            for (uint32_t k = 0; k < 4; ++k) {
-                px[k] = *(const uint32_t *)(row + ((size_t)kh * a.iw + kw) * 16) ^ 0x80808080u;
-                if (left > 1) {
-                    --left;
-                    ++kw;
-                    if (kw == a.fw) {
-                        kw = 0;
-                        ++kh;
-                    }
-                }
-            }
-            // 4 x 4 byte transpose (taps x channels -> channels x taps) with v_perm_b32, then one v_dot4_i32_i8 per channel
+        // 4 x 4 byte transpose (taps x channels -> channels x taps) with v_perm_b32, then one v_dot4_i32_i8 per channel
+        auto tap_group = [&](const uint32_t (&px)[4], const v4i wv) {
             const uint32_t ab_lo = __builtin_amdgcn_perm(px[1], px[0], 0x05010400u), ab_hi = __builtin_amdgcn_perm(px[1], px[0], 0x07030602u);
             const uint32_t cd_lo = __builtin_amdgcn_perm(px[3], px[2], 0x05010400u), cd_hi = __builtin_amdgcn_perm(px[3], px[2], 0x07030602u);
             const uint32_t ch0 = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u), ch1 = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
@@ -93,6 +77,41 @@ __global__ __launch_bounds__(256) void depthwise_u8s8_i32_kernel(DepthwiseArgs a
             acc[1] = __builtin_amdgcn_sdot4((int)ch1, wv.y, acc[1], false);
             acc[2] = __builtin_amdgcn_sdot4((int)ch2, wv.z, acc[2], false);
             acc[3] = __builtin_amdgcn_sdot4((int)ch3, wv.w, acc[3], false);
+        };
+        if constexpr (F3) {
+            // the nine taps at once; the three that pad the last group repeat tap 8 (their weights are zero)
+            uint32_t p9[9];
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                p9[t] = *(const uint32_t *)(row + ((size_t)(t / 3) * a.iw + (t % 3)) * 16) ^ 0x80808080u;
+            }
+            const uint32_t g0[4] = {p9[0], p9[1], p9[2], p9[3]}, g1[4] = {p9[4], p9[5], p9[6], p9[7]}, g2[4] = {p9[8], p9[8], p9[8], p9[8]};
+            tap_group(g0, wreg[0]);
+            tap_group(g1, wreg[1]);
+            tap_group(g2, wreg[2]);
+        } else {
+            // tap position carried along (kh, kw wrap at fw): no division inside the loop; everything here is wave-uniform
+            uint32_t kh = 0, kw = 0, left = taps;
+            for (uint32_t g = 0; g < groups; ++g) {
+                // channel i: its four taps of this group, one byte each
+                const v4i wv = held ? (g == 0 ? wreg[0] : (g == 1 ? wreg[1] : wreg[2])) : *(const v4i *)(w + (size_t)g * 64);
+                // the same four taps of the input: one dword (4 channels) per tap; taps past the end repeat the last one
+                // (their weights are zero)
+                uint32_t px[4];
+#pragma unroll
+                for (uint32_t k = 0; k < 4; ++k) {
+                    px[k] = *(const uint32_t *)(row + ((size_t)kh * a.iw + kw) * 16) ^ 0x80808080u;
+                    if (left > 1) {
+                        --left;
+                        ++kw;
+                        if (kw == a.fw) {
+                            kw = 0;
+                            ++kh;
+                        }
+                    }
+                }
+                tap_group(px, wv);
+            }
         }
         if (a.relu) {
 #pragma unroll
@@ -114,7 +133,11 @@ hipError_t launch_depthwise_u8s8_i32(const DepthwiseArgs &a, hipStream_t st)
         (uint64_t)(a.oh - 1) * a.sh + a.fh > a.ih || (uint64_t)(a.ow - 1) * a.sw + a.fw > a.iw) {
         return hipErrorInvalidValue;  // every window must lie inside the image
     }
-    hipLaunchKernelGGL(depthwise_u8s8_i32_kernel, dim3((uint32_t)(planes * chunks)), dim3(256), 0, st, a);
+    if (a.fh == 3 && a.fw == 3) {
+        hipLaunchKernelGGL(depthwise_u8s8_i32_kernel<true>, dim3((uint32_t)(planes * chunks)), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(depthwise_u8s8_i32_kernel<false>, dim3((uint32_t)(planes * chunks)), dim3(256), 0, st, a);
+    }
     return hipGetLastError();
 }
 
