@@ -385,6 +385,15 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                                                "that norm: single elements differ by up to 2.6e-3 of max|out| (0.02 % of them "
                                                "by more than 1e-3) where a 1-ulp fp32 difference ahead of a quantiser moves "
                                                "one activation by one int8 step"}
+        # twelve such layers back to back (a BERT-base encoder; the same weights twelve times, which changes nothing
+        # for the timing: 85 MB of packed weights per layer against 4 MiB of L2 per XCD), one C call for the stack:
+        # every layer but the first takes its input's maximum from the LayerNorm that closed the layer before it
+        from bolt_amd.host_encoder import EncoderStack
+        stack = EncoderStack(torch, [layer] * 12)
+        ts = timed(lambda: stack(hx, hy), 10, warm=3)
+        res["bert_base_12_layer_stack"] = {"ms": ts, "ms_per_layer": ts / 12, "tokens_per_s": batch * seq / (ts * 1e-3),
+                                           "note": "bolt_gfx950_encoder_stack_int8: bit-identical to twelve single-layer calls "
+                                                   "(tests/test_gpu_encoder.py); 11 launches for the first layer, 10 for the others"}
     # -- quantize family at the BERT FFN size (4096 x 3072). Two regimes: "hbm" rotates over 8 tensors (400 MB of
     #    fp32 / int32 input, more than the 256 MB Infinity Cache holds), "cache_resident" reuses one tensor, which is
     #    what a layer sees when the producer's output is still in the Infinity Cache

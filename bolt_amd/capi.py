@@ -237,6 +237,9 @@ SIGNATURES = {
     "bolt_gfx950_encoder_layer_int8_workspace_layout": (C.c_int, [C.POINTER(BoltEncoderLayerInt8),
                                                                   C.POINTER(C.c_size_t)]),
     "bolt_gfx950_encoder_layer_int8": (C.c_int, [C.POINTER(BoltEncoderLayerInt8), _vp, _vp, _vp, C.c_size_t]),
+    "bolt_gfx950_encoder_stack_int8_workspace_bytes": (C.c_int, [C.POINTER(BoltEncoderLayerInt8), _u32,
+                                                                 C.POINTER(C.c_size_t)]),
+    "bolt_gfx950_encoder_stack_int8": (C.c_int, [C.POINTER(BoltEncoderLayerInt8), _u32, _vp, _vp, _vp, C.c_size_t]),
     "bolt_gfx950_attention_f32": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _vp]),
     "bolt_gfx950_add_layernorm_f32": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "bolt_gfx950_gelu_f32": (C.c_int, [_vp, C.c_size_t]),

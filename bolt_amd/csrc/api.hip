@@ -3093,28 +3093,12 @@ EE bolt_gfx950_encoder_layer_int8_workspace_layout(const BoltEncoderLayerInt8 *l
     return SUCCESS;
 }
 
-EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float *hidden, float *out, void *workspace,
-    size_t workspaceBytes)
+// One layer's launches. input_max_ready: the scratch slots already hold max|hidden| (the LayerNorm that produced
+// `hidden` folded it), so no abs-max pass runs; fold_out_max: the last LayerNorm folds max|out| into those slots for
+// the layer that follows.
+static EE encoder_run(const BoltEncoderLayerInt8 &L, const EncoderPlan &p, const float *hidden, float *out, void *workspace,
+    bool input_max_ready, bool fold_out_max)
 {
-    EE e = encoder_check(layer);
-    if (e != SUCCESS) {
-        return e;
-    }
-    if (!hidden || !out || !workspace) {
-        return NULL_POINTER;
-    }
-    const BoltEncoderLayerInt8 &L = *layer;
-    const EncoderPlan p = encoder_plan(L);
-    if (workspaceBytes < p.total) {
-        return NOT_MATCH;
-    }
-    if (((uintptr_t)workspace & 255) || ((uintptr_t)hidden & 15) || ((uintptr_t)out & 15)) {
-        return fail(NOT_SUPPORTED, "workspace must be 256-byte aligned, hidden / out 16-byte aligned");
-    }
-    e = ensure_init();
-    if (e != SUCCESS) {
-        return e;
-    }
     hipStream_t st = ctx().stream;
     U8 *w = (U8 *)workspace;
     const U32 T = L.batch * L.seq, H = L.hidden, F = L.ffn;
@@ -3149,12 +3133,14 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
     // before the next one.
     Ctx &c = ctx();
     uint32_t *ws0 = c.enc_ws, *ws1 = ws0 + kWsWords, *ws2 = ws1 + kWsWords, *ws3 = ws2 + kWsWords;
-    if (c.enc_ws_dirty) {
-        HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
+    if (!input_max_ready) {
+        if (c.enc_ws_dirty) {
+            HIP_TRY(launch_fill_u32(ws0, 4 * kWsWords, 0, st));
+        }
+        c.enc_ws_dirty = true;
+        HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st, true));
     }
-    c.enc_ws_dirty = true;
     // x -> u8 (dynamic per-tensor scale), one quantisation shared by Q, K and V
-    HIP_TRY(launch_absmax_f32(hidden, T * H, ws0, st, true));
     HIP_TRY(launch_quantize_f32(hidden, T * H, xq, 1, ws0, 0.0f, nullptr, 0, sc + 0, st));
     HIP_TRY(gemm(xq, L.wqkv, 3 * H, H, sc + 0, L.sqkv, L.bqkv, qkv));
     HIP_TRY(launch_attention_f32(qkv, L.batch, L.seq, H, L.heads, cx, ws1, st, ws0));
@@ -3200,8 +3186,112 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
         HIP_TRY(launch_quantize_f32(f, T * F, xq2, 1, ws3, 0.0f, nullptr, 0, sc + 3, st, 1));
     }
     HIP_TRY(gemm(xq2, L.w2, H, F, sc + 3, L.s2, L.b2, o));
-    HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, nullptr, st, ws3));
+    // (ws0 was consumed by the first quantiser and cleared by the attention kernel: free for the next layer's maximum)
+    HIP_TRY(launch_add_layernorm(h1, o, L.ln2_gamma, L.ln2_beta, T, H, out, fold_out_max ? ws0 : nullptr, st, ws3));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float *hidden, float *out, void *workspace,
+    size_t workspaceBytes)
+{
+    EE e = encoder_check(layer);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (!hidden || !out || !workspace) {
+        return NULL_POINTER;
+    }
+    const BoltEncoderLayerInt8 &L = *layer;
+    const EncoderPlan p = encoder_plan(L);
+    if (workspaceBytes < p.total) {
+        return NOT_MATCH;
+    }
+    if (((uintptr_t)workspace & 255) || ((uintptr_t)hidden & 15) || ((uintptr_t)out & 15)) {
+        return fail(NOT_SUPPORTED, "workspace must be 256-byte aligned, hidden / out 16-byte aligned");
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    Ctx &c = ctx();
+    e = encoder_run(L, p, hidden, out, workspace, false, false);
+    if (e != SUCCESS) {
+        return e;
+    }
     c.enc_ws_dirty = false;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_encoder_stack_int8(const BoltEncoderLayerInt8 *layers, U32 numLayers, const float *hidden, float *out,
+    void *workspace, size_t workspaceBytes)
+{
+    if (!layers || !hidden || !out || !workspace) {
+        return NULL_POINTER;
+    }
+    if (numLayers == 0) {
+        return NOT_SUPPORTED;
+    }
+    size_t need = 0;
+    EE e = bolt_gfx950_encoder_stack_int8_workspace_bytes(layers, numLayers, &need);
+    if (e != SUCCESS) {
+        return e;
+    }
+    if (workspaceBytes < need) {
+        return NOT_MATCH;
+    }
+    if (((uintptr_t)workspace & 255) || ((uintptr_t)hidden & 15) || ((uintptr_t)out & 15)) {
+        return fail(NOT_SUPPORTED, "workspace must be 256-byte aligned, hidden / out 16-byte aligned");
+    }
+    e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    // the layers share one layer's workspace (the largest); behind it two [T, hidden] fp32 buffers take the
+    // activations from layer to layer
+    size_t one = 0;
+    for (U32 i = 0; i < numLayers; ++i) {
+        const size_t t = encoder_plan(layers[i]).total;
+        one = t > one ? t : one;
+    }
+    const size_t act = ((size_t)layers[0].batch * layers[0].seq * layers[0].hidden * 4 + 255) / 256 * 256;
+    float *pp[2] = {(float *)((U8 *)workspace + one), (float *)((U8 *)workspace + one + act)};
+    Ctx &c = ctx();
+    const float *in = hidden;
+    for (U32 i = 0; i < numLayers; ++i) {
+        const bool last = i + 1 == numLayers;
+        float *o = last ? out : pp[i & 1];
+        e = encoder_run(layers[i], encoder_plan(layers[i]), in, o, workspace, i != 0, !last);
+        if (e != SUCCESS) {
+            return e;
+        }
+        in = o;
+    }
+    c.enc_ws_dirty = false;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_encoder_stack_int8_workspace_bytes(const BoltEncoderLayerInt8 *layers, U32 numLayers, size_t *bytes)
+{
+    if (!layers || !bytes) {
+        return NULL_POINTER;
+    }
+    if (numLayers == 0) {
+        return NOT_SUPPORTED;
+    }
+    size_t one = 0;
+    for (U32 i = 0; i < numLayers; ++i) {
+        EE e = encoder_check(&layers[i]);
+        if (e != SUCCESS) {
+            return e;
+        }
+        if (layers[i].batch != layers[0].batch || layers[i].seq != layers[0].seq || layers[i].hidden != layers[0].hidden) {
+            return NOT_MATCH;  // the activations keep their shape from layer to layer
+        }
+        const size_t t = encoder_plan(layers[i]).total;
+        one = t > one ? t : one;
+    }
+    const size_t act = ((size_t)layers[0].batch * layers[0].seq * layers[0].hidden * 4 + 255) / 256 * 256;
+    *bytes = one + 2 * act;
     return SUCCESS;
 }
 

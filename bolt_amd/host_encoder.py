@@ -54,3 +54,23 @@ class EncoderLayer:
         shapes = (("qkv", 3 * H), ("ctx", H), ("attn_out", H), ("h1", H), ("ffn_pre", F), ("ffn_out", H))
         return {name: self.workspace[offs[i]:offs[i] + T * w * 4].view(self.torch.float32).view(T, w)
                 for i, (name, w) in enumerate(shapes)}
+
+
+class EncoderStack:
+    """Several EncoderLayer objects run back to back by bolt_gfx950_encoder_stack_int8 (same batch, seq and hidden)."""
+
+    def __init__(self, torch, layers):
+        self.torch = torch
+        self.layers = list(layers)   # keeps their weights alive
+        n = len(self.layers)
+        self.specs = (BoltEncoderLayerInt8 * n)(*[l.L for l in self.layers])
+        nbytes = C.c_size_t(0)
+        check(lib().bolt_gfx950_encoder_stack_int8_workspace_bytes(self.specs, n, C.byref(nbytes)), "encoder_stack_workspace_bytes")
+        self.workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=torch.device("cuda:0"))
+
+    def __call__(self, x, out=None):
+        if out is None:
+            out = self.torch.empty_like(x)
+        check(lib().bolt_gfx950_encoder_stack_int8(self.specs, len(self.layers), x.data_ptr(), out.data_ptr(),
+                                                  self.workspace.data_ptr(), self.workspace.numel()), "encoder_stack")
+        return out

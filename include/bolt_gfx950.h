@@ -424,6 +424,15 @@ EE bolt_gfx950_encoder_layer_int8(const BoltEncoderLayerInt8 *layer, const float
  * values are never stored: the quantiser ahead of the second FFN product applies GELU to what it
  * reads), FFN output [T, hidden]. */
 EE bolt_gfx950_encoder_layer_int8_workspace_layout(const BoltEncoderLayerInt8 *layer, size_t *offsets);
+/* numLayers such layers back to back (a BERT encoder is twelve): layer i + 1 reads what layer i wrote. The result is,
+ * bit for bit, that of numLayers calls of bolt_gfx950_encoder_layer_int8; what the stack saves is the abs-max pass over
+ * every layer's input but the first -- the LayerNorm that closes a layer folds max|out| into the scratch slots, which
+ * is exactly the maximum the next layer's input quantiser wants. All layers share batch, seq and hidden (else
+ * NOT_MATCH); the workspace (size from the query) holds one layer's intermediates and two [T, hidden] fp32 buffers
+ * that carry the activations from layer to layer. hidden and out may be the same buffer only for numLayers > 1. */
+EE bolt_gfx950_encoder_stack_int8_workspace_bytes(const BoltEncoderLayerInt8 *layers, U32 numLayers, size_t *bytes);
+EE bolt_gfx950_encoder_stack_int8(const BoltEncoderLayerInt8 *layers, U32 numLayers, const float *hidden, float *out,
+    void *workspace, size_t workspaceBytes);
 
 /* The layer's fp32 pieces on their own (device pointers, asynchronous):
  *   attention: qkv rows [Q | K | V] of 3*hidden floats -> ctx = softmax(Q K^T / 8) V per head of 64

@@ -231,3 +231,33 @@ def test_encoder_layer_fused_ffn_other_shape(torch_mod):
     fused = layer(x)
     capi.check(L.bolt_gfx950_synchronize(), "sync")
     assert torch.equal(fused, plain)
+
+
+@pytest.mark.gpu
+def test_encoder_stack_equals_layer_by_layer(torch_mod):
+    """bolt_gfx950_encoder_stack_int8 over three layers with different weights (two FFN widths, so the layers' workspaces
+    differ) gives, bit for bit, what three single-layer calls give: the maximum the LayerNorm at the end of a layer
+    folds for the next one is the maximum that layer's own abs-max pass would have found. Run twice, and once after
+    a single-layer call in between, so that slots left over from one form cannot leak into the other."""
+    from bolt_amd.host_encoder import EncoderStack
+    torch = torch_mod
+    batch, seq, hidden, heads = 8, 96, 256, 4
+    rng = np.random.default_rng(4242)
+    layers = []
+    for ffn in (1024, 512, 1024):
+        layers.append(EncoderLayer(torch, batch, seq, hidden, heads, ffn, make_params(rng, hidden, ffn, with_bias=True)))
+    x = dev(torch, rng.standard_normal((batch * seq, hidden)).astype(np.float32))
+    want = x
+    for l in layers:
+        want = l(want).clone()
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    stack = EncoderStack(torch, layers)
+    for rep in range(2):
+        got = stack(x)
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        assert torch.equal(got, want), "stack differs from layer-by-layer (repetition %d)" % rep
+        layers[1](x)   # a single-layer call between two stack calls
+    one = EncoderStack(torch, layers[:1])
+    assert torch.equal(one(x), layers[0](x))
+    n = capi.C.c_size_t(0)
+    assert capi.lib().bolt_gfx950_encoder_stack_int8_workspace_bytes(stack.specs, 0, capi.C.byref(n)) == capi.NOT_SUPPORTED
