@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--copies", type=int, default=64, help="replicas of the weight blob the batch rotates over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "quantize", "pool", "lstm", "deconv", "depthwise", "ptq"],
+    ap.add_argument("--only", choices=["gemm", "gemm_data", "fc", "conv", "bnn", "encoder", "encoder_stack", "quantize", "pool", "lstm", "deconv", "depthwise", "ptq"],
                     help="run just this secondary workload and print its figures (profiling aid; not the bench line)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary measurements (GEMM sweep, FC, conv, BNN, quantize) in `other_kernels`")
@@ -350,7 +350,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         res["bnn_c5_xnor"]["frac_fp4_mfma_peak"] = res["bnn_c5_xnor"]["binary_tops"] / 10100.0
         res["bnn_c5_xnor_int8_matrix_cores"]["frac_mfma_peak"] = res["bnn_c5_xnor_int8_matrix_cores"]["binary_tops"] / MFMA_PEAK_TOPS
     # -- C4: BERT-base int8 encoder layer, batch 32 x seq 128 (4096 tokens), one C call per layer
-    if want("encoder"):
+    if want("encoder") or want("encoder_stack"):
         from bolt_amd.capi import DT_I8
         from bolt_amd.host_encoder import EncoderLayer
         rs = np.random.default_rng(20240604)
@@ -373,9 +373,10 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         layer = EncoderLayer(torch, batch, seq, hidden, heads, ffn, P)
         hx = torch.randn((batch * seq, hidden), device=dev, generator=g)
         hy = torch.empty_like(hx)
-        t = timed(lambda: layer(hx, hy), 50)
+        t = timed(lambda: layer(hx, hy), 50) if want("encoder") else None
         gemm_ops = 2.0 * batch * seq * hidden * (3 * hidden + hidden + 2 * ffn)
-        res["bert_base_layer_c4"] = {"ms": t, "tokens_per_s": batch * seq / (t * 1e-3), "int8_gemm_tops": gemm_ops / t / 1e9,
+        if want("encoder"):
+            res["bert_base_layer_c4"] = {"ms": t, "tokens_per_s": batch * seq / (t * 1e-3), "int8_gemm_tops": gemm_ops / t / 1e9,
                                      "config": "hidden 768, 12 heads, FFN 3072, seq 128, batch 32; int8 GEMMs with per-channel "
                                                "weight scales, dynamic per-tensor activation quantisation, fp32 attention / "
                                                "LayerNorm / GELU",
@@ -388,12 +389,13 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         # twelve such layers back to back (a BERT-base encoder; the same weights twelve times, which changes nothing
         # for the timing: 85 MB of packed weights per layer against 4 MiB of L2 per XCD), one C call for the stack:
         # every layer but the first takes its input's maximum from the LayerNorm that closed the layer before it
-        from bolt_amd.host_encoder import EncoderStack
-        stack = EncoderStack(torch, [layer] * 12)
-        ts = timed(lambda: stack(hx, hy), 10, warm=3)
-        res["bert_base_12_layer_stack"] = {"ms": ts, "ms_per_layer": ts / 12, "tokens_per_s": batch * seq / (ts * 1e-3),
-                                           "note": "bolt_gfx950_encoder_stack_int8: bit-identical to twelve single-layer calls "
-                                                   "(tests/test_gpu_encoder.py); 11 launches for the first layer, 10 for the others"}
+        if want("encoder_stack"):
+            from bolt_amd.host_encoder import EncoderStack
+            stack = EncoderStack(torch, [layer] * 12)
+            ts = timed(lambda: stack(hx, hy), 10, warm=3)
+            res["bert_base_12_layer_stack"] = {"ms": ts, "ms_per_layer": ts / 12, "tokens_per_s": batch * seq / (ts * 1e-3),
+                                               "note": "bolt_gfx950_encoder_stack_int8: bit-identical to twelve single-layer calls "
+                                                       "(tests/test_gpu_encoder.py); 11 launches for the first layer, 10 for the others"}
     # -- quantize family at the BERT FFN size (4096 x 3072). Two regimes: "hbm" rotates over 8 tensors (400 MB of
     #    fp32 / int32 input, more than the 256 MB Infinity Cache holds), "cache_resident" reuses one tensor, which is
     #    what a layer sees when the producer's output is still in the Infinity Cache
