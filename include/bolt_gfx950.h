@@ -406,7 +406,7 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
  *                 [hidden, 3*hidden] (Q | K | V columns), [hidden, hidden], [hidden, ffn], [ffn, hidden]
  *   s*          : fp32 [N] weight scales, Bolt convention (quantised = real * scale)
  *   b*          : fp32 [N] biases or NULL;  ln*: fp32 [hidden]
- * All pointers are device pointers except `layer` itself; the call enqueues ~15 kernels on the
+ * All pointers are device pointers except `layer` itself; the call enqueues 11 kernels on the
  * library stream and returns. workspace: 256-byte aligned, size from the query. */
 typedef struct {
     U32 batch, seq, hidden, heads, ffn;
