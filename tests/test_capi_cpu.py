@@ -197,3 +197,40 @@ def test_pool_concat_lstm_argument_checks_and_size_queries():
     assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, N, K), hd, proj, C.byref(nb),
                                                     AMD_GFX950) == capi.NOT_SUPPORTED
     assert C.sizeof(RNNParamSpec) == 36
+
+
+def test_encoder_workspace_queries():
+    """Size queries of the encoder layer and of a stack of layers (no GPU involved): argument checks, and the stack's
+    workspace = the largest layer's + two [tokens, hidden] fp32 buffers that carry activations between layers."""
+    L = capi.lib()
+    C = capi.C
+    one = C.c_float(0)
+    ptr = C.cast(C.pointer(one), C.POINTER(C.c_float))
+
+    def spec(ffn, hidden=256, heads=4):
+        s = capi.BoltEncoderLayerInt8()
+        s.batch, s.seq, s.hidden, s.heads, s.ffn = 4, 32, hidden, heads, ffn
+        for name in ("wqkv", "wo", "w1", "w2"):
+            setattr(s, name, C.addressof(one))   # never dereferenced by the queries
+        for name in ("sqkv", "so", "s1", "s2", "ln1_gamma", "ln1_beta", "ln2_gamma", "ln2_beta"):
+            setattr(s, name, ptr)
+        return s
+
+    n = C.c_size_t(0)
+    a, b = spec(1024), spec(512)
+    capi.check(L.bolt_gfx950_encoder_layer_int8_workspace_bytes(C.byref(a), C.byref(n)), "layer a")
+    na = n.value
+    capi.check(L.bolt_gfx950_encoder_layer_int8_workspace_bytes(C.byref(b), C.byref(n)), "layer b")
+    nb = n.value
+    assert na > nb > 0
+    stack = (capi.BoltEncoderLayerInt8 * 3)(b, a, b)
+    capi.check(L.bolt_gfx950_encoder_stack_int8_workspace_bytes(stack, 3, C.byref(n)), "stack")
+    act = (4 * 32 * 256 * 4 + 255) // 256 * 256
+    assert n.value == na + 2 * act
+    assert L.bolt_gfx950_encoder_stack_int8_workspace_bytes(None, 3, C.byref(n)) == capi.NULL_POINTER
+    assert L.bolt_gfx950_encoder_stack_int8_workspace_bytes(stack, 3, None) == capi.NULL_POINTER
+    assert L.bolt_gfx950_encoder_stack_int8_workspace_bytes(stack, 0, C.byref(n)) == capi.NOT_SUPPORTED
+    mixed = (capi.BoltEncoderLayerInt8 * 2)(a, spec(1024, hidden=128, heads=2))
+    assert L.bolt_gfx950_encoder_stack_int8_workspace_bytes(mixed, 2, C.byref(n)) == capi.NOT_MATCH
+    bad = (capi.BoltEncoderLayerInt8 * 1)(spec(1024, hidden=256, heads=3))   # hidden != heads * 64
+    assert L.bolt_gfx950_encoder_stack_int8_workspace_bytes(bad, 1, C.byref(n)) == capi.NOT_SUPPORTED
