@@ -128,7 +128,7 @@ def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
         capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
         for M, K, N in [(1, 64, 16), (130, 128, 70), (256, 64, 256), (300, 256, 200), (257, 192, 513),
                         (512, 1024, 384), (100, 1040, 48), (260, 384, 300), (40, 896, 272), (512, 1536, 512),
-                        (300, 768, 600)]:
+                        (300, 768, 600), (128, 576, 128), (200, 448, 130), (129, 832, 257)]:
             say("variant", tile, M, K, N)
             A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
             W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
