@@ -942,10 +942,12 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
     }
 
     if constexpr (PIPE == 3) {
-        // Ping-pong schedule as PIPE == 2, with A requested in whole 128-byte lines. A request of 16 rows x 64
-        // bytes (one MFMA fragment, what the other loops issue) touches 16 half lines and the L1 / L2 path
-        // delivers such requests 2.5 times slower than 1 KB made of 8 whole lines (measured in isolation:
-        // 1 040 against 410 cycles per 16 KB and CU), which is more than the MFMAs of a K tile take. Here a
+        // Ping-pong schedule as PIPE == 2, with A requested in whole 128-byte lines. A request laid out like the
+        // MFMA operand (lane 16 g + i = 16 bytes of row i) puts a different row into every lane, the address unit
+        // takes each lane's 16 bytes as a piece of its own, and such a request takes 2.5 times longer to be
+        // accepted than 1 KB made of 8 whole lines (measured in isolation: 1 040 against 410 cycles per 16 KB and
+        // CU), which is more than the MFMAs of a K tile take. (The other loops now give a row to the four lanes of
+        // a quad, 64 contiguous bytes, which is accepted as fast.) Here a
         // request covers 8 rows x 128 bytes = the K bytes of two consecutive tiles, so A travels in pairs of
         // tiles: three slots of 256 rows x 128 bytes (tile pair p in slot p % 3, requested four tiles ahead
         // at the even tile) next to the four B slots of 16 KB (tile t in slot t % 4, requested three ahead).
@@ -1244,7 +1246,14 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
                 const uint32_t oy = r / a.conv.OW, ox = r % a.conv.OW;
                 off[q] = ((img * (a.conv.ICp / 16) * a.conv.Hp + oy * a.conv.sh) * a.conv.Wp + ox * a.conv.sw) * 16;
             } else {
-                off[q] = row * a.lda + g * 16;
+                // lane 4 r + c asks for 16 bytes of row r: the four lanes of a quad cover 64 contiguous bytes, which the
+                // address unit takes as one piece (with lane = 16 g + i, a lane per row, every lane is a piece of its
+                // own and a request takes several times longer to be accepted). Chunk c ^ (r / 4 % 4) rather than c,
+                // so that the fragment read below, 16 lanes = 16 rows of one chunk, spreads over all banks.
+                const uint32_t r4 = lane >> 2;
+                uint32_t rowq = m0 + (wave + q * T::kWaves) * 16 + r4;
+                rowq = rowq < a.M ? rowq : a.M - 1;
+                off[q] = rowq * a.lda + (((lane & 3) ^ ((r4 >> 2) & 3)) * 16);
             }
         } else {
             uint32_t nb = (n0 >> 4) + (wave + (q - kQA) * T::kWaves);
@@ -1253,6 +1262,8 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
         }
     }
     const uint32_t ksteps = K / 64;
+    // where lane (i, g) finds chunk g of row i inside a 1 KB A fragment in LDS (see the request layout above)
+    const uint32_t a_rd = CONV ? lane * 16 : i * 64 + ((g ^ ((i >> 2) & 3)) * 16);
 
 // slot: which LDS buffer (slot % STAGES); tile: which K tile to fetch. Past the end of K the
 // schedule keeps issuing (slot advances, tile is clamped to the last one) so that the number of
@@ -1331,7 +1342,7 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
             }
 #pragma unroll
             for (int x = 0; x < TM; ++x) {
-                v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + lane * 16);
+                v4i fa = *(const v4i *)(sA + (wm * TM + x) * 1024 + a_rd);
                 if (!CONV) {
                     fa ^= flip;
                 }
@@ -1385,7 +1396,7 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
                 }
 #pragma unroll
                 for (int x = 0; x < TM; ++x) {
-                    fa[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + lane * 16);
+                    fa[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + a_rd);
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): fragments in registers before the matrix phase
@@ -1428,6 +1439,67 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
             __builtin_amdgcn_s_barrier();
         }
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches
+    } else if constexpr (PIPE == 7) {
+        // Fragment prefetch as below, with the program order of a K step written out and pinned: a wave that is alone
+        // on its SIMD overlaps nothing by itself, and whatever stands in front of the first MFMA of a step runs with
+        // the matrix pipe idle. Here each fragment read, tile request and re-bias sits behind an MFMA and issues while
+        // that MFMA executes; the re-bias is applied when a fragment arrives, one step ahead of its use.
+        static_assert(!CONV && !FP4 && STAGES >= 3, "matrix product only");
+        static_assert(T::kLoads + TM + TN + TM <= TM * TN, "one slot behind each MFMA");
+        v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+#define BG7_STEP(tt, FA, FB, NA, NB)                                                         \
+    {                                                                                        \
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * T::kLoads) & 0xf0ff);            \
+        asm volatile("" ::: "memory");                                                       \
+        __builtin_amdgcn_s_barrier();                                                        \
+        asm volatile("" ::: "memory");                                                       \
+        const uint8_t *rA_ = smem + (BG_CLAMP((tt) + 1) % STAGES) * T::kStageBytes + wm * TM * 1024 + a_rd; \
+        const uint8_t *rB_ = smem + (BG_CLAMP((tt) + 1) % STAGES) * T::kStageBytes + (T::kAFrags + wn * TN) * 1024 + lane * 16; \
+        uint8_t *st_ = smem + (((tt) + (STAGES - 1)) % STAGES) * T::kStageBytes;             \
+        const uint32_t tl_ = BG_CLAMP((tt) + (STAGES - 1));                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                   \
+        _Pragma("unroll") for (int m = 0; m < TM * TN; ++m)                                  \
+        {                                                                                    \
+            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_16x16x64_i8(FB[m % TN], FA[m / TN], acc[m / TN][m % TN], 0, 0, 0); \
+            if (m < TM) {                                                                    \
+                NA[m] = *(const v4i *)(rA_ + m * 1024);                                      \
+            } else if (m < TM + TN) {                                                        \
+                NB[m - TM] = *(const v4i *)(rB_ + (m - TM) * 1024);                          \
+            } else if (m < TM + TN + T::kLoads) {                                            \
+                const int q = m - TM - TN;                                                   \
+                const uint8_t *base_ = (q < kQA) ? a.A + aoff_next : (const uint8_t *)a.Bp + (size_t)tl_ * 1024; \
+                const int f_ = (q < kQA) ? (wave + q * T::kWaves) : (T::kAFrags + wave + (q - kQA) * T::kWaves); \
+                __builtin_amdgcn_global_load_lds((gptr_t)(base_ + off[q]), (lptr_t)(st_ + f_ * 1024), 16, 0, 0); \
+            } else if (m >= TM * TN - TM) {                                                  \
+                NA[m - (TM * TN - TM)] ^= flip; /* the reads are 4+ MFMAs old by now */       \
+            }                                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                               \
+        }                                                                                    \
+        aoff_next = BG_AOFF(BG_CLAMP((tt) + STAGES));                                        \
+    }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            fb0[y] = *(const v4i *)(smem + (T::kAFrags + wn * TN + y) * 1024 + lane * 16);
+        }
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            fa0[x] = *(const v4i *)(smem + (wm * TM + x) * 1024 + a_rd) ^ flip;
+        }
+        uint32_t t = 0;
+        size_t aoff_next = BG_AOFF(BG_CLAMP(t + (STAGES - 1)));
+        for (; t + 1 < ksteps; t += 2) {
+            BG7_STEP(t, fa0, fb0, fa1, fb1);
+            BG7_STEP(t + 1, fa1, fb1, fa0, fb0);
+        }
+        if (t < ksteps) {
+            BG7_STEP(t, fa0, fb0, fa1, fb1);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+#undef BG7_STEP
     } else {
         // Fragment-prefetch schedule: the fragments of tile t+1 are read from LDS into a second
         // register set while the MFMAs of tile t run, so no MFMA ever waits for an LDS read. That
@@ -1444,7 +1516,7 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
         }                                                                                    \
         _Pragma("unroll") for (int x = 0; x < TM; ++x)                                       \
         {                                                                                    \
-            FA[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + lane * 16); /* raw u8 */      \
+            FA[x] = *(const v4i *)(sA_ + (wm * TM + x) * 1024 + a_rd); /* raw u8 */           \
         }                                                                                    \
     }
 #define BG_STEP(tt, FA, FB, NA, NB)                                                          \
@@ -2047,7 +2119,7 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
                 tile = 13;
             }
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
-            tile = k64 ? 10 : 2;
+            tile = k64 ? 15 : 2;  // 15 against 10 (the compiler's order): 8.4 / 17.9 / 14.1 against 9.5 / 20.0 / 16.4 us at 4096 x 768 x 768, 4096 x 3072 x 768, 2048^3
         }
     }
     if (g_force_tile >= 0 && (tiled_ok || g_force_tile == 0)) {
@@ -2091,6 +2163,8 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 4, 8, 4, 5, 3>(a, st);  // the same with A requested in whole 128-byte lines (160 KB of LDS)
         case 13:
             return launch_dma<2, 4, 8, 4, 3, 4>(a, st);  // as 12 with the B fragments loaded straight into registers (96 KB of LDS)
+        case 15:
+            return launch_dma<2, 2, 4, 4, 4, 7>(a, st);  // 128 x 128, fragment prefetch in a pinned program order
         default:
             break;
     }
