@@ -886,12 +886,14 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 template <int WM, int WN, int TM, int TN, int STAGES, int PIPE, bool CONV = false, bool FP4 = false, bool GELU_DYN = false>
 // Two waves per SIMD are asked for also where a workgroup has four waves: with a budget of 512 registers per lane
 // the compiler keeps the accumulators in AGPRs and spends dozens of v_accvgpr moves per K tile on shuffling them.
-__global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs a)
+__global__ __launch_bounds__(WM *WN * 64 * (PIPE == 8 ? 2 : 1), PIPE == 8 ? 1 : 2) void gemm_u8s8_dma_kernel(GemmArgs a)
 {
     using T = GemmDma<WM, WN, TM, TN, STAGES>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lane = threadIdx.x & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it scalar
+    const uint32_t wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it scalar
+    // PIPE == 8: two groups of WM x WN waves work on the same tile, group gidx on the K tiles 2 j + gidx
+    const uint32_t gidx = (PIPE == 8) ? wave_all / (WM * WN) : 0u, wave = (PIPE == 8) ? wave_all % (WM * WN) : wave_all;
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
     if (CONV) {
@@ -1313,7 +1315,7 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
     }
 
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) {
+    for (int s = 0; s < (PIPE == 8 ? 0 : STAGES - 1); ++s) {
         BG_ISSUE((uint32_t)s, BG_CLAMP((uint32_t)s), (CONV ? BG_CV_OFF() : BG_AOFF(BG_CLAMP((uint32_t)s))));
         if (CONV && (uint32_t)s + 1 < ksteps) {
             BG_CV_ADVANCE();
@@ -1439,6 +1441,116 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
             __builtin_amdgcn_s_barrier();
         }
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the clamped refetches
+    } else if constexpr (PIPE == 8) {
+        // Two groups of four waves on one 128 x 128 tile, each running the pinned-order loop of PIPE 7 over every other
+        // K tile in a stage ring of its own: every SIMD then holds two waves whose MFMAs fill each other's issue
+        // gaps, without a second workgroup (these grids have fewer tiles than the part has CUs). The partial
+        // sums meet in LDS after the loop (integer sums: the order does not matter) and group 0 runs the epilogue.
+        static_assert(!CONV && !FP4 && STAGES >= 3, "matrix product only");
+        static_assert(T::kLoads + TM + TN + TM <= TM * TN, "one slot behind each MFMA");
+        uint8_t *ring = smem + gidx * T::kLdsBytes;
+        const uint32_t gsteps = ksteps / 2;  // the launcher only comes here with an even number of K tiles
+        v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+#define BG8_TILE(j) (2 * ((j) < gsteps ? (j) : gsteps - 1) + gidx) /* K tile of this group's step j, clamped */
+#define BG8_REQ(slot_, j_)                                                                   \
+    {                                                                                        \
+        uint8_t *st_ = ring + ((slot_) % STAGES) * T::kStageBytes;                           \
+        const uint32_t tl_ = BG8_TILE(j_);                                                   \
+        _Pragma("unroll") for (int q = 0; q < T::kLoads; ++q)                                \
+        {                                                                                    \
+            const uint8_t *base_ = (q < kQA) ? a.A + (size_t)tl_ * 64 : (const uint8_t *)a.Bp + (size_t)tl_ * 1024; \
+            const int f_ = (q < kQA) ? (wave + q * T::kWaves) : (T::kAFrags + wave + (q - kQA) * T::kWaves); \
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_ + off[q]), (lptr_t)(st_ + f_ * 1024), 16, 0, 0); \
+        }                                                                                    \
+    }
+#define BG8_STEP(tt, FA, FB, NA, NB)                                                         \
+    {                                                                                        \
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * T::kLoads) & 0xf0ff);            \
+        asm volatile("" ::: "memory");                                                       \
+        __builtin_amdgcn_s_barrier();                                                        \
+        asm volatile("" ::: "memory");                                                       \
+        const uint32_t rd_ = ((tt) + 1 < gsteps ? (tt) + 1 : gsteps - 1) % STAGES;           \
+        const uint8_t *rA_ = ring + rd_ * T::kStageBytes + wm * TM * 1024 + a_rd;            \
+        const uint8_t *rB_ = ring + rd_ * T::kStageBytes + (T::kAFrags + wn * TN) * 1024 + lane * 16; \
+        uint8_t *st_ = ring + (((tt) + (STAGES - 1)) % STAGES) * T::kStageBytes;             \
+        const uint32_t tl_ = BG8_TILE((tt) + (STAGES - 1));                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                   \
+        _Pragma("unroll") for (int m = 0; m < TM * TN; ++m)                                  \
+        {                                                                                    \
+            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_16x16x64_i8(FB[m % TN], FA[m / TN], acc[m / TN][m % TN], 0, 0, 0); \
+            if (m < TM) {                                                                    \
+                NA[m] = *(const v4i *)(rA_ + m * 1024);                                      \
+            } else if (m < TM + TN) {                                                        \
+                NB[m - TM] = *(const v4i *)(rB_ + (m - TM) * 1024);                          \
+            } else if (m < TM + TN + T::kLoads) {                                            \
+                const int q = m - TM - TN;                                                   \
+                const uint8_t *base_ = (q < kQA) ? a.A + (size_t)tl_ * 64 : (const uint8_t *)a.Bp + (size_t)tl_ * 1024; \
+                const int f_ = (q < kQA) ? (wave + q * T::kWaves) : (T::kAFrags + wave + (q - kQA) * T::kWaves); \
+                __builtin_amdgcn_global_load_lds((gptr_t)(base_ + off[q]), (lptr_t)(st_ + f_ * 1024), 16, 0, 0); \
+            } else if (m >= TM * TN - TM) {                                                  \
+                NA[m - (TM * TN - TM)] ^= flip;                                              \
+            }                                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                               \
+        }                                                                                    \
+    }
+        // (the shared prologue above requested tiles 0 .. STAGES-2 into the first ring for everybody: redo it per group)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int s_ = 0; s_ < STAGES - 1; ++s_) {
+            BG8_REQ((uint32_t)s_, (uint32_t)s_);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * T::kLoads));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            fb0[y] = *(const v4i *)(ring + (T::kAFrags + wn * TN + y) * 1024 + lane * 16);
+        }
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            fa0[x] = *(const v4i *)(ring + (wm * TM + x) * 1024 + a_rd) ^ flip;
+        }
+        uint32_t t = 0;
+        for (; t + 1 < gsteps; t += 2) {
+            BG8_STEP(t, fa0, fb0, fa1, fb1);
+            BG8_STEP(t + 1, fa1, fb1, fa0, fb0);
+        }
+        if (t < gsteps) {
+            BG8_STEP(t, fa0, fb0, fa1, fb1);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();  // nobody reads fragments any more: the rings are free
+        asm volatile("" ::: "memory");
+        {   // group 1 hands its partial sums over: register r of lane l of wave w at ((w * TM * TN + r) * 64 + l) * 16
+            v4i *xch = (v4i *)smem + (size_t)wave * (TM * TN) * 64 + lane;
+            if (gidx == 1) {
+#pragma unroll
+                for (int x = 0; x < TM; ++x) {
+#pragma unroll
+                    for (int y = 0; y < TN; ++y) {
+                        xch[(x * TN + y) * 64] = acc[x][y];
+                    }
+                }
+            }
+            __syncthreads();
+            if (gidx == 0) {
+#pragma unroll
+                for (int x = 0; x < TM; ++x) {
+#pragma unroll
+                    for (int y = 0; y < TN; ++y) {
+                        acc[x][y] += xch[(x * TN + y) * 64];
+                    }
+                }
+            }
+        }
+#undef BG8_STEP
+#undef BG8_REQ
+#undef BG8_TILE
     } else if constexpr (PIPE == 7) {
         // Fragment prefetch as below, with the program order of a K step written out and pinned: a wave that is alone
         // on its SIMD overlaps nothing by itself, and whatever stands in front of the first MFMA of a step runs with
@@ -1599,6 +1711,9 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_dma_kernel(GemmArgs 
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+    }
+    if (PIPE == 8 && gidx == 1) {
+        return;  // its sums are in group 0's accumulators
     }
     if constexpr (GELU_DYN) {
         epilogue_gelu_sync<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
@@ -1915,7 +2030,7 @@ static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
     static bool attr_set = false;
     auto kern = gemm_u8s8_dma_kernel<WM, WN, TM, TN, STAGES, PIPE, CONV, FP4, GELU_DYN>;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes);
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes * (PIPE == 8 ? 2 : 1));
         if (e != hipSuccess) {
             return e;
         }
@@ -1926,7 +2041,7 @@ static hipError_t launch_dma(const GemmArgs &a, hipStream_t st)
     // a result much larger than the L2s (8 x 4 MiB) is written in several rounds of tiles: keep it from
     // displacing the operand panels (measured at 8192^3: 6 % faster; at 64 MiB and below: level or slower)
     b.stream_c = !CONV && (uint64_t)a.M * a.N * 4 > ((uint64_t)96 << 20);
-    hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), T::kLdsBytes, st, b);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64 * (PIPE == 8 ? 2 : 1)), T::kLdsBytes * (PIPE == 8 ? 2 : 1), st, b);
     return hipGetLastError();
 }
 
@@ -2120,6 +2235,11 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             }
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
             tile = k64 ? 15 : 2;  // 15 against 10 (the compiler's order): 8.4 / 17.9 / 14.1 against 9.5 / 20.0 / 16.4 us at 4096 x 768 x 768, 4096 x 3072 x 768, 2048^3
+            // long K on a grid that leaves CUs idle: two wave groups per tile on alternate K tiles (17.0 against 18.1 us at
+            // 4096 x 3072 x 768; slower for short K and for grids of several rounds)
+            if (tile == 15 && a.K % 128 == 0 && a.K >= 2048 && b128 <= 256) {
+                tile = 16;
+            }
         }
     }
     if (g_force_tile >= 0 && (tiled_ok || g_force_tile == 0)) {
@@ -2165,6 +2285,11 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             return launch_dma<2, 4, 8, 4, 3, 4>(a, st);  // as 12 with the B fragments loaded straight into registers (96 KB of LDS)
         case 15:
             return launch_dma<2, 2, 4, 4, 4, 7>(a, st);  // 128 x 128, fragment prefetch in a pinned program order
+        case 16:
+            if (a.K % 128 != 0) {
+                return launch_dma<2, 2, 4, 4, 4, 7>(a, st);
+            }
+            return launch_dma<2, 2, 4, 4, 4, 8>(a, st);  // the same by two groups of four waves on alternate K tiles
         default:
             break;
     }

@@ -118,7 +118,7 @@ def test_mmm_all_outputs_device(torch_mod, oracle, M, K, N):
     assert np.array_equal(got, oracle.mmm(A, W, off, Cin, DT_I32))
 
 
-@pytest.mark.parametrize("tile", [0, 2, 7, 10, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [0, 2, 7, 10, 11, 12, 13, 14, 15, 16])
 def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
     """Each GEMM kernel (general, register-staged tiles, LDS-DMA pipelines) is forced in turn on
     shapes with ragged M / N edges, one and many K tiles, and all four epilogues."""
