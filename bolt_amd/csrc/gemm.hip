@@ -2237,7 +2237,7 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             tile = k64 ? 15 : 2;  // 15 against 10 (the compiler's order): 8.4 / 17.9 / 14.1 against 9.5 / 20.0 / 16.4 us at 4096 x 768 x 768, 4096 x 3072 x 768, 2048^3
             // long K on a grid that leaves CUs idle: two wave groups per tile on alternate K tiles (17.0 against 18.1 us at
             // 4096 x 3072 x 768; slower for short K and for grids of several rounds)
-            if (tile == 15 && a.K % 128 == 0 && a.K >= 2048 && b128 <= 256) {
+            if (tile == 15 && a.K % 128 == 0 && a.K >= 2048 && b128 <= 224) {
                 tile = 16;
             }
         }
