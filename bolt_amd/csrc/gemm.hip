@@ -535,6 +535,55 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
 #undef BG_LOAD_CIN
 }
 
+// Full-tile epilogue for u8 results of a matrix product, through a wave-private LDS panel of 16 rows x 64 bytes
+// (pitch 80: the 4-byte writes of the fragment layout and the 16-byte reads of the row layout are both free of bank
+// conflicts). Straight from the accumulators a store instruction puts 4 bytes of a different row into every lane,
+// 64 pieces for the address unit; from the panel lane 4 r + c stores 16 bytes of row r, a quad = one 64-byte piece.
+template <int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_rows_lds_u8(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
+{
+    static_assert(TN == 4, "a wave's tile row must be 64 columns");
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const float factor = epi_factor(a.epi);
+    uint32_t base[TN * 4];
+    {
+        uint32_t nn[TN * 4];
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                nn[y * 4 + c] = n0 + (wn * TN + y) * 16 + 4 * g + c;
+            }
+        }
+        column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, a.fold_scale, nn, base);
+    }
+    constexpr uint32_t kPitch = 80;
+    uint8_t *pan = smem + wave * (16 * kPitch);
+    uint8_t *wr = pan + i * kPitch + g * 4;  // + 16 * y
+    const uint8_t *rd = pan + (lane >> 2) * kPitch + (lane & 3) * 16;
+    uint8_t *out = (uint8_t *)a.C + (size_t)(m0 + wm * TM * 16 + (lane >> 2)) * a.N + n0 + wn * 64 + (lane & 3) * 16;
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            unsigned b[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                b[c] = epi_u8((int)((uint32_t)acc[x][y][c] + base[y * 4 + c]), factor);  // int32 wrap
+            }
+            *(uint32_t *)(wr + 16 * y) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        const v4i row = *(const v4i *)rd;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        *(v4i *)(out + (size_t)x * 16 * a.N) = row;
+    }
+}
+
 // EPI_U8_GELU_DYN: the FullyConnected in front of a GELU whose result the next FullyConnected wants quantised with a
 // tensor-wide dynamic scale. Written as separate kernels that is an fp32 matrix stored, read for max|gelu|, and read
 // again to be quantised; here the accumulators never leave the registers:
@@ -664,6 +713,12 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
             } else {
                 epilogue_rows_lds<MODE, WM, WN, TM, TN, 0, false>(a, acc, smem, lane, wave, m0, n0);
             }
+            return;
+        }
+    }
+    if constexpr (!CONV && MODE == EPI_U8 && TN == 4) {
+        if (full && smem && (a.N & 15) == 0 && ((uintptr_t)a.C & 15) == 0) {
+            epilogue_rows_lds_u8<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             return;
         }
     }
