@@ -49,8 +49,9 @@ const char *bolt_gfx950_last_error(void);
  * kernels (256x256 fragment-prefetch, 128x128 fragment-prefetch, 256x256 ping-pong; need
  * K % 64 == 0), 12 the 256x256 ping-pong kernel that requests A in whole 128-byte lines (needs
  * K % 128 == 0, else it runs as 11), 13 the same with the B fragments loaded straight into registers instead of
- * through LDS (K % 128 == 0, else 11), 14 the few-rows kernel; a variant whose shape requirement fails falls back to
- * the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
+ * through LDS (K % 128 == 0, else 11), 14 the few-rows kernel, 15 the 128x128 fragment-prefetch kernel with the
+ * program order of a K step written out (K % 64 == 0), 16 the same run by two groups of four waves on alternate
+ * K tiles (K % 128 == 0, else 15); a variant whose shape requirement fails falls back to the general kernel. "conv_panel": which kernel a convolution with up to 64 output channels and
  * K <= 1024 uses: 4 (default) / 2 the filter-panel-in-LDS kernel with 64 / 32 pixels per wave, 0 the
  * shared-pipeline kernel. "conv_direct": whether that filter-panel kernel gathers from the caller's
  * u8 tensor in place when the channel count is a multiple of 16: 1 (default) for int32 and fp32
