@@ -1014,6 +1014,7 @@ __global__ __launch_bounds__(WM *WN * 64 * (PIPE == 8 ? 2 : 1), PIPE == 8 ? 1 : 
         // 16 consecutive lanes = 16 rows) spreads over all 64 banks.
         static_assert(PIPE != 3 || (!CONV && !FP4 && WM * WN == 8 && STAGES == 5 && T::kAFrags == 16 && T::kBFrags == 16),
             "the whole-line loop is written for 256 x 256 matrix tiles in 160 KB of LDS");
+        static_assert(PIPE != 3 || (WM == 2 && WN == 4 && TM == 8 && TN == 4), "checked for eight waves of 128 x 64 only");
         constexpr uint32_t kASlot = T::kAFrags * 2048, kBBase = 3 * kASlot, kBSlot = T::kBFrags * 1024;
         constexpr int kQA2 = 2 * T::kAFrags / T::kWaves;  // requests per wave and tile pair
         constexpr int kQB = T::kBFrags / T::kWaves;       // requests per wave and tile
@@ -1144,6 +1145,7 @@ __global__ __launch_bounds__(WM *WN * 64 * (PIPE == 8 ? 2 : 1), PIPE == 8 ? 1 : 
         // 128 bytes per cycle was as long as the 1024 cycles the tile's MFMAs take.
         static_assert(PIPE != 4 || (!CONV && !FP4 && WM * WN == 8 && STAGES == 3 && T::kAFrags == 16 && T::kBFrags == 16 && TN == 4),
             "the register-B loop is written for 256 x 256 matrix tiles");
+        static_assert(PIPE != 4 || (WM == 2 && WN == 4 && TM == 8 && TN == 4), "checked for eight waves of 128 x 64 only");
         constexpr uint32_t kASlot = T::kAFrags * 2048;
         constexpr int kQA2 = 2 * T::kAFrags / T::kWaves;  // A requests per wave and tile pair
         static_assert(3 * kASlot == (uint32_t)T::kLdsBytes, "LDS layout");
