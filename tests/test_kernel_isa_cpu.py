@@ -57,3 +57,39 @@ def test_no_spill_stores_inside_the_register_b_loop(gemm_asm):
         assert len(text_loads) >= 12, "%s: the B loads issued as text are missing from the loop" % name
         stores = [ins for ins in region if ins.startswith("scratch_store")]
         assert not stores, "%s: the compiler spills inside the loop with hand-counted loads: %s" % (name, stores[:3])
+
+
+def test_pinned_order_loops_keep_their_order(gemm_asm):
+    """The 128 x 128 loops whose K step is written out instruction by instruction (PIPE 7, and PIPE 8 = the same by two
+    wave groups): their point is that every fragment read, tile request and re-bias sits BEHIND an MFMA, so that a
+    wave alone on its SIMD issues it while the matrix pipe is busy. Checked on the generated code: inside the K loop no
+    MFMA is preceded by more than a handful of vector / memory instructions, nothing spills, and a step's four
+    tile requests and (but for a walk's last step) eight fragment reads are all there."""
+    ks = kernels(gemm_asm)
+    for pipe in (7, 8):
+        names = [n for n in ks if re.search(r"gemm_u8s8_dma_kernelILi2ELi2ELi4ELi4ELi4ELi%dE" % pipe, n)]
+        assert names, "no instantiation of the pinned-order loop (PIPE %d)" % pipe
+        for name in names:
+            body = ks[name]
+            bars = [i for i, ins in enumerate(body) if ins == "s_barrier"]
+            # a K step = the stretch between two barriers that holds exactly 16 MFMAs
+            steps = []
+            for b0, b1 in zip(bars, bars[1:]):
+                seg = body[b0 + 1:b1]
+                if sum(ins.startswith("v_mfma_i32_16x16x64_i8") for ins in seg) == 16:
+                    steps.append(seg)
+            assert len(steps) >= 2, "%s: found %d K steps of 16 MFMAs" % (name, len(steps))
+            for seg in steps:
+                assert not any(ins.startswith("scratch_") for ins in seg), name
+                assert sum(ins.startswith("global_load_lds_dwordx4") for ins in seg) == 4, name
+                # (the last step of a walk reads no fragments: nothing would use them)
+                assert sum(ins.startswith("ds_read_b128") for ins in seg) in (0, 8), name
+                run = 0  # vector ALU / LDS / memory instructions since the last MFMA (scalar ones issue beside them)
+                first = True
+                for ins in seg:
+                    if ins.startswith("v_mfma"):
+                        limit = 4 if first else 9  # in front of the first MFMA only address arithmetic may stand
+                        assert run <= limit, "%s: %d vector instructions in front of an MFMA" % (name, run)
+                        run, first = 0, False
+                    elif ins.startswith(("v_", "ds_", "global_", "buffer_")):
+                        run += 1
