@@ -93,3 +93,4 @@ def test_pinned_order_loops_keep_their_order(gemm_asm):
                         run, first = 0, False
                     elif ins.startswith(("v_", "ds_", "global_", "buffer_")):
                         run += 1
+
