@@ -2285,16 +2285,29 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
             // ping-pong: 12 % faster than the fragment-prefetch loop at 8192^3, level elsewhere; with A requested in
             // whole lines another 4 % at 8192^3 and level at 4096^3 (needs K % 128 == 0 and 160 KB of LDS)
             tile = (a.K % 128 == 0) ? 12 : 11;
-            // up to two rounds of tiles the register-B form is 6-18 % faster (4096^3, the encoder's FFN shapes); long
-            // multi-round launches run at the clock the power limit allows either way and measure level
-            if (tile == 12 && b256 <= 512) {
+            // within one round of tiles the register-B form is level or ahead (4096^3, the encoder's FFN shapes); from
+            // two rounds on the LDS form is (8192 x 4096 x 4096: 122.5 against 128.5 us)
+            if (tile == 12 && b256 <= 256) {
                 tile = 13;
+            }
+            // 256 x 256 tiles that leave CUs idle while the 128 x 128 ones come out at exactly two per CU: the smaller
+            // tiles win by 20-29 % (2048 x 4096 x 4096 39.8 against 47.2 us, 8192 x 1024 x 1024 16.4 against 20.6,
+            // 4096 x 2048 x 2048 25.0 against 29.5); with a ragged last round (576 tiles: 3072^3, 4096 x 768 x 2304)
+            // they are level or behind
+            if (b256 < 256 && b128 <= 512 && a.epi.mode != EPI_U8_GELU_DYN) {  // (that epilogue needs the large tiles)
+                tile = 15;
+            }
+            // several rounds of large tiles with a short K spend half their time in prologues and epilogues; two small
+            // workgroups per CU overlap those with each other's K loops (8192 x 1024 x 4096 53.2 against 58.9 us,
+            // 8192 x 768 x 2304 28.7 against 34.0)
+            if (b256 > 256 && a.K <= 1024 && a.epi.mode != EPI_U8_GELU_DYN) {
+                tile = 15;
             }
         } else if (b128 >= 32 || (a.M >= 128 && a.N >= 128)) {
             tile = k64 ? 15 : 2;  // 15 against 10 (the compiler's order): 8.4 / 17.9 / 14.1 against 9.5 / 20.0 / 16.4 us at 4096 x 768 x 768, 4096 x 3072 x 768, 2048^3
             // long K on a grid that leaves CUs idle: two wave groups per tile on alternate K tiles (17.0 against 18.1 us at
             // 4096 x 3072 x 768; slower for short K and for grids of several rounds)
-            if (tile == 15 && a.K % 128 == 0 && a.K >= 2048 && b128 <= 224) {
+            if (tile == 15 && a.K % 128 == 0 && ((a.K >= 2048 && b128 <= 224) || (a.K >= 4096 && b128 <= 256))) {
                 tile = 16;
             }
         }
