@@ -2340,6 +2340,24 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
         }
         return launch_dma<2, 4, 8, 4, 4, 2, false, false, true>(a, st);
     }
+    // Few rows: the kernel that gives a 16-column weight panel to a workgroup and splits K over its 8 waves beats the
+    // 128 x 128 tiles while it has at most one workgroup per CU -- 16 x 4096 x 4096 7.2 against 16.2 us, 256 x 3072 x 768
+    // 8.8 against 13.1, 256 x 4096 x 1024 10.8 against 15.6 -- and loses beyond (256 x 4096 x 4096: 34.7 against 16.9).
+    // Both sides are priced from measurements: 5.8 us + 21 ns per K tile and 16-row block of a workgroup's 64 rows
+    // against 4.5 us + 0.18 us per K tile and round of 128 x 128 tiles.
+    if (g_force_tile < 0 && dma_ok && (tile == 15 || tile == 16) && a.epi.mode != EPI_U8_GELU_DYN) {
+        const uint64_t wgs = (uint64_t)((a.N + 15) / 16) * ((a.M + 63) / 64);
+        if (wgs <= 256) {
+            const uint32_t rows16 = (a.M + 15) / 16 < 4 ? (a.M + 15) / 16 : 4, ks = a.K / 64;
+            const uint64_t b128 = (uint64_t)((a.M + 127) / 128) * ((a.N + 127) / 128);
+            const float few = 5.8f + 0.0214f * (float)ks * (float)rows16;
+            const float tiled = 4.5f + 0.18f * (float)ks * (float)((b128 + 255) / 256);
+            if (few < tiled) {
+                hipLaunchKernelGGL(gemm_u8s8_skinny_kernel, dim3((a.N + 15) / 16, (a.M + 63) / 64), dim3(512), 0, st, a);
+                return hipGetLastError();
+            }
+        }
+    }
     switch (tile) {
         case 2:
             return launch_tiled<2, 2, 4, 4>(a, st);  // 128 x 128
