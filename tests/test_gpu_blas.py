@@ -150,6 +150,46 @@ def test_mmm_every_kernel_variant(torch_mod, oracle, tile):
         L.bolt_gfx950_set_option(b"gemm_tile", -1)
 
 
+@pytest.mark.parametrize("shape", [(4096, 3072, 768), (4096, 768, 768), (2048, 4096, 4096), (8192, 1024, 1024),
+                                   (256, 3072, 768), (16, 4096, 4096)])
+def test_mmm_variants_agree_at_full_size(torch_mod, oracle, shape):
+    """The shapes whose kernel the launcher picks by measurement (128 x 128 tiles in pinned order, the two-group form,
+    256 x 256 tiles, the few-rows kernel): at full size every variant and the launcher's own choice must give the same
+    int32 and the same u8 bytes, and a sample of rows must equal the oracle."""
+    torch = torch_mod
+    M, K, N = shape
+    L = capi.lib()
+    g = torch.Generator(device="cuda").manual_seed(M + K + N)
+    A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+    W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+    off = blob[rhs:rhs + 4 * N].clone()
+    ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+    r = np.float32(1.0 / (64.0 * np.sqrt(K)))
+    outs = {}
+    try:
+        for tile in (-1, 12, 13, 14, 15, 16):
+            say("full-size variant", tile, M, K, N)
+            capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
+            Ci = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+            capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Ci, tensor2df(DT_I32, DF_NORMAL, M, N), None), "mmm i32")
+            Cu = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+            capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cu, tensor2df(DT_U8_Q, DF_NORMAL, M, N), [-1, r]), "mmm u8")
+            capi.check(L.bolt_gfx950_synchronize(), "sync")
+            outs[tile] = (Ci, Cu)
+    finally:
+        L.bolt_gfx950_set_option(b"gemm_tile", -1)
+    for tile, (Ci, Cu) in outs.items():
+        assert torch.equal(Ci, outs[13][0]), tile
+        assert torch.equal(Cu, outs[13][1]), tile
+    rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(1).integers(0, M, 6)]))
+    Ah, Wh, offh = A[torch.from_numpy(rows).cuda()].cpu().numpy(), W.cpu().numpy(), off.cpu().numpy().view(np.int32)
+    want = oracle.mmm(Ah, Wh, offh, np.zeros((len(rows), N), np.int32), DT_I32)
+    assert np.array_equal(outs[-1][0].cpu().numpy()[rows], want)
+    wantu = oracle.mmm(Ah, Wh, offh, np.zeros((len(rows), N), np.uint8), DT_U8_Q, scale=[-1, r])
+    assert np.array_equal(outs[-1][1].cpu().numpy()[rows], wantu)
+
+
 def test_mmm_full_size_properties(torch_mod, oracle):
     """At the square-sweep size (4096^3) the oracle would take minutes, so the result is pinned by
     size-independent properties: linearity in A (A1 + A2 in the signed domain), rows reproduced by
