@@ -29,7 +29,8 @@ def make_case(oracle, M, K, N, seed):
 
 
 @pytest.mark.parametrize("device_mode", [False, True])
-@pytest.mark.parametrize("M,K,N", [(64, 1024, 1024), (1, 1024, 1024), (1, 77, 100), (5, 40, 33), (128, 768, 768)])
+@pytest.mark.parametrize("M,K,N", [(64, 1024, 1024), (1, 1024, 1024), (1, 77, 100), (5, 40, 33), (128, 768, 768),
+                                   (16, 2048, 1024), (256, 3072, 768), (320, 1024, 512)])  # the last three: few rows, K deep enough for the column-panel kernel to be chosen over tiles
 def test_fully_connected(torch_mod, oracle, device_mode, M, K, N):
     torch = torch_mod
     xq, sI, W, sW, bias = make_case(oracle, M, K, N, 20240601 + M)
