@@ -190,6 +190,43 @@ def test_mmm_variants_agree_at_full_size(torch_mod, oracle, shape):
     assert np.array_equal(outs[-1][1].cpu().numpy()[rows], wantu)
 
 
+def test_mmm_launcher_choice_equals_general_kernel(torch_mod):
+    """Sixty random shapes (few rows to 2 048, 1 to 4 096 columns, K a multiple of 16 or 64 up to 4 480) through whatever
+    kernel the launcher picks -- few-rows kernel, 128 x 128 tiles, two-group form, 256 x 256 tiles, register-staged tiles
+    -- against the plain general kernel: the same int32 (accumulating into C), fp32 and u8 bits."""
+    torch = torch_mod
+    L = capi.lib()
+    rng = np.random.default_rng(11)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    try:
+        for it in range(60):
+            M = int(rng.choice([rng.integers(1, 20), rng.integers(20, 300), rng.integers(300, 1200), rng.choice([128, 256, 512, 1024, 2048])]))
+            N = int(rng.choice([rng.integers(1, 80), rng.integers(80, 600), rng.integers(600, 1500), rng.choice([256, 512, 768, 1024, 2304, 3072, 4096])]))
+            K = int(rng.choice([64 * rng.integers(1, 12), 64 * rng.integers(12, 70), rng.choice([768, 1024, 2048, 3072, 4096]), 16 * rng.integers(4, 100)]))
+            say("launcher choice", it, M, K, N)
+            A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+            W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+            blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            off = blob[rhs:rhs + 4 * N].clone()
+            ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+            r = np.float32(1.0 / (64.0 * np.sqrt(K)))
+            outs = []
+            for tile in (-1, 0):
+                capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
+                Ci = torch.full((M, N), 7, dtype=torch.int32, device="cuda")
+                capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Ci, tensor2df(DT_I32, DF_NORMAL, M, N), None), "i32")
+                Cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+                capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cf, tensor2df(DT_F32, DF_NORMAL, M, N), [3.5]), "f32")
+                Cu = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+                capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cu, tensor2df(DT_U8_Q, DF_NORMAL, M, N), [-1, r]), "u8")
+                capi.check(L.bolt_gfx950_synchronize(), "sync")
+                outs.append((Ci, Cf.view(torch.int32), Cu))
+            for a_, b_ in zip(outs[0], outs[1]):
+                assert torch.equal(a_, b_), (M, K, N)
+    finally:
+        L.bolt_gfx950_set_option(b"gemm_tile", -1)
+
+
 def test_mmm_full_size_properties(torch_mod, oracle):
     """At the square-sweep size (4096^3) the oracle would take minutes, so the result is pinned by
     size-independent properties: linearity in A (A1 + A2 in the signed domain), rows reproduced by
