@@ -239,6 +239,29 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                 del tmp, out
             del A, W, blob
         res["gemm_int8"] = gemm
+        # -- few rows (a serving batch of 16-256 tokens against a layer's weights): these go to the kernel that hands every
+        #    workgroup a 16-column weight panel and splits K over its waves, where it prices below the 128 x 128 tiles
+        few = []
+        for (M, K, N) in ((16, 4096, 4096), (64, 4096, 4096), (256, 3072, 768), (256, 4096, 1024), (256, 4096, 4096)):
+            A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
+            W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
+            blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            bias = torch.randn(N, device=dev, generator=g) * 0.1
+            ad = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+            fdesc = tensor2df(DT_I8, DF_NKNxKx, K, N)
+            nbytes = host.fully_connected_tmp_bytes(M, K, N, DF_NKNxKx, DT_F32, AMD_GFX950_DEVICE)
+            tmp = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            out = torch.empty((M, N), dtype=torch.float32, device=dev)
+            so = C.c_float(-1.0)
+            od = tensor2df(DT_F32, DF_NORMAL, M, N)
+            t = timed(lambda: capi.check(L.fully_connected_gfx950(ad, host.ptr(A), 30.0, fdesc, host.ptr(blob), 100.0,
+                                                                  tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp),
+                                                                  od, host.ptr(out), C.byref(so), AMD_GFX950_DEVICE),
+                                         "fully_connected"), 50)
+            few.append({"M": M, "K": K, "N": N, "path": "fully_connected", "out": "f32", "ms": t,
+                        "weight_gbps": N * K / t / 1e6, "tops": 2.0 * M * N * K / t / 1e9})
+            del A, W, blob, tmp, out
+        res["gemm_int8_few_rows"] = few
     if want("gemm_data"):
         from bolt_amd.capi import AMD_GFX950_DEVICE, DT_I8, tensor1d
         # -- the same kernel against what the device sustains: the clock it holds depends on how many operand
