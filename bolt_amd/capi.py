@@ -217,7 +217,7 @@ SIGNATURES = {
     "dequantize_int4_weight_gfx950": (C.c_int, [C.c_int, C.c_float, _vp, _vp, C.c_int]),
     "dequantize_int4_int8_gfx950": (C.c_int, [C.c_int, _vp, _vp, C.c_int]),
     "dequantize_int4_u8_q_gfx950": (C.c_int, [C.c_int, _vp, _vp, C.c_int]),
-    "bolt_gfx950_operator_scales": (C.c_int, [_vp, _u32, C.c_int, C.c_float, C.c_float, _f32p, C.POINTER(C.c_int)]),
+    "bolt_gfx950_operator_scales": (C.c_int, [C.c_int, _vp, _u32, C.c_int, C.c_int, C.c_float, C.c_float, _f32p, C.POINTER(C.c_int)]),
     "convolution_transform_filter_bytes_bnn_gfx950": (C.c_int, [TensorDesc, _u32p, C.c_int]),
     "convolution_transform_filter_bnn_gfx950": (C.c_int, [TensorDesc, _vp, C.POINTER(TensorDesc), _vp, C.c_int]),
     "convolution_infer_forward_tmp_bytes_bnn_gfx950": (C.c_int, [TensorDesc, ConvolutionParamSpec, _u32p, C.c_int]),

@@ -148,34 +148,52 @@ EE dequantize_int4_u8_q_gfx950(int num, INT8 *q, UINT8 *d, Arch arch)
     return expand(num, 1.0f, q, 1, 2, d, arch);
 }
 
-EE bolt_gfx950_operator_scales(const QuantSpec *featureScale, U32 numQuantFeature, DataType inputDataType,
-    F32 inputTensorScale, F32 filterScale, F32 scales[3], int *labelledNoQuant)
+EE bolt_gfx950_operator_scales(int operatorKind, const QuantSpec *featureScale, U32 numQuantFeature, DataType inputDataType,
+    DataType outputDataType, F32 inputTensorScale, F32 filterScale, F32 scales[3], int *labelledNoQuant)
 {
     if (!scales || (numQuantFeature && !featureScale)) {
         return NULL_POINTER;
+    }
+    if (operatorKind != BOLT_GFX950_OP_CONVOLUTION && operatorKind != BOLT_GFX950_OP_FULLY_CONNECTED &&
+        operatorKind != BOLT_GFX950_OP_DECONVOLUTION) {
+        return NOT_SUPPORTED;
     }
     for (U32 i = 0; i < numQuantFeature; ++i) {
         if (featureScale[i].num_scale < 1 || !featureScale[i].scale) {
             return NOT_MATCH;
         }
     }
-    // inference/engine/include/cpu/convolution_cpu.hpp:143-157 (fully_connected_cpu.hpp and deconvolution_cpu.hpp:65-84
-    // apply the same rule): the input scale is the producing tensor's unless the input still has to be quantised and
-    // the record carries a positive calibrated scale; the output scale is the last record's, -2 meaning "leave it to
-    // the operator" (dynamic, -1)
+    const bool inQuantised = inputDataType == DT_I8 || inputDataType == DT_U8_Q;
+    const bool outQuantised = outputDataType == DT_I8 || outputDataType == DT_U8_Q;
+    const F32 first = numQuantFeature ? featureScale[0].scale[0] : 0.0f;
+    const F32 last = numQuantFeature ? featureScale[numQuantFeature - 1].scale[0] : 0.0f;
     scales[0] = inputTensorScale;
-    if (inputDataType != DT_I8 && inputDataType != DT_U8_Q && numQuantFeature > 0 && featureScale[0].scale[0] > 0) {
-        scales[0] = featureScale[0].scale[0];
-    }
-    if (numQuantFeature > 0 && featureScale[numQuantFeature - 1].scale[0] != -2) {
-        scales[1] = featureScale[numQuantFeature - 1].scale[0];
-    } else {
-        scales[1] = -1;
-    }
     scales[2] = filterScale;
+    if (operatorKind == BOLT_GFX950_OP_CONVOLUTION) {
+        // inference/engine/include/cpu/convolution_cpu.hpp:143-157: one record is enough for the calibrated input scale;
+        // the last record is the output scale whatever the output type, -2 there (or no record) leaves it dynamic
+        if (!inQuantised && numQuantFeature > 0 && first > 0) {
+            scales[0] = first;
+        }
+        scales[1] = (numQuantFeature > 0 && last != -2) ? last : -1.0f;
+    } else {
+        // fully_connected_cpu.hpp:92-103 and deconvolution_cpu.hpp:70-84: the calibrated input scale needs MORE than one
+        // record (a single record is the output's), the output scale is set only for a quantised output type, and the
+        // last record goes through as it is (-2 included)
+        if (!inQuantised && numQuantFeature > 1 && first > 0) {
+            scales[0] = first;
+        }
+        if (outQuantised) {
+            scales[1] = numQuantFeature > 0 ? last : -1.0f;
+        } else {
+            // FullyConnected leaves the output tensor's scale alone (reported as -1: nothing to set); the deconvolution's
+            // `F32 scales[3] = {-1}` leaves a zero in slot 1 (deconvolution_cpu.hpp:65)
+            scales[1] = operatorKind == BOLT_GFX950_OP_DECONVOLUTION ? 0.0f : -1.0f;
+        }
+    }
     if (labelledNoQuant) {
         // inference/engine/include/operator.hpp:164-169: a first record of 0 labels the operator as not quantised
-        *labelledNoQuant = (numQuantFeature != 0 && featureScale[0].scale[0] == 0) ? 1 : 0;
+        *labelledNoQuant = (numQuantFeature != 0 && first == 0) ? 1 : 0;
     }
     return SUCCESS;
 }

@@ -287,15 +287,26 @@ EE dequantize_int8_weight_gfx950(int num, F32 scale, INT8 *q, F32 *d, Arch arch)
 EE dequantize_int4_weight_gfx950(int num, F32 scale, INT8 *q, F32 *d, Arch arch);
 EE dequantize_int4_int8_gfx950(int num, INT8 *q, INT8 *d, Arch arch);
 EE dequantize_int4_u8_q_gfx950(int num, INT8 *q, UINT8 *d, Arch arch);
-/* The rule by which the engine's int8 operators turn the QuantSpec records a .bolt model stores for them
+/* The rules by which the engine's int8 operators turn the QuantSpec records a .bolt model stores for them
  * (OperatorSpec::feature_scale, common/uni/include/parameter_spec.h:753-756; copied by Operator::init_feature_scale,
- * inference/engine/include/operator.hpp:139-150) into the scales[3] = {input, output, filter} they pass down
- * (inference/engine/include/cpu/convolution_cpu.hpp:143-157, deconvolution_cpu.hpp:65-84): a calibrated input scale
- * is used only while the input is not yet quantised; the last record is the output scale, -2 there (or no record)
- * leaves it dynamic (-1); *labelledNoQuant (optional) = 1 when the first record is 0 (operator.hpp:164-169).
+ * inference/engine/include/operator.hpp:139-150) into scales[3] = {input, output, filter}. The three operator
+ * classes differ, and operatorKind selects whose rule is applied:
+ *   BOLT_GFX950_OP_CONVOLUTION      (convolution_cpu.hpp:143-157) input: the first record, if positive and the input is
+ *       not yet I8 / U8_Q, else the tensor's own scale; output: the last record, -2 there or no record -> -1 (dynamic),
+ *       whatever the output type.
+ *   BOLT_GFX950_OP_FULLY_CONNECTED  (fully_connected_cpu.hpp:92-103) input: as above but only with MORE than one record;
+ *       output: only for an I8 / U8_Q output type, the last record unchanged (-2 stays -2), no record -> -1; for
+ *       any other output type the operator leaves the tensor's scale alone and scales[1] is returned as -1.
+ *   BOLT_GFX950_OP_DECONVOLUTION    (deconvolution_cpu.hpp:65-84) as FullyConnected; for a non-quantised output type
+ *       scales[1] is the 0 that `F32 scales[3] = {-1}` leaves there.
+ * MatMul has two inputs and three records (matmul_cpu.hpp:46-56) and is not covered.
+ * *labelledNoQuant (optional) = 1 when the first record is 0 (operator.hpp:164-169).
  * Pure host logic: no GPU is touched, no Arch. A clip value c from the tool's scale table is stored as 127 / c. */
-EE bolt_gfx950_operator_scales(const QuantSpec *featureScale, U32 numQuantFeature, DataType inputDataType,
-    F32 inputTensorScale, F32 filterScale, F32 scales[3], int *labelledNoQuant);
+#define BOLT_GFX950_OP_CONVOLUTION 0
+#define BOLT_GFX950_OP_FULLY_CONNECTED 1
+#define BOLT_GFX950_OP_DECONVOLUTION 2
+EE bolt_gfx950_operator_scales(int operatorKind, const QuantSpec *featureScale, U32 numQuantFeature, DataType inputDataType,
+    DataType outputDataType, F32 inputTensorScale, F32 filterScale, F32 scales[3], int *labelledNoQuant);
 
 /* ---- 1-bit (XNOR / DoReFa) convolution ---------------------------------------------- */
 /* compute/tensor/src/cpu/arm/bnn/convolution.cpp:16-72 (convolution_bnn), filter transform

@@ -109,29 +109,66 @@ def test_load_time_expansion(oracle, ref, n):
 
 
 def test_operator_scales_rule():
-    """bolt_gfx950_operator_scales (pure host logic) against the engine's rule
-    (inference/engine/include/cpu/convolution_cpu.hpp:143-157, operator.hpp:164-169), case by case."""
+    """bolt_gfx950_operator_scales (pure host logic) against the three rules of the engine's operator classes, each
+    written out here from the header it comes from and evaluated case by case:
+      convolution     inference/engine/include/cpu/convolution_cpu.hpp:143-157
+      fully connected inference/engine/include/cpu/fully_connected_cpu.hpp:92-103
+      deconvolution   inference/engine/include/cpu/deconvolution_cpu.hpp:65-84
+    and operator.hpp:164-169 for the no-quant label."""
     from bolt_amd import capi
-    from bolt_amd.capi import DT_F32, DT_U8_Q
+    from bolt_amd.capi import DT_F32, DT_I8, DT_U8_Q
+    CONV, FC, DECONV = 0, 1, 2
 
     class QuantSpec(C.Structure):
         _fields_ = [("num_scale", C.c_int32), ("scale", C.POINTER(C.c_float))]
     assert C.sizeof(QuantSpec) == 16
 
-    def call(records, idt, in_scale, f_scale=F(50.0)):
+    def call(kind, records, idt, odt, in_scale, f_scale=F(50.0)):
         keep = [(C.c_float * len(r))(*r) for r in records]
         arr = (QuantSpec * max(1, len(records)))()
         for i, k in enumerate(keep):
             arr[i].num_scale, arr[i].scale = len(k), C.cast(k, C.POINTER(C.c_float))
         out, noq = (C.c_float * 3)(), C.c_int(-1)
-        e = capi.lib().bolt_gfx950_operator_scales(C.cast(arr, C.c_void_p) if records else None, len(records), idt,
+        e = capi.lib().bolt_gfx950_operator_scales(kind, C.cast(arr, C.c_void_p) if records else None, len(records), idt, odt,
                                                    in_scale, f_scale, out, C.byref(noq))
         assert e == capi.SUCCESS
         return [F(v) for v in out], noq.value
 
-    assert call([], DT_F32, F(-1.0)) == ([F(-1.0), F(-1.0), F(50.0)], 0)                        # nothing stored: all dynamic
-    assert call([[12.5], [31.0]], DT_F32, F(-1.0)) == ([F(12.5), F(31.0), F(50.0)], 0)          # calibrated in and out
-    assert call([[12.5], [31.0]], DT_U8_Q, F(9.0)) == ([F(9.0), F(31.0), F(50.0)], 0)           # already quantised input keeps its own scale
-    assert call([[12.5], [-2.0]], DT_F32, F(-1.0)) == ([F(12.5), F(-1.0), F(50.0)], 0)          # -2: output left to the operator
-    assert call([[0.0], [31.0]], DT_F32, F(-1.0)) == ([F(-1.0), F(31.0), F(50.0)], 1)           # first record 0: labelled no-quant
-    assert call([[127.0 / 2.5]], DT_F32, F(-1.0))[0][:2] == [F(127.0 / 2.5), F(127.0 / 2.5)]   # one record (clip 2.5) serves both ends
+    def header_rule(kind, fs, idt, odt, in_scale, f_scale):
+        """the three run() bodies, statement by statement"""
+        quant = (DT_I8, DT_U8_Q)
+        s = [None, None, f_scale]
+        s[0] = in_scale
+        if kind == CONV:
+            if idt not in quant and len(fs) > 0 and fs[0][0] > 0:
+                s[0] = F(fs[0][0])
+            s[1] = F(fs[-1][0]) if (len(fs) > 0 and fs[-1][0] != -2) else F(-1)
+        else:
+            if len(fs) > 1 and fs[0][0] > 0 and idt not in quant:
+                s[0] = F(fs[0][0])
+            if odt in quant:
+                s[1] = F(fs[-1][0]) if len(fs) > 0 else F(-1)
+            else:
+                s[1] = F(0) if kind == DECONV else F(-1)   # `F32 scales[3] = {-1}`: slot 1 starts at 0 / tensor untouched
+        return s
+
+    cases = ([], [[12.5], [31.0]], [[12.5], [-2.0]], [[0.0], [31.0]], [[127.0 / 2.5]], [[-2.0]], [[12.5], [7.0], [31.0]])
+    for kind in (CONV, FC, DECONV):
+        for fs in cases:
+            for idt, in_scale in ((DT_F32, F(-1.0)), (DT_U8_Q, F(9.0)), (DT_I8, F(4.5))):
+                for odt in (DT_F32, DT_U8_Q, DT_I8):
+                    got, noq = call(kind, fs, idt, odt, in_scale)
+                    assert got == header_rule(kind, fs, idt, odt, in_scale, F(50.0)), (kind, fs, idt, odt)
+                    assert noq == (1 if (fs and fs[0][0] == 0) else 0)
+    # the cases the three classes disagree on, spelled out
+    one = [[127.0 / 2.5]]                                           # a single positive record (a clip value of 2.5)
+    assert call(CONV, one, DT_F32, DT_U8_Q, F(-1.0))[0][:2] == [F(127.0 / 2.5), F(127.0 / 2.5)]    # serves both ends
+    assert call(FC, one, DT_F32, DT_U8_Q, F(-1.0))[0][:2] == [F(-1.0), F(127.0 / 2.5)]             # output only
+    assert call(DECONV, one, DT_F32, DT_U8_Q, F(-1.0))[0][:2] == [F(-1.0), F(127.0 / 2.5)]
+    assert call(CONV, [[12.5], [-2.0]], DT_F32, DT_U8_Q, F(-1.0))[0][1] == F(-1.0)                 # -2 -> dynamic
+    assert call(FC, [[12.5], [-2.0]], DT_F32, DT_U8_Q, F(-1.0))[0][1] == F(-2.0)                   # passed through
+    assert call(DECONV, [[12.5], [-2.0]], DT_F32, DT_U8_Q, F(-1.0))[0][1] == F(-2.0)
+    assert call(CONV, [[12.5], [31.0]], DT_F32, DT_F32, F(-1.0))[0][1] == F(31.0)                  # whatever the output type
+    assert call(FC, [[12.5], [31.0]], DT_F32, DT_F32, F(-1.0))[0][1] == F(-1.0)                    # tensor left alone
+    assert call(DECONV, [[12.5], [31.0]], DT_F32, DT_F32, F(-1.0))[0][1] == F(0.0)
+    assert capi.lib().bolt_gfx950_operator_scales(7, None, 0, DT_F32, DT_F32, F(1.0), F(1.0), (C.c_float * 3)(), None) == capi.NOT_SUPPORTED
