@@ -299,7 +299,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                             "ms": t, "tops": tops, "frac_mfma_peak": tops / MFMA_PEAK_TOPS})
             del A, W, blob, tmp, out
         rate = {}
-        probe_so = os.path.join(ROOT, "bolt_amd", "libbolt_gfx950_benchprobe.so")   # bench-only library, not the product
+        probe_so = os.path.join(ROOT, "bench_probe", "libbench_probe.so")   # bench-only library, not the product
         if os.path.exists(probe_so):
             P = C.CDLL(probe_so)
             P.bench_probe_mfma_int8_rate.argtypes = [C.c_int, C.POINTER(C.c_float)]

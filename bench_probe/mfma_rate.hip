@@ -4,7 +4,7 @@
 // registers; there is no memory traffic inside the loop. With random operand bits the device lowers its
 // clock under the load, with all-zero operands it does not: the two figures bracket what any int8 kernel
 // can reach here, and the GEMM figures are read against them.
-// Built into its own bench-only library (libbolt_gfx950_benchprobe.so); the product library does not contain it.
+// Built into its own bench-only library (bench_probe/libbench_probe.so); the product library does not contain it.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 

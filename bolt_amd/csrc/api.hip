@@ -3148,7 +3148,10 @@ static EE encoder_run(const BoltEncoderLayerInt8 &L, const EncoderPlan &p, const
     HIP_TRY(gemm(xq, L.wo, H, H, sc + 1, L.so, L.bo, ao));
     HIP_TRY(launch_add_layernorm(hidden, ao, L.ln1_gamma, L.ln1_beta, T, H, h1, ws2, st, ws1));
     HIP_TRY(launch_quantize_f32(h1, T * H, xq, 1, ws2, 0.0f, nullptr, 0, sc + 2, st));
-    if (g_encoder_fused && gemm_gelu_dyn_fits(T, F, H)) {
+    // (the fused kernel is one of the tiled ones: it needs what launch_gemm_u8s8 asks of those -- operands on 16-byte
+    // boundaries -- and reads the per-column vectors 16 bytes at a time; anything else takes the unfused sequence)
+    const bool fused_aligned = ((((uintptr_t)L.w1) | ((uintptr_t)xq) | ((uintptr_t)L.s1) | ((uintptr_t)L.b1)) & 15) == 0;
+    if (g_encoder_fused && fused_aligned && gemm_gelu_dyn_fits(T, F, H)) {
         // FullyConnected + GELU + dynamic quantisation in one launch: the accumulators stay in registers across a
         // grid-wide agreement on max|gelu|; the [T, F] fp32 tensor is never written. Should that agreement be abandoned
         // (the CUs were held by other work), the kernel leaves the activated values in f, sets the status word, and

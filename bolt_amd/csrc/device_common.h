@@ -318,9 +318,10 @@ __device__ __forceinline__ uint32_t grid_sync_decide(unsigned long long *release
 // (values whose signed-integer order is the wanted order: non-negative floats' bits or ints). `lds`: 18 ints of
 // the workgroup's LDS; workgroups of whole waves, at most 16; blockIdx.x numbers the workgroups. Returns the
 // grid-wide maximum or kGridAbandoned, the same value in every thread of the grid.
-__device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int *lds)
+// `tid` = threadIdx.x; a kernel with no register to spare across its main loop hands in a value it has formed afresh.
+__device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int *lds, uint32_t tid)
 {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const uint32_t lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
     m = wave_reduce_max_i(m);
     if (lane == 0) {
         lds[wave] = m;
@@ -384,17 +385,22 @@ __device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int
     return (uint32_t)lds[17];
 }
 
+__device__ __forceinline__ uint32_t grid_max_sync(const GridSync &gs, int m, int *lds)
+{
+    return grid_max_sync(gs, m, lds, threadIdx.x);
+}
+
 
 // What a kernel does when grid_max_sync() was abandoned and it cannot leave the job to the host: every workgroup
 // first stores its partial result where a second pass can read it, then calls this (all threads); exactly one
 // workgroup -- the last to arrive -- gets true and does that second pass alone, the others return. No workgroup
 // waits for another, so it works whatever part of the grid is resident. The fences make the others' stores visible
 // to the one that continues. `lds`: the 18 ints grid_max_sync used.
-__device__ __forceinline__ bool grid_last_arrival(const GridSync &gs, int *lds)
+__device__ __forceinline__ bool grid_last_arrival(const GridSync &gs, int *lds, uint32_t tid)
 {
     __threadfence();
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
         const unsigned prev = __hip_atomic_fetch_add(gs.done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const bool last = prev + 1 == gs.blocks;
         if (last) {
@@ -410,11 +416,16 @@ __device__ __forceinline__ bool grid_last_arrival(const GridSync &gs, int *lds)
     return last;
 }
 
+__device__ __forceinline__ bool grid_last_arrival(const GridSync &gs, int *lds)
+{
+    return grid_last_arrival(gs, lds, threadIdx.x);
+}
+
 // Both passes of a dynamic fp32 -> u8 quantisation (scale 127 / max|x|, 1 for an all-zero tensor) by ONE workgroup of
 // whole waves (at most 16): the second pass of grid_last_arrival()'s survivor. `red`: 16 floats of LDS.
-__device__ __forceinline__ void quantize_f32_u8_alone(const float *x, uint32_t n, uint8_t *q, float *ds_out, float *red)
+__device__ __forceinline__ void quantize_f32_u8_alone(const float *x, uint32_t n, uint8_t *q, float *ds_out, float *red, uint32_t tid)
 {
-    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint32_t nt = blockDim.x;
     float m = 0.0f;
     for (uint32_t k = tid; k < n; k += nt) {
         const float a_ = fabsf(x[k]);
@@ -437,6 +448,11 @@ __device__ __forceinline__ void quantize_f32_u8_alone(const float *x, uint32_t n
     for (uint32_t k = tid; k < n; k += nt) {
         q[k] = (uint8_t)q_u8(x[k], s);
     }
+}
+
+__device__ __forceinline__ void quantize_f32_u8_alone(const float *x, uint32_t n, uint8_t *q, float *ds_out, float *red)
+{
+    quantize_f32_u8_alone(x, n, q, ds_out, red, threadIdx.x);
 }
 
 }  // namespace bg

@@ -601,10 +601,11 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
 {
     static_assert(TN == 4, "a wave's tile row must be 64 columns");
     const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t tid = wave * 64 + lane;  // the thread's index, from what the caller formed afresh (see there)
     const uint32_t wm = wave / WN, wn = wave % WN;
     const float sI = *a.epi.scaleI;
     if (a.clear_ws && blockIdx.x == 0) {
-        for (uint32_t k = threadIdx.x; k < kWsWords; k += blockDim.x) {
+        for (uint32_t k = tid; k < kWsWords; k += blockDim.x) {
             a.clear_ws[k] = 0;
         }
     }
@@ -642,9 +643,9 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
             }
         }
     }
-    const uint32_t outcome = grid_max_sync(a.sync, (int)__float_as_uint(amax), (int *)smem);
+    const uint32_t outcome = grid_max_sync(a.sync, (int)__float_as_uint(amax), (int *)smem, tid);
     if (outcome == kGridAbandoned) {
-        if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (blockIdx.x == 0 && tid == 0) {
             *a.status = 1u;
         }
 #pragma unroll
@@ -657,14 +658,14 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
             }
         }
         // no workgroup can wait for the others now; the last one to get here quantises the whole result alone
-        if (grid_last_arrival(a.sync, (int *)smem)) {
-            quantize_f32_u8_alone(a.C32, a.M * a.N, (uint8_t *)a.C, a.dscale_out, (float *)smem);
+        if (grid_last_arrival(a.sync, (int *)smem, tid)) {
+            quantize_f32_u8_alone(a.C32, a.M * a.N, (uint8_t *)a.C, a.dscale_out, (float *)smem, tid);
         }
         return;
     }
     const float mx = __uint_as_float(outcome);
     const float s = (mx == 0.0f) ? 1.0f : 127.0f / mx;  // resolve_scale with no caller's scale: max(0, 127 / max)
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (blockIdx.x == 0 && tid == 0) {
         *a.status = 0u;
         *a.dscale_out = s;
     }
@@ -1183,7 +1184,8 @@ __global__ __launch_bounds__(WM *WN * 64 * (PIPE == 8 ? 2 : 1), PIPE == 8 ? 1 : 
             /* issued as text, so that the compiler's own wait insertion does not see these loads: next to the */ \
             /* LDS-bound requests it would wait for ALL outstanding memory operations before the first use.   */ \
             /* The waits are the explicit vmcnt counts below; nothing reads FB between a load and its wait.    */ \
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(FB[y]) : "v"(base_ + offB[y]) : "memory");     \
+            /* 32-bit lane offset + wave-uniform 64-bit base in scalar registers: no per-lane address arithmetic */ \
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(FB[y]) : "v"(offB[y]), "s"(base_) : "memory");  \
         }                                                                                                         \
     }
         // Request order: A0 B0 A1 B1 B2 | tile 0: A2 .. B3 | tile 1: .. B4 | tile 2: A3 .. B5 | ... : the even tile t
@@ -1773,7 +1775,10 @@ __global__ __launch_bounds__(WM *WN * 64 * (PIPE == 8 ? 2 : 1), PIPE == 8 ? 1 : 
         return;  // its sums are in group 0's accumulators
     }
     if constexpr (GELU_DYN) {
-        epilogue_gelu_sync<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+        // the lane index formed afresh (from the execution mask) rather than kept in a register across the K loop: with the
+        // register-B loop this instantiation has none to spare, and the loops with hand-counted loads must not spill
+        const uint32_t lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        epilogue_gelu_sync<WM, WN, TM, TN>(a, acc, smem, lane_e, wave, m0, n0);
     } else {
         epilogue_panel<WM, WN, TM, TN, CONV>(a, acc, smem, lane, wave, m0, n0, T::kLdsBytes);
     }

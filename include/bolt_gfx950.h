@@ -472,7 +472,10 @@ EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *
  * it initialise the rest of the library). At most BOLT_GFX950_NOALLOC_MAX_ELEMENTS elements (NOT_SUPPORTED beyond,
  * with the reason in bolt_gfx950_last_error()). Enqueued on the library's stream (bolt_gfx950_set_stream; the
  * default stream if none was set). All calls on one GPU share that array: calls that overlap on one GPU (two
- * streams, two threads) race. */
+ * streams, two threads) race. The array's device address is looked up once per GPU -- by bolt_gfx950_init(), or else
+ * by the first call on that GPU, and that lookup (a module load and a symbol query) is neither capture-safe nor free of
+ * allocation inside the runtime: call bolt_gfx950_init() or make one warm-up call on the GPU before using this entry
+ * point under graph capture or inside a region that forbids allocation. */
 #define BOLT_GFX950_NOALLOC_MAX_ELEMENTS (1u << 30)
 EE bolt_gfx950_quantize_f32_noalloc(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode);
 EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,

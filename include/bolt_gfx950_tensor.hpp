@@ -47,7 +47,11 @@ inline Tensor device_tensor(TensorDesc desc)
     Tensor t(CPUMem);
     t.resize(desc);
     void *p = bolt_gfx950_malloc(tensorNumBytes(desc));
-    ((CpuMemory *)(t.get_memory()))->set_shared_ptr(std::shared_ptr<U8>((U8 *)p, [](U8 *q) { bolt_gfx950_free(q); }));
+    if (p) {
+        ((CpuMemory *)(t.get_memory()))->set_shared_ptr(std::shared_ptr<U8>((U8 *)p, [](U8 *q) { bolt_gfx950_free(q); }));
+    }
+    // allocation refused: the tensor keeps no buffer (ptr_of() == nullptr) and every call it is handed to returns
+    // NULL_POINTER; bolt_gfx950_last_error() has the reason
     return t;
 }
 
@@ -258,8 +262,9 @@ inline EE deconvolution_infer_forward_tmp_bytes(Tensor inputTensor, Tensor filte
         outputTensor.get_desc(), convParamSpec, algorithm, bytes, archInfo->arch);
 }
 
-// scale: host F32[3] = {input scale, filter scale, output scale}, read and rewritten as on x86 (DeconvolutionCPU::run,
-// deconvolution_cpu.hpp:65-84); the scale descriptor is the filter's, as deconvolution.cpp:255 passes it
+// scale: host F32[3]: scale[0] = input scale, scale[1] = output scale (in / out: below 0 = dynamic, rewritten with the
+// scale the call chose), scale[2] = filter scale -- the order DeconvolutionCPU::run fills them in
+// (deconvolution_cpu.hpp:65-84); the scale descriptor is the filter's, as deconvolution.cpp:255 passes it
 inline EE deconvolution(Tensor inputTensor, Tensor filterTensor, ConvolutionParamSpec convParamSpec,
     ConvolutionForwardAlgorithm algorithm, void *scale, Tensor biasTensor, Tensor tmpTensor, Tensor outputTensor,
     ActivationParamSpec activationDesc, ArchInfo_t archInfo)

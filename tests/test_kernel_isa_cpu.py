@@ -1,8 +1,10 @@
-"""Build-time guard for the GEMM loop whose B fragments are loaded by instructions issued as text
-(gemm_u8s8_dma_kernel, PIPE 4): the compiler does not know those loads, so if it ever spilled a register inside the
-loop it could store one whose data has not arrived yet -- silently wrong results on some shapes. The test compiles
-gemm.hip to gfx950 assembly (no GPU needed) and checks, for every instantiation of that loop, that nothing is stored
-to scratch between its first and its last matrix instruction, and that the text loads are there at all."""
+"""Build-time guards for the GEMM loops that count their own memory operations (gemm_u8s8_dma_kernel: explicit
+`s_waitcnt vmcnt(n)` around LDS-bound tile requests, and, with PIPE 4, B fragments loaded by instructions issued as
+text). The compiler does not know the text loads, so a register it spilled or re-used while such a load is in flight
+would be stored before its data arrived or overwritten when the load returns; and every scratch access is itself a
+vector memory operation that the hand-written counts do not include. The tests compile gemm.hip to gfx950 assembly
+(no GPU needed) and check that NO instantiation of that kernel uses scratch memory at all -- prologue, loop, tail and
+epilogue alike -- that the text loads are there, and that the pinned-order loops keep their order."""
 import os
 import re
 import shutil
@@ -44,6 +46,35 @@ def kernels(asm):
     return res
 
 
+def resources(asm):
+    """name -> {"ScratchSize": n, "NumVgprs": n, ...} from the compiler's per-kernel report"""
+    res, name = {}, None
+    for line in asm.splitlines():
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name = m.group(1)
+        m = re.match(r"^; (NumVgprs|NumAgprs|ScratchSize|Occupancy): (\d+)", line)
+        if m and name:
+            res.setdefault(name, {})[m.group(1)] = int(m.group(2))
+    return res
+
+
+def test_no_scratch_in_any_loop_with_hand_counted_memory_operations(gemm_asm):
+    """Whole-kernel check: the compiler's own resource report must say 0 bytes of scratch for every instantiation of
+    gemm_u8s8_dma_kernel, and no scratch instruction may appear anywhere in their bodies (the stretch from the first
+    tile request to the final drain included, and the epilogues behind it)."""
+    rs, ks = resources(gemm_asm), kernels(gemm_asm)
+    names = [n for n in rs if "gemm_u8s8_dma_kernel" in n]
+    assert len(names) >= 12, sorted(names)
+    pipes = set()
+    for n in names:
+        pipes.add(int(re.search(r"gemm_u8s8_dma_kernelILi\d+ELi\d+ELi\d+ELi\d+ELi\d+ELi(\d+)E", n).group(1)))
+        assert rs[n]["ScratchSize"] == 0, "%s: %d bytes of scratch per lane" % (n, rs[n]["ScratchSize"])
+        assert rs[n]["NumVgprs"] + rs[n]["NumAgprs"] <= 256, n    # two waves per SIMD
+        assert not [ins for ins in ks[n] if ins.startswith("scratch_")], n
+    assert {3, 4} <= pipes, "the whole-line loops (PIPE 3 and 4) are missing: %s" % sorted(pipes)
+
+
 def test_no_spill_stores_inside_the_register_b_loop(gemm_asm):
     ks = kernels(gemm_asm)
     # template arguments <WM, WN, TM, TN, STAGES, PIPE, ...>: PIPE == 4 is the sixth
@@ -53,7 +84,8 @@ def test_no_spill_stores_inside_the_register_b_loop(gemm_asm):
         mf = [i for i, ins in enumerate(body) if ins.startswith("v_mfma_i32_16x16x64_i8")]
         assert mf, name
         region = body[mf[0]:mf[-1] + 1]
-        text_loads = [ins for ins in region if ins.startswith("global_load_dwordx4") and ins.endswith("off")]
+        # (32-bit lane offset in a vector register + the wave's 64-bit base in a scalar pair)
+        text_loads = [ins for ins in region if re.match(r"global_load_dwordx4 v\[\d+:\d+\], v\d+, s\[\d+:\d+\]", ins)]
         assert len(text_loads) >= 12, "%s: the B loads issued as text are missing from the loop" % name
         stores = [ins for ins in region if ins.startswith("scratch_store")]
         assert not stores, "%s: the compiler spills inside the loop with hand-counted loads: %s" % (name, stores[:3])

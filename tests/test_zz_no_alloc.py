@@ -40,6 +40,30 @@ def test_no_alloc_matches_async_two_calls_in_a_row():
                 assert np.float32(got[1][1].item()) == np.float32(127.0) / np.float32(0.0425)
 
 
+def test_no_alloc_leaves_device_memory_alone():
+    """After the one-time set-up (bolt_gfx950_init or a first call), a run of calls changes neither the free device
+    memory the driver reports nor torch's own allocator's reservation."""
+    import torch
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_init(), "init")
+    x = torch.randn(1 << 20, device="cuda")
+    q = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    ds = torch.tensor([-1.0], device="cuda")
+    capi.check(L.bolt_gfx950_quantize_f32_noalloc(x.data_ptr(), x.numel(), DT_U8_Q, q.data_ptr(), ds.data_ptr(), 0), "warm-up")
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for n in (1 << 20, 1000, 1 << 18, 64):
+        for _ in range(8):
+            capi.check(L.bolt_gfx950_quantize_f32_noalloc(x.data_ptr(), n, DT_U8_Q, q.data_ptr(), ds.data_ptr(), 0), "quantize")
+    capi.check(L.bolt_gfx950_synchronize(), "sync")
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert torch.cuda.memory_reserved() == reserved0
+
+
 def test_no_alloc_rejects_and_edges():
     import torch
     L = capi.lib()
