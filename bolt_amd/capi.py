@@ -246,6 +246,13 @@ SIGNATURES = {
     "bolt_gfx950_quantize_f32_async": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_quantize_f32_noalloc": (C.c_int, [_vp, _u32, C.c_int, _vp, _vp, C.c_int]),
     "bolt_gfx950_mmm_int8_perchannel": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "bolt_gfx950_mmm_int8_perchannel_u8": (C.c_int, [_u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_float]),
+    "bolt_gfx950_convolution_int8_perchannel": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, _vp,
+                                                          TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, _f32p,
+                                                          ActivationParamSpec, C.c_int]),
+    "bolt_gfx950_convolution_async": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, TensorDesc, _vp,
+                                                _u32, _vp, TensorDesc, _vp, _vp, C.c_float, _vp, _vp, C.c_float,
+                                                ActivationParamSpec]),
     "bolt_gfx950_mvm_int8_perchannel": (C.c_int, [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bolt_gfx950_mvm_int8_strided_batch": (C.c_int, [_u32, _u32, _u32, _vp, C.c_size_t, _u32, _vp, _vp, _vp, _vp,
                                                      _vp]),

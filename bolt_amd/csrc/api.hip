@@ -142,13 +142,15 @@ EE ensure_init()
         return fail(NOT_SUPPORTED, "no HIP device available", e);
     }
     if (!c.ws) {
-        e = hipMalloc((void **)&c.ws, (kWsWords + 64 + 4 * kWsWords) * sizeof(uint32_t));
+        e = hipMalloc((void **)&c.ws, (kWsWords + 64 + 4 * kWsWords + 2 * kWsWords) * sizeof(uint32_t));
         if (e != hipSuccess) {
             c.ws = nullptr;
             return fail(ALLOC_FAILED, "hipMalloc(scratch words)", e);
         }
     }
     c.enc_ws = c.ws + kWsWords + 64;
+    c.conv_ws[0] = c.enc_ws + 4 * kWsWords;
+    c.conv_ws[1] = c.conv_ws[0] + kWsWords;
     if (!c.fsync.slots) {
         void *p = nullptr;
         e = hipMalloc(&p, kFusedSyncBytes);
@@ -3393,6 +3395,39 @@ EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const voi
     g.epi.scaleI = dscaleI;
     g.epi.scaleW = scaleW;
     g.epi.bias = bias;
+    HIP_TRY(launch_gemm_u8s8(g, ctx().stream));
+    return SUCCESS;
+}
+
+EE bolt_gfx950_mmm_int8_perchannel_u8(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
+    void *C, const float *dscaleI, const float *scaleW, const float *bias, F32 outputScale)
+{
+    if (!A || !packedB || !offsetC || !C || !dscaleI || !scaleW) {
+        return NULL_POINTER;
+    }
+    if (!(outputScale > 0)) {
+        return fail(NOT_MATCH, "the output scale must be positive (this epilogue is the static form)");
+    }
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = (const uint8_t *)A;
+    g.lda = K;
+    g.Bp = (const int8_t *)packedB;
+    g.M = M;
+    g.N = N;
+    g.K = K;
+    g.ob = offsetC;
+    g.comp = (const int32_t *)((const U8 *)packedB + packed_matrix_bytes(N, K));
+    g.C = C;
+    g.epi.mode = EPI_U8_CH;
+    g.epi.scaleI = dscaleI;
+    g.epi.scaleW = scaleW;
+    g.epi.bias = bias;
+    g.epi.factor = outputScale;
     HIP_TRY(launch_gemm_u8s8(g, ctx().stream));
     return SUCCESS;
 }

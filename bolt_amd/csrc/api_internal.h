@@ -29,6 +29,11 @@ struct Ctx {
     bg::FusedSync fsync;  // sync area of the one-launch dynamic quantiser
     uint32_t *enc_ws = nullptr;  // the encoder layer's four arrays of max slots (behind ws), kept clear between calls
     bool enc_ws_dirty = true;
+    // two arrays of max slots (behind enc_ws) that the two-pass u8 convolutions of api_conv_ext.hip alternate between:
+    // the second pass of a call clears the array the NEXT call folds into, so no call spends a launch on clearing
+    uint32_t *conv_ws[2] = {nullptr, nullptr};
+    int conv_ws_next = 0;
+    bool conv_ws_dirty = true;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     bool reused = false;  // taken over from a thread that has ended: its last work may still be running

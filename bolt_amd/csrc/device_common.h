@@ -44,16 +44,29 @@ enum EpiMode : int {
     EPI_U8_TRUNC = 4,  // (int)(cvt(acc) * factor + 128.0f), > 255 -> 255, else low byte
     // y = gelu_tanh(cvt(acc) * (1.0f / (sI * sW[n])) + bias[n]); u8 = quantise(y) with the tensor-wide dynamic scale
     // max(0, 127 / max|y|), the maximum agreed on by all workgroups of the launch while y is still in registers
-    EPI_U8_GELU_DYN = 5
+    EPI_U8_GELU_DYN = 5,
+    // per-output-channel extension with a u8 result: q_u8(cvt(acc) * (1.0f / (sI * sW[n])) + bias[n], factor) -- the
+    // fp32 value of EPI_F32_CH put through the fp32 -> u8 quantiser with the given (static) output scale
+    EPI_U8_CH = 6,
+    // int8 convolution with per-output-channel filter scales (GemmArgs::conv.ch_out says what is done with the value):
+    // f = cvt(acc) * (1.0f / (sI * sW[oc])) + bias[oc] (+ eltwise), ReLU
+    EPI_CONV_CH = 7
+};
+
+// what EPI_CONV_CH does with its fp32 values
+enum ConvChOut : int {
+    CONV_CH_F32 = 0,   // stored as they are
+    CONV_CH_U8 = 1,    // q_u8(f, s): s = epi.factor when > 0 (static), else 127 / max|f| from the scratch slots (1 for 0)
+    CONV_CH_MAX = 2    // nothing stored: max|f| (its bits, an order-preserving int) folded into the scratch slots
 };
 
 struct Epilogue {
     int mode = 0;
     float factor = 0;            // EPI_F32 / EPI_U8 when dfactor == nullptr
     const float *dfactor = nullptr;    // optional device scalar: EPI_F32 uses 1.0f / *dfactor, EPI_U8 uses *dfactor
-    const float *scaleI = nullptr;     // EPI_F32_CH: device scalar input scale
-    const float *scaleW = nullptr;     // EPI_F32_CH: device per-channel weight scales [N]
-    const float *bias = nullptr;       // EPI_F32_CH: optional device fp32 bias [N]
+    const float *scaleI = nullptr;     // EPI_F32_CH / EPI_U8_CH: device scalar input scale
+    const float *scaleW = nullptr;     // EPI_F32_CH / EPI_U8_CH / EPI_CONV_CH: device per-channel weight scales [N]
+    const float *bias = nullptr;       // EPI_F32_CH / EPI_U8_CH / EPI_CONV_CH: optional device fp32 bias [N]
 };
 
 __device__ __forceinline__ float epi_factor(const Epilogue &e)

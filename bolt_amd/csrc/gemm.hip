@@ -31,9 +31,10 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v4i &acc, ui
     float factor = 0.0f, sI = 0.0f, sW = 0.0f;
     if (a.epi.mode == EPI_F32 || a.epi.mode == EPI_U8) {
         factor = epi_factor(a.epi);
-    } else if (a.epi.mode == EPI_F32_CH) {
+    } else if (a.epi.mode == EPI_F32_CH || a.epi.mode == EPI_U8_CH) {
         sI = *a.epi.scaleI;
         sW = a.epi.scaleW[n];
+        factor = a.epi.factor;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -43,7 +44,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v4i &acc, ui
         }
         const size_t idx = (size_t)m * a.N + n;
         uint32_t v = (uint32_t)acc[r] + base;
-        if (a.add_cin && a.epi.mode != EPI_U8) {
+        if (a.add_cin && a.epi.mode != EPI_U8 && a.epi.mode != EPI_U8_CH) {
             v += (uint32_t)((const int32_t *)a.C)[idx];
         }
         const int vi = (int)v;
@@ -59,6 +60,9 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v4i &acc, ui
                 break;
             case EPI_F32_CH:
                 ((float *)a.C)[idx] = epi_f32_ch(vi, sI, sW, a.epi.bias, n);
+                break;
+            case EPI_U8_CH:
+                ((uint8_t *)a.C)[idx] = (uint8_t)q_u8(epi_f32_ch(vi, sI, sW, a.epi.bias, n), factor);
                 break;
             default:
                 break;
@@ -182,7 +186,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
-    const bool use_cin = (CIN == 2) ? (!CONV && a.add_cin && MODE != EPI_U8) : (CIN == 1);
+    const bool use_cin = (CIN == 2) ? (!CONV && a.add_cin && MODE != EPI_U8 && MODE != EPI_U8_CH) : (CIN == 1);
     const bool n_vec = FULL || CONV || ((a.N & 3) == 0);
     int lane_max = 0;
 
@@ -195,13 +199,15 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         }
         factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
         if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out && !a.sync.slots) {
-            *a.conv.dscale_out = a.conv.scaleO * factor;
+            *a.conv.dscale_out = conv_acc_scale(a.conv) * factor;
         }
     } else if (MODE == EPI_F32 || MODE == EPI_U8) {
-        factor = epi_factor(a.epi);
-    } else if (MODE == EPI_F32_CH) {
+        factor = (CONV && a.conv.dscaleI) ? 1.0f / conv_acc_scale(a.conv) : epi_factor(a.epi);
+    } else if (MODE == EPI_F32_CH || MODE == EPI_U8_CH) {
         sI = CONV ? 1.0f : *a.epi.scaleI;
+        factor = a.epi.factor;  // EPI_U8_CH: the output scale
     }
+    const float fold_scale = (CONV && a.conv.dscaleI) ? conv_acc_scale(a.conv) : a.fold_scale;
 
     uint32_t base[TN][4];
     float qs[TN][4], bs[TN][4];
@@ -212,8 +218,9 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         // offsets ahead of its K loop, while it was waiting for memory anyway.
         uint32_t nn[TN * 4], flat[TN * 4];
         float sw[TN * 4], bi[TN * 4];
-        const float *swp = (MODE == EPI_F32_CH) ? a.epi.scaleW : (const float *)a.comp;
-        const float *bip = (MODE == EPI_F32_CH && a.epi.bias) ? a.epi.bias : (const float *)a.comp;
+        constexpr bool kCh = (MODE == EPI_F32_CH || MODE == EPI_U8_CH);
+        const float *swp = kCh ? a.epi.scaleW : (const float *)a.comp;
+        const float *bip = (kCh && a.epi.bias) ? a.epi.bias : (const float *)a.comp;
 #pragma unroll
         for (int y = 0; y < TN; ++y) {
 #pragma unroll
@@ -225,7 +232,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             }
         }
         if (!pre_base) {
-            column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, a.fold_scale, nn, flat);
+            column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, fold_scale, nn, flat);
         }
 #pragma unroll
         for (int y = 0; y < TN; ++y) {
@@ -236,7 +243,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 base[y][c] = pre_base ? pre_base[y][c] : (ok ? flat[y * 4 + c] : 0u);
                 qs[y][c] = 1.0f;
                 bs[y][c] = 0.0f;
-                if (MODE == EPI_F32_CH && ok) {
+                if ((MODE == EPI_F32_CH || MODE == EPI_U8_CH) && ok) {
                     if (CONV) {
                         // 1-bit convolution on the matrix cores: fma(S, scale[oc], bias[oc]), scale used as it is
                         qs[y][c] = sw[y * 4 + c];
@@ -288,7 +295,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         }
         factor = ((int)outcome == 0) ? 1.0f : 127.0f / (float)(int)outcome;
         if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
-            *a.conv.dscale_out = a.conv.scaleO * factor;
+            *a.conv.dscale_out = conv_acc_scale(a.conv) * factor;
         }
     }
 
@@ -370,12 +377,20 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                         ((int32_t *)a.C)[idx + c] = t[c];
                     }
                 }
-            } else if (MODE == EPI_U8) {
+            } else if (MODE == EPI_U8 || MODE == EPI_U8_CH) {
                 unsigned b[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    // stand-alone requantisation adds 128.0f before rounding, the GEMM's own u8 mode after
-                    b[c] = CONV ? usat8_u(rne_i32((float)t[c] * factor + 128.0f)) : epi_u8(t[c], factor);
+                    if (MODE == EPI_U8_CH) {
+                        float f = (float)t[c] * qs[y][c];
+                        if (a.epi.bias) {
+                            f = f + bs[y][c];
+                        }
+                        b[c] = q_u8(f, factor);
+                    } else {
+                        // stand-alone requantisation adds 128.0f before rounding, the GEMM's own u8 mode after
+                        b[c] = CONV ? usat8_u(rne_i32((float)t[c] * factor + 128.0f)) : epi_u8(t[c], factor);
+                    }
                 }
                 if (vec) {
                     *(uint32_t *)((uint8_t *)a.C + idx) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
@@ -539,25 +554,38 @@ __device__ __forceinline__ void epilogue_rows_lds(const GemmArgs &a, v4i (&acc)[
 // (pitch 80: the 4-byte writes of the fragment layout and the 16-byte reads of the row layout are both free of bank
 // conflicts). Straight from the accumulators a store instruction puts 4 bytes of a different row into every lane,
 // 64 pieces for the address unit; from the panel lane 4 r + c stores 16 bytes of row r, a quad = one 64-byte piece.
-template <int WM, int WN, int TM, int TN>
+// CH: the per-output-channel form (EPI_U8_CH), the fp32 value of EPI_F32_CH quantised with the static scale epi.factor.
+template <int WM, int WN, int TM, int TN, bool CH = false>
 __device__ __forceinline__ void epilogue_rows_lds_u8(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
     static_assert(TN == 4, "a wave's tile row must be 64 columns");
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
-    const float factor = epi_factor(a.epi);
+    const float factor = CH ? a.epi.factor : epi_factor(a.epi);
     uint32_t base[TN * 4];
+    float qs[TN * 4], bs[TN * 4];
     {
         uint32_t nn[TN * 4];
+        float sw[TN * 4], bi[TN * 4];
+        const float *swp = CH ? a.epi.scaleW : (const float *)a.comp;
+        const float *bip = (CH && a.epi.bias) ? a.epi.bias : (const float *)a.comp;
 #pragma unroll
         for (int y = 0; y < TN; ++y) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 nn[y * 4 + c] = n0 + (wn * TN + y) * 16 + 4 * g + c;
+                sw[y * 4 + c] = swp[nn[y * 4 + c]];
+                bi[y * 4 + c] = bip[nn[y * 4 + c]];
             }
         }
         column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, a.fold_scale, nn, base);
+        const float sI = CH ? *a.epi.scaleI : 1.0f;
+#pragma unroll
+        for (int k = 0; k < TN * 4; ++k) {
+            qs[k] = CH ? 1.0f / (sI * sw[k]) : 1.0f;
+            bs[k] = (CH && a.epi.bias) ? bi[k] : 0.0f;
+        }
     }
     constexpr uint32_t kPitch = 80;
     uint8_t *pan = smem + wave * (16 * kPitch);
@@ -571,7 +599,16 @@ __device__ __forceinline__ void epilogue_rows_lds_u8(const GemmArgs &a, v4i (&ac
             unsigned b[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                b[c] = epi_u8((int)((uint32_t)acc[x][y][c] + base[y * 4 + c]), factor);  // int32 wrap
+                const int t_ = (int)((uint32_t)acc[x][y][c] + base[y * 4 + c]);  // int32 wrap
+                if (CH) {
+                    float f = (float)t_ * qs[y * 4 + c];
+                    if (a.epi.bias) {
+                        f = f + bs[y * 4 + c];
+                    }
+                    b[c] = q_u8(f, factor);
+                } else {
+                    b[c] = epi_u8(t_, factor);
+                }
             }
             *(uint32_t *)(wr + 16 * y) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
         }
@@ -694,13 +731,129 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
     }
 }
 
+// EPI_CONV_CH: the int8 convolution with one filter scale per OUTPUT CHANNEL. Not in the reference, whose kernels
+// carry one scale for the whole filter (convolution_direct.cpp:2406-2422, 2687-2692); the arithmetic is the per-channel
+// matrix epilogue's (EPI_F32_CH) with the convolution's own tail:
+//   f = cvt(acc + ob[oc] - comp[oc]) * (1.0f / (sI * sW[oc]))   single fp32 operations, reciprocal first
+//   f = f + bias[oc]                                             when a bias is given
+//   f = f + eltwise[...]                                         fp32 result only, as :2410-2422 place it
+//   f = max(f, 0)                                                with ReLU
+// and then, by conv.ch_out: stored as fp32; or quantised like a fp32 tensor (q_u8, avx512/quantize.cpp:150-155) with
+// the static scale epi.factor or the dynamic one 127 / max|f| from the scratch slots; or only max|f| folded into those
+// slots. With every sW[oc] equal, no bias and an fp32 result this is the reference's epilogue bit for bit.
+template <int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[TM][TN], uint32_t lane, uint32_t wave,
+    uint32_t m0, uint32_t n0)
+{
+    const uint32_t i = lane & 15, g = lane >> 4;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const float sI = a.conv.dscaleI ? *a.conv.dscaleI : a.conv.scaleI;
+    const int out = a.conv.ch_out;
+    uint32_t base[TN][4], cblk_off[TN], cblk_w[TN];
+    float qs[TN][4], bs[TN][4];
+    {
+        // every per-column term in one batch of loads, none behind a branch; columns past N read column N - 1
+        uint32_t nn[TN * 4], flat[TN * 4];
+        float sw[TN * 4], bi[TN * 4];
+        const float *bip = a.epi.bias ? a.epi.bias : a.epi.scaleW;
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g + c;
+                nn[y * 4 + c] = n < a.N ? n : a.N - 1;
+                sw[y * 4 + c] = a.epi.scaleW[nn[y * 4 + c]];
+                bi[y * 4 + c] = bip[nn[y * 4 + c]];
+            }
+        }
+        column_bases<TN * 4>(a.ob, a.comp, nullptr, 0.0f, nn, flat);
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                base[y][c] = flat[y * 4 + c];
+                qs[y][c] = 1.0f / (sI * sw[y * 4 + c]);
+                bs[y][c] = a.epi.bias ? bi[y * 4 + c] : 0.0f;
+            }
+            const uint32_t xc = a.conv.out_c, blk = n / xc;
+            cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
+            cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+        }
+    }
+    float s = 0.0f;
+    if (out == CONV_CH_U8) {
+        if (a.epi.factor > 0.0f) {
+            s = a.epi.factor;
+        } else {
+            const float mx = __uint_as_float((uint32_t)ws_read_max(a.conv.absmax));
+            s = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+        }
+        if (blockIdx.x == 0 && wave == 0 && lane == 0 && a.conv.dscale_out) {
+            *a.conv.dscale_out = s;
+        }
+    }
+    int lane_max = 0;
+#pragma unroll
+    for (int x = 0; x < TM; ++x) {
+        const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+        if (m >= a.M) {
+            continue;
+        }
+        const uint32_t img = m / a.conv.OHW, pix = m - img * a.conv.OHW;
+        const size_t rowbase = (size_t)img * a.N * a.conv.OHW;
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+            if (n >= a.N) {
+                continue;
+            }
+            const size_t idx = rowbase + cblk_off[y] + (size_t)pix * cblk_w[y];
+            float f[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                f[c] = (float)(int)((uint32_t)acc[x][y][c] + base[y][c]) * qs[y][c];
+                if (a.epi.bias) {
+                    f[c] = f[c] + bs[y][c];
+                }
+                if (out == CONV_CH_F32 && a.conv.eltwise && n + c < a.N) {
+                    f[c] = f[c] + a.conv.eltwise[idx + c];
+                }
+                if (a.conv.relu && !(f[c] > 0.0f)) {
+                    f[c] = 0.0f;
+                }
+            }
+            if (out == CONV_CH_MAX) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (n + c < a.N) {
+                        const int av = (int)__float_as_uint(fabsf(f[c]));  // a NaN's bits never win against a number's:
+                        lane_max = (f[c] == f[c] && av > lane_max) ? av : lane_max;  // the quantiser's maximum skips NaNs too
+                    }
+                }
+            } else if (out == CONV_CH_U8) {
+                const unsigned b0 = q_u8(f[0], s), b1 = q_u8(f[1], s), b2 = q_u8(f[2], s), b3 = q_u8(f[3], s);
+                *(uint32_t *)((uint8_t *)a.C + idx) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            } else {
+                store_c16<false>((v4f *)((float *)a.C + idx), (v4f){f[0], f[1], f[2], f[3]});
+            }
+        }
+    }
+    if (out == CONV_CH_MAX) {
+        lane_max = wave_reduce_max_i(lane_max);
+        if (lane == 0) {
+            ws_fold_max(a.conv.absmax, blockIdx.x * 8 + wave, lane_max);
+        }
+    }
+}
+
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0, const uint32_t (*pre_base)[4] = nullptr)
 {
     const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
-    const bool cin = !CONV && a.add_cin && MODE != EPI_U8;
-    if constexpr (!CONV && MODE != EPI_U8 && TN == 4) {
+    const bool cin = !CONV && a.add_cin && MODE != EPI_U8 && MODE != EPI_U8_CH;
+    if constexpr (!CONV && MODE != EPI_U8 && MODE != EPI_U8_CH && TN == 4) {
         // smem: the kernel's LDS, free by now and at least 8 waves x 4352 bytes (the DMA kernels); null otherwise
         if (full && smem) {
             if (a.stream_c) {
@@ -717,15 +870,15 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
             return;
         }
     }
-    if constexpr (!CONV && MODE == EPI_U8 && TN == 4) {
+    if constexpr (!CONV && (MODE == EPI_U8 || MODE == EPI_U8_CH) && TN == 4) {
         if (full && smem && (a.N & 15) == 0 && ((uintptr_t)a.C & 15) == 0) {
-            epilogue_rows_lds_u8<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_rows_lds_u8<WM, WN, TM, TN, MODE == EPI_U8_CH>(a, acc, smem, lane, wave, m0, n0);
             return;
         }
     }
     if (full && !cin) {
         epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0, pre_base);
-    } else if (full && MODE != EPI_U8 && !CONV) {
+    } else if (full && MODE != EPI_U8 && MODE != EPI_U8_CH && !CONV) {
         epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1>(a, acc, smem, lane, wave, m0, n0, pre_base);
     } else {
         epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2>(a, acc, smem, lane, wave, m0, n0, pre_base);
@@ -744,6 +897,8 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
             epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_F32_CH) {
             epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
+        } else if (a.epi.mode == EPI_CONV_CH) {
+            epilogue_conv_ch<WM, WN, TM, TN>(a, acc, lane, wave, m0, n0);
         } else {
             epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         }
@@ -758,6 +913,9 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
             break;
         case EPI_U8:
             epilogue_mode<EPI_U8, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            break;
+        case EPI_U8_CH:
+            epilogue_mode<EPI_U8_CH, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
             break;
         default:
             epilogue_mode<EPI_F32_CH, false, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
@@ -901,12 +1059,39 @@ __global__ __launch_bounds__(WM *WN * 64, 2) void gemm_u8s8_tiled_kernel(GemmArg
 // the same factor for its own arithmetic) does not store it a second time.
 __device__ __forceinline__ void conv_publish_scale(GemmArgs &a, uint32_t wave)
 {
+    if (a.clear_ws && blockIdx.x == 0) {
+        // an array of max slots that no kernel still in flight reads (the caller alternates between two): cleared
+        // here for the call that will fold into it next
+        for (uint32_t k = threadIdx.x; k < kWsWords; k += blockDim.x) {
+            a.clear_ws[k] = 0;
+        }
+    }
+    if (a.conv.dscale_out && a.conv.dscaleI && (a.epi.mode == EPI_F32 || (a.epi.mode == EPI_I32 && a.C))) {
+        // asynchronous form, fp32 / int32 result: the scale of the accumulators is what the synchronous call reports
+        if (blockIdx.x == 0 && wave == 0 && (threadIdx.x & 63) == 0) {
+            *a.conv.dscale_out = conv_acc_scale(a.conv);
+        }
+        a.conv.dscale_out = nullptr;
+    }
     if (a.epi.mode == EPI_U8 && a.conv.dscale_out && !a.sync.slots) {
         if (blockIdx.x == 0 && wave == 0) {
             const int mx = ws_read_max(a.conv.absmax);
             const float factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
             if ((threadIdx.x & 63) == 0) {
-                *a.conv.dscale_out = a.conv.scaleO * factor;
+                *a.conv.dscale_out = conv_acc_scale(a.conv) * factor;
+            }
+        }
+        a.conv.dscale_out = nullptr;
+    } else if (a.epi.mode == EPI_CONV_CH && a.conv.ch_out == CONV_CH_U8 && a.conv.dscale_out) {
+        // the per-channel form: the scale the u8 result is quantised with (given, or from the first pass's max|f|)
+        if (blockIdx.x == 0 && wave == 0) {
+            float s = a.epi.factor;
+            if (!(s > 0.0f)) {
+                const float mx = __uint_as_float((uint32_t)ws_read_max(a.conv.absmax));
+                s = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+            }
+            if ((threadIdx.x & 63) == 0) {
+                *a.conv.dscale_out = s;
             }
         }
         a.conv.dscale_out = nullptr;
@@ -1877,12 +2062,13 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
         }
     };
     auto pre_base_form = [&]() {
+        const float fold_scale_ = a.conv.dscaleI ? conv_acc_scale(a.conv) : a.fold_scale;
 #pragma unroll
         for (int y = 0; y < 4; ++y) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t n = y * 16 + 4 * g + c;
-                const float p_ = pb_f[y][c] * a.fold_scale;  // as column_base() forms it
+                const float p_ = pb_f[y][c] * fold_scale_;  // as column_base() forms it
                 const int32_t o_ = fold ? (int32_t)(round((double)p_) + (double)pb_c[y][c]) : pb_o[y][c];
                 pre_base[y][c] = (n < a.N) ? (uint32_t)o_ - (uint32_t)pb_c[y][c] : 0u;
             }

@@ -62,7 +62,22 @@ struct ConvGeom {
                                // nothing is stored); u8 mode reads them for the tensor-wide dynamic scale
     float scaleO = 0;              // u8 mode: scale of the accumulators (input scale * filter scale)
     float *dscale_out = nullptr;         // u8 mode: device word that receives the resulting output scale
+    // The input scale may live in device memory (a chain of quantised operators that never waits for the host): then
+    // the accumulators' scale is *dscaleI * filter_scale, formed by every consumer inside the kernel with the same
+    // single fp32 multiplication the host would do, and scaleO / GemmArgs::fold_scale / the fp32 factor are not used.
+    const float *dscaleI = nullptr;
+    float filter_scale = 0;
+    // EPI_CONV_CH (per-output-channel filter scales in epi.scaleW, fp32 bias in epi.bias): the input scale is *dscaleI
+    // when that is set, else scaleI; ch_out is a ConvChOut
+    float scaleI = 0;
+    int ch_out = 0;
 };
+
+// scale of a convolution's accumulators: input scale * filter scale (convolution_direct.cpp:2687)
+__device__ __forceinline__ float conv_acc_scale(const ConvGeom &c)
+{
+    return c.dscaleI ? (*c.dscaleI * c.filter_scale) : c.scaleO;
+}
 
 struct GemmArgs {
     const uint8_t *A = nullptr;    // u8 activations

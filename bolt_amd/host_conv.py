@@ -69,6 +69,65 @@ def convolution(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias,
     return out
 
 
+def _conv_call_setup(x, idf, n, ic, ih, iw, ftm, oc, fh, fw, stride, pad, odt, odf, dilation, tmp, out):
+    arch = arch_of(x)
+    p = conv_param_spec(oc, fh, fw, stride, pad, dilation)
+    oh, ow = conv_out_hw(ih, iw, fh, fw, stride, pad, dilation)
+    idesc = tensor4df(DT_U8_Q, idf, n, ic, ih, iw)
+    odesc = tensor4df(odt, odf, n, oc, oh, ow)
+    b = C.c_uint32(0)
+    check(lib().convolution_infer_forward_tmp_bytes_gfx950(idesc, ftm, odesc, p, CONVOLUTION_ALGORITHM_DIRECT, C.byref(b),
+                                                           arch), "conv_tmp_bytes")
+    if tmp is None:
+        tmp = _empty_like_mode(x, b.value)
+    elif (tmp.numel() if _is_torch(tmp) else tmp.nbytes) < b.value:
+        raise ValueError("tmp holds %d bytes, the convolution needs %d" % (tmp.numel() if _is_torch(tmp) else tmp.nbytes, b.value))
+    count = n * oc * oh * ow
+    if out is not None:
+        pass
+    elif _is_torch(x):
+        import torch
+        tdt = {DT_F32: torch.float32, DT_I32: torch.int32, DT_U8_Q: torch.uint8}[odt]
+        out = torch.zeros(count, dtype=tdt, device=x.device)
+    else:
+        out = np.zeros(count, NP_OF[odt])
+    return arch, p, idesc, odesc, b.value, tmp, out
+
+
+def convolution_perchannel(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, scale_w, bias, scale, relu, odt,
+                           odf=DF_NCHWC16, eltwise=None, dilation=1, tmp=None, out=None):
+    """The int8 convolution with one filter scale per output channel (bolt_gfx950_convolution_int8_perchannel; not in
+    the reference). scale_w: fp32 [oc]; bias: fp32 [oc] or None; scale = [sI, sO] (list): sO > 0 on entry = static u8
+    output scale, else dynamic and updated. odt: DT_F32 or DT_U8_Q."""
+    arch, p, idesc, odesc, nbytes, tmp, out = _conv_call_setup(x, idf, n, ic, ih, iw, ftm, oc, fh, fw, stride, pad, odt, odf,
+                                                               dilation, tmp, out)
+    sarr = (C.c_float * 2)(*[float(np.float32(v)) for v in scale])
+    act = ActivationParamSpec()
+    act.mode = ACTIVATION_RELU if relu else ACTIVATION_NULL
+    e = lib().bolt_gfx950_convolution_int8_perchannel(idesc, ptr(x), ptr(eltwise), ftm, ptr(blob), p, ptr(scale_w),
+                                                      tensor1d(DT_F32, oc), ptr(bias), nbytes, ptr(tmp), odesc, ptr(out),
+                                                      sarr, act, arch)
+    check(e, "convolution_perchannel")
+    for i in range(2):
+        scale[i] = np.float32(sarr[i])
+    return out
+
+
+def convolution_async(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias, dscale_in, filter_scale, scale_w,
+                      dscale_out, relu, odt, odf=DF_NCHWC16, static_out=0.0, eltwise=None, dilation=1, tmp=None, out=None):
+    """bolt_gfx950_convolution_async: device tensors only; dscale_in / dscale_out are one-element fp32 device tensors
+    (input scale read, output scale left there); scale_w None = one filter scale `filter_scale`, else fp32 [oc] device."""
+    arch, p, idesc, odesc, nbytes, tmp, out = _conv_call_setup(x, idf, n, ic, ih, iw, ftm, oc, fh, fw, stride, pad, odt, odf,
+                                                               dilation, tmp, out)
+    act = ActivationParamSpec()
+    act.mode = ACTIVATION_RELU if relu else ACTIVATION_NULL
+    e = lib().bolt_gfx950_convolution_async(idesc, ptr(x), ptr(eltwise), ftm, ptr(blob), p, tensor1d(DT_F32, oc), ptr(bias),
+                                            nbytes, ptr(tmp), odesc, ptr(out), ptr(dscale_in), float(filter_scale),
+                                            ptr(scale_w), ptr(dscale_out), float(static_out), act)
+    check(e, "convolution_async")
+    return out
+
+
 def bnn_transform_filter(filt_bits, fdt, fdf, oc, ic, fh, fw):
     """1-bit filter (DF_NCHW bit string or DF_NCHWN16C8 bytes) -> this library's blob
     (compute/tensor/src/cpu/arm/bnn/convolution_transform_bnn.h:32-86)."""

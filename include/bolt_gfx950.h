@@ -207,6 +207,38 @@ EE convolution_gfx950(TensorDesc inputDesc, const void *input, const void *eltwi
     const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, F32 *scale,
     ActivationParamSpec activationDesc, Arch arch);
 
+/* Int8 convolution with one filter scale per OUTPUT CHANNEL. No counterpart in the reference, whose int8 kernels
+ * carry one scale for the whole filter (compute/tensor/src/cpu/x86/int8/avx512/convolution_direct.cpp:2406-2422,
+ * 2687-2692); this is the convolution a channel-wise quantised filter needs. Same descs, filter blob, tmp size and
+ * layouts as convolution_gfx950; scaleW = oc fp32 scales (device memory with AMD_GFX950_DEVICE, host memory with
+ * AMD_GFX950), bias = oc fp32 values or NULL.
+ *   f = cvt(acc) * (1.0f / (scale[0] * scaleW[oc]))      single fp32 operations, the reciprocal first
+ *   f = f + bias[oc]; f = f + eltwise (DT_F32 result only); f = max(f, 0) with ACTIVATION_RELU
+ *   DT_F32  : f is the result; scale[1] is left alone.
+ *   DT_U8_Q : one output scale for the tensor. scale[1] > 0 on entry: static, q = quantise(f, scale[1]); otherwise
+ *             dynamic, s = 127 / max|f| over the tensor (1 when that is 0), q = quantise(f, s), scale[1] = s on return
+ *             (quantise = the fp32 -> u8 arithmetic of quantize_gfx950: rne(f * s + 128.0f) clamped to [1, 255]).
+ * With every scaleW[oc] equal, bias NULL or all zero and a DT_F32 result this is convolution_gfx950 (the reference) bit
+ * for bit; the u8 result equals quantize_gfx950 applied to the DT_F32 result. scale = host {input, output}. */
+EE bolt_gfx950_convolution_int8_perchannel(TensorDesc inputDesc, const void *input, const void *eltwiseInput,
+    TensorDesc filterDesc, const void *filter, ConvolutionParamSpec convParamSpec, const F32 *scaleW, TensorDesc biasDesc,
+    const void *bias, U32 tmpBytes, void *tmp, TensorDesc outputDesc, void *output, F32 *scale,
+    ActivationParamSpec activationDesc, Arch arch);
+/* convolution_gfx950 / bolt_gfx950_convolution_int8_perchannel for chains of quantised operators that must not wait
+ * for the host (no counterpart in the reference, which returns the new output scale through the host pointer
+ * scale[1]): device pointers only, the input scale is READ from device memory (*dscaleI, e.g. what the producing
+ * call left there) and the output scale is LEFT in device memory (*dscaleO); the call only enqueues.
+ *   scaleW == NULL: one filter scale filterScale; DT_F32 / DT_I32 / DT_U8_Q results and every byte as convolution_gfx950
+ *                   gives them for scale = {*dscaleI, -, filterScale}; *dscaleO = what that call leaves in scale[1]
+ *                   (dscaleO may be NULL for DT_F32 / DT_I32). bias is required, as there.
+ *   scaleW != NULL: the per-channel form above; DT_U8_Q with staticOutputScale > 0 quantises with that scale, otherwise
+ *                   dynamically; *dscaleO = the scale used (untouched for DT_F32).
+ * A dynamic u8 result runs the convolution twice (maximum, then store); no launch needs all its workgroups resident. */
+EE bolt_gfx950_convolution_async(TensorDesc inputDesc, const void *input, const void *eltwiseInput, TensorDesc filterDesc,
+    const void *filter, ConvolutionParamSpec convParamSpec, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
+    TensorDesc outputDesc, void *output, const float *dscaleI, F32 filterScale, const F32 *scaleW, float *dscaleO,
+    F32 staticOutputScale, ActivationParamSpec activationDesc);
+
 /* ---- tensor_computing: int8 deconvolution (transposed convolution) ------------------------ */
 /* The (TensorDesc + pointer) forms behind the reference's deconvolution*() on x86:
  *   deconvolution_infer_output_size_cpu        compute/tensor/src/deconvolution.cpp:23-65
@@ -480,6 +512,12 @@ EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *
 EE bolt_gfx950_quantize_f32_noalloc(const float *data, U32 n, DataType qdt, void *q, float *dscale, int mode);
 EE bolt_gfx950_mmm_int8_perchannel(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
     float *C, const float *dscaleI, const float *scaleW, const float *bias);
+/* The same product with a u8 result for the next quantised operator: the fp32 value above put through the fp32 -> u8
+ * quantiser (quantize_gfx950's arithmetic, avx512/quantize.cpp:150-155: rne(f * s + 128.0f) clamped to [1, 255]) with
+ * the static output scale outputScale > 0. No counterpart in the reference, whose u8 epilogue has one scale for all
+ * columns (blas_common_int8.h:565-590). C: [M][N] u8, device. */
+EE bolt_gfx950_mmm_int8_perchannel_u8(U32 M, U32 N, U32 K, const void *A, const void *packedB, const I32 *offsetC,
+    void *C, const float *dscaleI, const float *scaleW, const float *bias, F32 outputScale);
 EE bolt_gfx950_mvm_int8_perchannel(U32 N, U32 K, const void *packedW, const void *x, const I32 *offsetC, float *y,
     const float *dscaleI, const float *scaleW, const float *bias);
 /* `batch` independent matrix_vector_multiply products in ONE launch (decode serving: many

@@ -44,6 +44,16 @@ def from_conv_layout(buf, n, oc, oh, ow, out_c):
     return out
 
 
+def to_conv_layout(x_nchw, out_c):
+    """plain [n][oc][oh][ow] -> the x86 path's output order (inverse of from_conv_layout), flattened"""
+    n, oc, oh, ow = x_nchw.shape
+    parts = []
+    for b0 in range(0, oc, out_c):
+        bw = min(out_c, oc - b0)
+        parts.append(x_nchw[:, b0:b0 + bw].transpose(0, 2, 3, 1).reshape(n, oh * ow * bw))
+    return np.ascontiguousarray(np.concatenate(parts, axis=1)).reshape(-1)
+
+
 class ConvOracle:
     def __init__(self, oracle=None):
         self.lib = (oracle or Oracle()).lib
@@ -66,6 +76,36 @@ class ConvOracle:
         out = np.zeros(d.n * d.oc * d.oh * d.ow, NP_OF[d.odt])
         self.lib.orc_conv_int8(C.byref(d), _p(x), _p(f), _p(b), _p(e), _p(s), _p(out))
         return out, s
+
+    def conv_perchannel(self, oracle, d, in_nchwc8, filt_nchw, scale_w, bias, scale_in, out_scale=-1.0, eltwise=None):
+        """The int8 convolution with one filter scale per output channel, which the reference does not have: a
+        composition of two pinned pieces with three fp32 numpy operations between them,
+          acc  = the reference-pinned int32 convolution (orc_conv_int8_acc through conv(), no bias, no ReLU)
+          f    = cvt(acc) * (1.0f / (sI * sW[oc]))  [+ bias[oc]]  [+ eltwise]  [ReLU]
+          u8   = the reference-pinned fp32 -> u8 quantiser (orc_quantize_f32_u8): static with out_scale > 0, else dynamic
+        d.odt selects DT_F32 or DT_U8_Q. Returns (output in the x86 layout of d.out_c, output scale or None).
+        tests/test_oracle_conv.py holds it against the reference's own epilogue (equal scales) and against closed forms."""
+        di = ConvDesc.from_buffer_copy(d)
+        di.relu, di.odt = 0, DT_I32
+        acc, _ = self.conv(di, in_nchwc8, filt_nchw, None, [scale_in, -1.0, 1.0])
+        acc = from_conv_layout(acc, d.n, d.oc, d.oh, d.ow, d.out_c)                      # [n][oc][oh][ow]
+        sw = np.ascontiguousarray(scale_w, dtype=np.float32)
+        r = np.float32(1.0) / (np.float32(scale_in) * sw)                                   # reciprocal first
+        f = acc.astype(np.float32) * r[None, :, None, None]
+        if bias is not None:
+            f = f + np.ascontiguousarray(bias, dtype=np.float32)[None, :, None, None]
+        if eltwise is not None:
+            f = f + from_conv_layout(np.ascontiguousarray(eltwise, dtype=np.float32), d.n, d.oc, d.oh, d.ow, d.out_c)
+        if d.relu:
+            f = np.where(f > 0, f, np.float32(0)).astype(np.float32)
+        flat = to_conv_layout(f.astype(np.float32), d.out_c)
+        if d.odt == DT_F32:
+            return flat, None
+        if out_scale > 0:
+            q, s = oracle.quantize_f32(flat, DT_U8_Q, out_scale, 1)
+        else:
+            q, s = oracle.quantize_f32(flat, DT_U8_Q)
+        return q, s
 
     def bnn_desc(self, n, ic, ih, iw, oc, fh, fw, stride, pad, xnor):
         oh, ow = conv_out_hw(ih, iw, fh, fw, stride, stride, pad, pad, pad, pad)

@@ -438,6 +438,46 @@ def test_per_channel_epilogue(torch_mod, oracle):
             assert np.array_equal(y.cpu().numpy().view(np.int32), want[0].view(np.int32))
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 2, 7, 10, 11, 12, 13, 14, 15, 16])
+def test_per_channel_u8_epilogue_every_kernel_variant(torch_mod, oracle, tile):
+    """bolt_gfx950_mmm_int8_perchannel_u8 (not in the reference): the per-channel fp32 value -- the closed form that
+    test_per_channel_epilogue holds against the reference's per-tensor epilogue -- put through the reference-pinned
+    fp32 -> u8 quantiser with a static scale. Every kernel forced in turn, ragged and full tiles, with and without
+    bias; equal to quantising the fp32 entry point's own output."""
+    torch = torch_mod
+    rng = np.random.default_rng(50 + tile)
+    L = capi.lib()
+    try:
+        capi.check(L.bolt_gfx950_set_option(b"gemm_tile", tile), "set_option")
+        for M, K, N in [(1, 64, 16), (130, 128, 70), (256, 64, 256), (257, 192, 513), (512, 1024, 384), (300, 768, 600),
+                        (128, 576, 128), (512, 256, 512)]:
+            say("per-channel u8", tile, M, K, N)
+            A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+            W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+            off = oracle.offsetC(W, True)
+            acc = oracle.mmm(A, W, off, np.zeros((M, N), np.int32), DT_I32)
+            sI = np.float32(31.75)
+            sW = (1.0 / rng.uniform(0.005, 0.02, size=N)).astype(np.float32)
+            bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+            blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            dA, dB, dOff = dev(torch, A), dev(torch, blob), dev(torch, off)
+            dsI, dsW, dbias = dev(torch, np.array([sI])), dev(torch, sW), dev(torch, bias)
+            for b, db in ((bias, dbias), (None, None)):
+                f = oracle.dequant_per_channel(acc, sI, sW, b)
+                so = np.float32(100.0 / max(1e-6, np.abs(f).max()))     # some values saturate at 1 / 255
+                want, _ = oracle.quantize_f32(f, DT_U8_Q, so, 1)
+                out = torch.full((M, N), 7, dtype=torch.uint8, device="cuda")
+                capi.check(L.bolt_gfx950_mmm_int8_perchannel_u8(M, N, K, dA.data_ptr(), dB.data_ptr(), dOff.data_ptr(), out.data_ptr(),
+                                                                dsI.data_ptr(), dsW.data_ptr(), db.data_ptr() if db is not None else None,
+                                                                float(so)), "mmm_perchannel_u8")
+                capi.check(L.bolt_gfx950_synchronize(), "sync")
+                assert np.array_equal(out.cpu().numpy(), want), (tile, M, K, N, b is not None)
+        assert L.bolt_gfx950_mmm_int8_perchannel_u8(1, 16, 64, dA.data_ptr(), dB.data_ptr(), dOff.data_ptr(), out.data_ptr(),
+                                                    dsI.data_ptr(), dsW.data_ptr(), None, 0.0) == capi.NOT_MATCH
+    finally:
+        L.bolt_gfx950_set_option(b"gemm_tile", -1)
+
+
 def _strided_batch_case(torch, oracle, N, K, batch, copies, with_bias, seed, pad=0):
     """One call of bolt_gfx950_mvm_int8_strided_batch checked row by row: slice b multiplies weight copy
     b % copies (every copy holds DIFFERENT weights, so a wrong copy index shows), has its own activation scale,

@@ -84,6 +84,58 @@ def test_conv_int8_closed_form(oracle, co):
     assert np.array_equal(from_conv_layout(got, n, oc, ih, iw, 8), acc.astype(np.int32))
 
 
+@pytest.mark.parametrize("case", CASES[:5])
+@pytest.mark.parametrize("relu", [False, True])
+def test_conv_perchannel_oracle_reduces_to_the_reference(oracle, co, ref, case, relu):
+    """The per-output-channel composition (ConvOracle.conv_perchannel) with every channel scale equal and no bias is the
+    reference's own fp32 epilogue (convolution_direct.cpp:2406-2422), bit for bit against the compiled reference; with
+    eltwise too. A scale applied as a multiplication instead of a reciprocal, a ReLU before the eltwise sum or a
+    transposed output layout fails here."""
+    n, ic, ih, iw, oc, fh, fw, stride, pad = case
+    xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, sum(case))
+    zero = np.zeros(oc, np.float32)
+    for out_c in (16, 8):
+        d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, relu, DT_F32, out_c)
+        elt = np.random.default_rng(3).standard_normal(n * oc * d.oh * d.ow).astype(np.float32)
+        for e in (None, elt):
+            want, _ = (ref_conv(ref, d, xq, DF_NCHWC8, W, zero, [sI, -1.0, sF], eltwise=e) if out_c == 16
+                       else co.conv(d, xq, W, zero, [sI, -1.0, sF], eltwise=e))
+            got, _ = co.conv_perchannel(oracle, d, xq, W, np.full(oc, sF, np.float32), None, sI, eltwise=e)
+            assert np.array_equal(got.view(np.int32), want.view(np.int32)), (case, out_c, e is not None)
+            got0, _ = co.conv_perchannel(oracle, d, xq, W, np.full(oc, sF, np.float32), zero, sI, eltwise=e)
+            assert np.array_equal(got0.view(np.int32), want.view(np.int32))    # an all-zero bias changes nothing
+
+
+def test_conv_perchannel_oracle_closed_forms(oracle, co):
+    """What the reference cannot pin: (1) with an input that is all zero point the accumulators vanish and the result
+    is the bias of each channel, in the output layout; (2) a channel's scale touches that channel only, and doubling it
+    halves its values exactly; (3) the u8 form is the pinned quantiser applied to the fp32 form, with the maximum taken
+    over the whole tensor (dynamic) or not at all (static)."""
+    n, ic, ih, iw, oc, fh, fw = 2, 16, 6, 5, 24, 3, 3
+    rng = np.random.default_rng(11)
+    xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, 11)
+    sw = rng.uniform(40.0, 160.0, oc).astype(np.float32)
+    d = co.desc(n, ic, ih, iw, oc, fh, fw, 1, 1, False, DT_F32, 16)
+    flat, _ = co.conv_perchannel(oracle, d, np.full_like(xq, 128), W, sw, bias, sI)
+    assert np.array_equal(from_conv_layout(flat, n, oc, d.oh, d.ow, 16), np.broadcast_to(bias[None, :, None, None], (n, oc, d.oh, d.ow)))
+    base, _ = co.conv_perchannel(oracle, d, xq, W, sw, None, sI)
+    sw2 = sw.copy()
+    sw2[5] *= 2
+    dbl, _ = co.conv_perchannel(oracle, d, xq, W, sw2, None, sI)
+    b4, d4 = from_conv_layout(base, n, oc, d.oh, d.ow, 16), from_conv_layout(dbl, n, oc, d.oh, d.ow, 16)
+    assert np.array_equal(np.delete(b4, 5, axis=1), np.delete(d4, 5, axis=1))
+    assert np.array_equal(d4[:, 5] * 2, b4[:, 5]) and np.any(b4[:, 5] != 0)
+    du = co.desc(n, ic, ih, iw, oc, fh, fw, 1, 1, True, DT_U8_Q, 16)
+    df = co.desc(n, ic, ih, iw, oc, fh, fw, 1, 1, True, DT_F32, 16)
+    f32, _ = co.conv_perchannel(oracle, df, xq, W, sw, bias, sI)
+    q, s = co.conv_perchannel(oracle, du, xq, W, sw, bias, sI)
+    assert s == np.float32(127.0) / np.abs(f32).max()
+    assert np.array_equal(q, np.clip(np.rint(f32 * s + np.float32(128.0)), 1, 255).astype(np.uint8))
+    q2, s2 = co.conv_perchannel(oracle, du, xq, W, sw, bias, sI, out_scale=3.5)
+    assert s2 == np.float32(3.5)
+    assert np.array_equal(q2, np.clip(np.rint(f32 * np.float32(3.5) + np.float32(128.0)), 1, 255).astype(np.uint8))
+
+
 @pytest.mark.parametrize("xnor", [True, False])
 @pytest.mark.parametrize("shape", [(1, 32, 4, 4, 32, 3, 3, 1, 1), (2, 64, 5, 6, 32, 1, 1, 1, 0),
                                    (1, 32, 7, 7, 64, 3, 3, 2, 1)])
