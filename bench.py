@@ -341,12 +341,60 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         cb = torch.randn(oc, device=dev, generator=g) * 0.1
         ops = 2.0 * n * ih * iw * oc * ic * 9
         ctmp = torch.empty(64 << 20, dtype=torch.uint8, device=dev)      # reused across calls, as an engine's shared tmp is
+        # Every form is called through the C-ABI with arguments marshalled once, as a C++ caller's are: the synchronous
+        # forms return the new output scale through a host pointer, so whatever the caller spends between two calls
+        # adds to the time per call (the Python wrapper of the tests would add ~15 us of its own).
+        from bolt_amd.capi import (ACTIVATION_RELU, AMD_GFX950_DEVICE, CONVOLUTION_ALGORITHM_DIRECT, ActivationParamSpec,
+                                   tensor1d, tensor4df)
+        act = ActivationParamSpec()
+        act.mode = ACTIVATION_RELU
+        idesc = tensor4df(DT_U8_Q, DF_NCHWC8, n, ic, ih, iw)
+        bdesc = tensor1d(DT_F32, oc)
+        sw = 1.0 / (torch.rand(oc, device=dev, generator=g) * 0.015 + 0.005)       # 1 / U(0.005, 0.02)
+        dsi = torch.tensor([40.0], dtype=torch.float32, device=dev)
+        dso = torch.zeros(1, dtype=torch.float32, device=dev)
+        alg_bytes_u8 = 12882432
+        alg_bytes_i32 = 6422528 * 5 + 36864 + 512
+
+        def entry(nm, t, nbytes, note):
+            res[nm] = {"ms": t, "tops": ops / t / 1e9, "frac_mfma_peak": ops / t / 1e9 / MFMA_PEAK_TOPS,
+                       "algorithmic_bytes": nbytes, "note": note}
         for odt, nm, tdt in ((DT_U8_Q, "u8_dynamic_scale", torch.uint8), (DT_I32, "i32", torch.int32)):
             cout = torch.empty(n * oc * ih * iw, dtype=tdt, device=dev)
-            t = timed(lambda: host_conv.convolution(xq, DF_NCHWC8, n, ic, ih, iw, cblob, ftm, oc, 3, 3, 1, 1, cb,
-                                                    [40.0, -1.0, 80.0], True, odt, DF_NCHWC16, tmp=ctmp, out=cout), 20)
-            res["conv_c3_" + nm] = {"ms": t, "tops": ops / t / 1e9, "frac_mfma_peak": ops / t / 1e9 / MFMA_PEAK_TOPS,
-                                    "algorithmic_bytes": 12882432 if odt == DT_U8_Q else 6422528 * 5 + 36864 + 512}
+            odesc = tensor4df(odt, DF_NCHWC16, n, oc, ih, iw)
+            sc = (C.c_float * 3)(40.0, -1.0, 80.0)
+            args = (idesc, host.ptr(xq), None, ftm, host.ptr(cblob), p, CONVOLUTION_ALGORITHM_DIRECT, bdesc, host.ptr(cb),
+                    ctmp.numel(), host.ptr(ctmp), odesc, host.ptr(cout), sc, act, AMD_GFX950_DEVICE)
+            t = timed(lambda: capi.check(L.convolution_gfx950(*args), "convolution"), 50)
+            entry("conv_c3_" + nm, t, alg_bytes_u8 if odt == DT_U8_Q else alg_bytes_i32,
+                  "convolution_gfx950, one filter scale (the reference's contract: the u8 form returns its output scale "
+                  "through the host pointer, so every call waits for the device once)")
+        cout = torch.empty(n * oc * ih * iw, dtype=torch.uint8, device=dev)
+        odesc = tensor4df(DT_U8_Q, DF_NCHWC16, n, oc, ih, iw)
+        # BASELINE configs[2] as worded: per-output-channel filter scales, fp32 bias, ReLU, one output scale for the tensor
+        sc2 = (C.c_float * 2)(40.0, -1.0)
+
+        def perchannel_dynamic():
+            sc2[1] = -1.0
+            capi.check(L.bolt_gfx950_convolution_int8_perchannel(idesc, host.ptr(xq), None, ftm, host.ptr(cblob), p, host.ptr(sw), bdesc,
+                                                                 host.ptr(cb), ctmp.numel(), host.ptr(ctmp), odesc, host.ptr(cout), sc2, act,
+                                                                 AMD_GFX950_DEVICE), "conv perchannel")
+        entry("conv_c3_u8_perchannel", timed(perchannel_dynamic, 50), alg_bytes_u8 + 512,
+              "per-output-channel filter scales, dynamic output scale returned to the host (two passes of the convolution)")
+        sc3 = (C.c_float * 2)(40.0, 2.5)
+        t = timed(lambda: capi.check(L.bolt_gfx950_convolution_int8_perchannel(
+            idesc, host.ptr(xq), None, ftm, host.ptr(cblob), p, host.ptr(sw), bdesc, host.ptr(cb), ctmp.numel(), host.ptr(ctmp), odesc,
+            host.ptr(cout), sc3, act, AMD_GFX950_DEVICE), "conv perchannel static"), 50)
+        entry("conv_c3_u8_perchannel_static_scale", t, alg_bytes_u8 + 512,
+              "per-output-channel filter scales, calibrated (static) output scale: one pass, nothing returned")
+        for nm, swp, fs, so, note in (
+                ("conv_c3_u8_async", None, 80.0, 0.0, "one filter scale, dynamic output scale left in device memory: no wait for the host"),
+                ("conv_c3_u8_perchannel_async", host.ptr(sw), 0.0, 0.0, "per-output-channel scales, dynamic output scale left in device memory"),
+                ("conv_c3_u8_perchannel_static_async", host.ptr(sw), 0.0, 2.5, "per-output-channel scales, static output scale, asynchronous")):
+            t = timed(lambda: capi.check(L.bolt_gfx950_convolution_async(
+                idesc, host.ptr(xq), None, ftm, host.ptr(cblob), p, bdesc, host.ptr(cb), ctmp.numel(), host.ptr(ctmp), odesc, host.ptr(cout),
+                host.ptr(dsi), fs, swp, host.ptr(dso), so, act), "conv async"), 50)
+            entry(nm, t, alg_bytes_u8 + (512 if swp else 0), note)
     # -- C5: XNOR convolution 64x256x28x28 -> 256, fp32 out
     if want("bnn"):
         n, ic, ih, iw, oc = 64, 256, 28, 28, 256

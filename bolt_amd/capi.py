@@ -250,6 +250,7 @@ SIGNATURES = {
     "bolt_gfx950_convolution_int8_perchannel": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, _vp,
                                                           TensorDesc, _vp, _u32, _vp, TensorDesc, _vp, _f32p,
                                                           ActivationParamSpec, C.c_int]),
+    "bolt_gfx950_convolution_async_tmp_bytes": (C.c_int, [TensorDesc, TensorDesc, TensorDesc, ConvolutionParamSpec, _u32p]),
     "bolt_gfx950_convolution_async": (C.c_int, [TensorDesc, _vp, _vp, TensorDesc, _vp, ConvolutionParamSpec, TensorDesc, _vp,
                                                 _u32, _vp, TensorDesc, _vp, _vp, C.c_float, _vp, _vp, C.c_float,
                                                 ActivationParamSpec]),

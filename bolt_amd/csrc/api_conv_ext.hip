@@ -26,7 +26,26 @@ struct ConvExt {
     float filterScale = 0;
     float staticOut = 0;              // u8 result: > 0 = quantise with this scale, else dynamic
     float *dscaleO = nullptr;         // device word that receives the output scale; null: the context's pinned word
+    // where a one-pass u8 launch may park its values should its grid-wide agreement be abandoned (asynchronous form:
+    // 4 bytes per output element); null in the synchronous forms, which hand an abandoned launch back to the host
+    void *spill = nullptr;
+    bool host_waits = false;          // synchronous form: the scale is taken from the pinned word, a NaN there = redo
+    F32 *host_scale = nullptr;        //   ... and handed back here
 };
+
+size_t conv_out_elems(const ConvShape &s)
+{
+    return (size_t)s.n * s.oc * s.oh * s.ow;
+}
+
+// tmp of the asynchronous form: the synchronous call's, then room for one 32-bit value per output element
+size_t conv_async_tmp_layout(const ConvShape &s, size_t *spill_off)
+{
+    size_t off;
+    const size_t base = (conv_tmp_layout(s, &off) + 255) / 256 * 256;
+    *spill_off = base;
+    return base + conv_out_elems(s) * 4;
+}
 
 // the context's two arrays of max slots, clear before the first two-pass call (and after one that failed half way)
 EE conv_ws_ready(Ctx &c)
@@ -123,6 +142,40 @@ EE conv_device_ext(const ConvShape &s, DataFormat idf, const void *input, const 
     if (e != SUCCESS) {
         return e;
     }
+    // ONE pass where the filter-panel kernel runs and all its workgroups are resident at once: they agree on the
+    // tensor-wide maximum with their values still in registers (the convolution is computed once instead of twice)
+    const uint32_t M_pix = s.n * s.oh * s.ow;
+    const bool onepass = direct && conv_panel_grid(M_pix) <= conv_onepass_max_grid(s.Kp) && (x.host_waits || x.spill);
+    if (onepass) {
+        g.C = output;
+        g.C32 = (float *)x.spill;
+        g.conv.absmax = c.conv_ws[c.conv_ws_next];  // touched only if the agreement is abandoned; left clear again
+        g.sync = c.fsync.next(conv_panel_grid(M_pix));
+        if (per_channel) {
+            g.conv.ch_out = CONV_CH_U8;
+            g.epi.factor = 0;
+        } else {
+            g.epi.mode = EPI_U8;
+        }
+        HIP_TRY(launch_conv_u8s8(g, c.stream));
+        if (!x.host_waits) {
+            return SUCCESS;
+        }
+        bool gave_up = false;
+        float got = 0;
+        EE te = take_scale(c, &got, &gave_up);
+        if (te != SUCCESS) {
+            return te;
+        }
+        if (!gave_up) {
+            *x.host_scale = got;
+            return SUCCESS;
+        }
+        // the bounded wait expired (other work held the CUs): nothing was stored, the two passes below redo it
+        g_fused_fallbacks.fetch_add(1);
+        memset(&g.sync, 0, sizeof(g.sync));
+        arm_scale(c);
+    }
     uint32_t *mine = c.conv_ws[c.conv_ws_next], *other = c.conv_ws[c.conv_ws_next ^ 1];
     c.conv_ws_dirty = true;  // until both passes are enqueued
     g.conv.absmax = mine;
@@ -147,7 +200,7 @@ EE conv_device_ext(const ConvShape &s, DataFormat idf, const void *input, const 
     HIP_TRY(launch_conv_u8s8(g, c.stream));
     c.conv_ws_next ^= 1;
     c.conv_ws_dirty = false;
-    return SUCCESS;
+    return x.host_waits ? take_scale(c, x.host_scale) : SUCCESS;
 }
 
 EE check_common(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, ActivationParamSpec act,
@@ -221,6 +274,8 @@ EE bolt_gfx950_convolution_int8_perchannel(TensorDesc inputDesc, const void *inp
     const bool dynamic = odt == DT_U8_Q && !(x.staticOut > 0);
     if (dynamic) {
         x.dscaleO = cx.hscale_dev;  // the new output scale goes straight into pinned host memory
+        x.host_waits = true;
+        x.host_scale = &scale[1];
     }
     if (arch == AMD_GFX950_DEVICE) {
         if (((uintptr_t)tmp & 15) || ((uintptr_t)filter & 15) || ((uintptr_t)output & 15) || ((uintptr_t)input & 7)) {
@@ -230,11 +285,7 @@ EE bolt_gfx950_convolution_int8_perchannel(TensorDesc inputDesc, const void *inp
         if (dynamic) {
             arm_scale(cx);
         }
-        e = conv_device_ext(s, inputDesc.df, input, eltwiseInput, filter, bias, tmp, odt, outputDesc.df, output, relu, x);
-        if (e != SUCCESS) {
-            return e;
-        }
-        return dynamic ? take_scale(cx, &scale[1]) : SUCCESS;
+        return conv_device_ext(s, inputDesc.df, input, eltwiseInput, filter, bias, tmp, odt, outputDesc.df, output, relu, x);
     }
     Stage st;
     const size_t inB = (size_t)s.n * s.ic * s.ih * s.iw;
@@ -266,7 +317,27 @@ EE bolt_gfx950_convolution_int8_perchannel(TensorDesc inputDesc, const void *inp
     }
     HIP_TRY(hipMemcpyAsync(output, dO, outB, hipMemcpyDeviceToHost, cx.stream));
     HIP_TRY(hipStreamSynchronize(cx.stream));
-    return dynamic ? take_scale(cx, &scale[1]) : SUCCESS;
+    return SUCCESS;
+}
+
+EE bolt_gfx950_convolution_async_tmp_bytes(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec p, U32 *bytes)
+{
+    if (!bytes) {
+        return NULL_POINTER;
+    }
+    ConvShape s;
+    EE e = conv_shape(inputDesc, filterDesc, outputDesc, p, &s);
+    if (e != SUCCESS) {
+        return e;
+    }
+    size_t spill_off;
+    const size_t total = conv_async_tmp_layout(s, &spill_off);
+    if (total > 0xffffffffull) {
+        return NOT_SUPPORTED;
+    }
+    *bytes = (U32)total;
+    return SUCCESS;
 }
 
 EE bolt_gfx950_convolution_async(TensorDesc inputDesc, const void *input, const void *eltwiseInput, TensorDesc filterDesc,
@@ -318,6 +389,10 @@ EE bolt_gfx950_convolution_async(TensorDesc inputDesc, const void *input, const 
     x.filterScale = filterScale;
     x.staticOut = staticOutputScale;
     x.dscaleO = dscaleO;
+    size_t spill_off;
+    if (tmpBytes >= conv_async_tmp_layout(s, &spill_off)) {
+        x.spill = (U8 *)tmp + spill_off;  // room for the one-pass form's parking area
+    }
     return conv_device_ext(s, inputDesc.df, input, eltwiseInput, filter, bias, tmp, odt, outputDesc.df, output,
         activationDesc.mode == ACTIVATION_RELU, x);
 }

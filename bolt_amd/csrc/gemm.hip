@@ -287,9 +287,63 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
             }
         }
         const uint32_t outcome = grid_max_sync(a.sync, lm, (int *)smem);
-        if (outcome == kGridAbandoned) {  // nothing is stored; the host sees a NaN scale and runs the two passes
+        if (outcome == kGridAbandoned && !a.C32) {  // nothing is stored; the host sees a NaN scale and runs the two passes
             if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
                 *a.conv.dscale_out = __int_as_float(0x7fc00000);
+            }
+            return;
+        }
+        if (outcome == kGridAbandoned) {
+            // Asynchronous form: no host is waiting, and no workgroup may wait for another any more. Every workgroup
+            // parks its int32 values (bias folded, ReLU applied) in C32 -- laid out like the result -- and folds its
+            // maximum into the scratch slots; the last one to arrive requantises the whole tensor alone. Slow, and
+            // only reached when other work held the CUs.
+#pragma unroll
+            for (int x = 0; x < TM; ++x) {
+                const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+                if (m >= a.M) {
+                    continue;
+                }
+                const uint32_t img = m / a.conv.OHW, pix = m - img * a.conv.OHW;
+#pragma unroll
+                for (int y = 0; y < TN; ++y) {
+                    const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+                    if (n >= a.N) {
+                        continue;
+                    }
+                    v4i t;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int v = (int)((uint32_t)acc[x][y][c] + base[y][c]);
+                        t[c] = (a.conv.relu && v < 0) ? 0 : v;
+                    }
+                    *(v4i *)((int32_t *)a.C32 + (size_t)img * a.N * a.conv.OHW + cblk_off[y] + (size_t)pix * cblk_w[y]) = t;
+                }
+            }
+            lm = wave_reduce_max_i(lm);
+            if (lane == 0) {
+                ws_fold_max(a.conv.absmax, blockIdx.x * 8 + wave, lm);
+            }
+            if (grid_last_arrival(a.sync, (int *)smem)) {
+                const int mx = ws_read_max(a.conv.absmax);
+                const float fct = (mx == 0) ? 1.0f : 127.0f / (float)mx;
+                if (threadIdx.x == 0 && a.conv.dscale_out) {
+                    *a.conv.dscale_out = conv_acc_scale(a.conv) * fct;
+                }
+                const uint32_t total4 = (a.M * a.N) / 4;  // N is a multiple of 8
+                for (uint32_t k = threadIdx.x; k < total4; k += blockDim.x) {
+                    const v4i t = ((const v4i *)a.C32)[k];
+                    unsigned b[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        b[c] = usat8_u(rne_i32((float)t[c] * fct + 128.0f));
+                    }
+                    ((uint32_t *)a.C)[k] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                }
+                __syncthreads();  // every wave has read the maximum
+                for (uint32_t k = threadIdx.x; k < kWsWords; k += blockDim.x) {
+                    a.conv.absmax[k] = 0;  // the slots go back clear
+                }
             }
             return;
         }
@@ -742,8 +796,8 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
 // the static scale epi.factor or the dynamic one 127 / max|f| from the scratch slots; or only max|f| folded into those
 // slots. With every sW[oc] equal, no bias and an fp32 result this is the reference's epilogue bit for bit.
 template <int WM, int WN, int TM, int TN>
-__device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[TM][TN], uint32_t lane, uint32_t wave,
-    uint32_t m0, uint32_t n0)
+__device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
+    uint32_t wave, uint32_t m0, uint32_t n0)
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -780,6 +834,94 @@ __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[T
             cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
             cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
         }
+    }
+    if (out == CONV_CH_U8 && a.sync.slots) {
+        // ONE pass (filter-panel kernel, every workgroup resident): the fp32 values replace the accumulators in their
+        // registers, the workgroups agree on max|f| (smem: 18 ints of LDS nobody reads tiles from), and each quantises
+        // its own values. Should that agreement be abandoned: with no spill buffer (synchronous form) nothing is
+        // stored and a NaN scale tells the host to run the two passes; with one (C32, asynchronous form) every
+        // workgroup parks its fp32 values there and the last to arrive quantises the tensor alone.
+        float amax = 0.0f;
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float f = (float)(int)((uint32_t)acc[x][y][c] + base[y][c]) * qs[y][c];
+                    if (a.epi.bias) {
+                        f = f + bs[y][c];
+                    }
+                    if (a.conv.relu && !(f > 0.0f)) {
+                        f = 0.0f;
+                    }
+                    acc[x][y][c] = __float_as_int(f);
+                    const float af = fabsf(f);
+                    amax = (m < a.M && n < a.N && af > amax) ? af : amax;  // a NaN never wins, as in the quantiser
+                }
+            }
+        }
+        const uint32_t outcome = grid_max_sync(a.sync, (int)__float_as_uint(amax), (int *)smem);
+        if (outcome == kGridAbandoned && !a.C32) {
+            if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+                *a.conv.dscale_out = __int_as_float(0x7fc00000);
+            }
+            return;
+        }
+        const bool parked = outcome == kGridAbandoned;
+        const float mxf = __uint_as_float(outcome);
+        const float so = (mxf == 0.0f) ? 1.0f : 127.0f / mxf;
+        if (!parked && blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out) {
+            *a.conv.dscale_out = so;
+        }
+#pragma unroll
+        for (int x = 0; x < TM; ++x) {
+            const uint32_t m = m0 + (wm * TM + x) * 16 + i;
+            if (m >= a.M) {
+                continue;
+            }
+            const uint32_t img = m / a.conv.OHW, pix = m - img * a.conv.OHW;
+#pragma unroll
+            for (int y = 0; y < TN; ++y) {
+                const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+                if (n >= a.N) {
+                    continue;
+                }
+                const size_t idx = (size_t)img * a.N * a.conv.OHW + cblk_off[y] + (size_t)pix * cblk_w[y];
+                if (parked) {
+                    *(v4i *)((int32_t *)a.C32 + idx) = acc[x][y];
+                } else {
+                    const unsigned b0 = q_u8(__int_as_float(acc[x][y][0]), so), b1 = q_u8(__int_as_float(acc[x][y][1]), so);
+                    const unsigned b2 = q_u8(__int_as_float(acc[x][y][2]), so), b3 = q_u8(__int_as_float(acc[x][y][3]), so);
+                    *(uint32_t *)((uint8_t *)a.C + idx) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+                }
+            }
+        }
+        if (parked) {
+            const int wmax = wave_reduce_max_i((int)__float_as_uint(amax));
+            if (lane == 0) {
+                ws_fold_max(a.conv.absmax, blockIdx.x * 8 + wave, wmax);
+            }
+            if (grid_last_arrival(a.sync, (int *)smem)) {
+                const float mx = __uint_as_float((uint32_t)ws_read_max(a.conv.absmax));
+                const float sl = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+                if (threadIdx.x == 0 && a.conv.dscale_out) {
+                    *a.conv.dscale_out = sl;
+                }
+                const uint32_t total4 = (a.M * a.N) / 4;
+                for (uint32_t k = threadIdx.x; k < total4; k += blockDim.x) {
+                    const v4f t = ((const v4f *)a.C32)[k];
+                    ((uint32_t *)a.C)[k] = q_u8(t.x, sl) | (q_u8(t.y, sl) << 8) | (q_u8(t.z, sl) << 16) | (q_u8(t.w, sl) << 24);
+                }
+                __syncthreads();
+                for (uint32_t k = threadIdx.x; k < kWsWords; k += blockDim.x) {
+                    a.conv.absmax[k] = 0;
+                }
+            }
+        }
+        return;
     }
     float s = 0.0f;
     if (out == CONV_CH_U8) {
@@ -898,7 +1040,7 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
         } else if (a.epi.mode == EPI_F32_CH) {
             epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_CONV_CH) {
-            epilogue_conv_ch<WM, WN, TM, TN>(a, acc, lane, wave, m0, n0);
+            epilogue_conv_ch<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
         } else {
             epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
         }
@@ -1082,7 +1224,7 @@ __device__ __forceinline__ void conv_publish_scale(GemmArgs &a, uint32_t wave)
             }
         }
         a.conv.dscale_out = nullptr;
-    } else if (a.epi.mode == EPI_CONV_CH && a.conv.ch_out == CONV_CH_U8 && a.conv.dscale_out) {
+    } else if (a.epi.mode == EPI_CONV_CH && a.conv.ch_out == CONV_CH_U8 && a.conv.dscale_out && !a.sync.slots) {
         // the per-channel form: the scale the u8 result is quantised with (given, or from the first pass's max|f|)
         if (blockIdx.x == 0 && wave == 0) {
             float s = a.epi.factor;

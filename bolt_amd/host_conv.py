@@ -114,11 +114,20 @@ def convolution_perchannel(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride,
 
 
 def convolution_async(x, idf, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, bias, dscale_in, filter_scale, scale_w,
-                      dscale_out, relu, odt, odf=DF_NCHWC16, static_out=0.0, eltwise=None, dilation=1, tmp=None, out=None):
+                      dscale_out, relu, odt, odf=DF_NCHWC16, static_out=0.0, eltwise=None, dilation=1, tmp=None, out=None,
+                      one_pass_room=True):
     """bolt_gfx950_convolution_async: device tensors only; dscale_in / dscale_out are one-element fp32 device tensors
-    (input scale read, output scale left there); scale_w None = one filter scale `filter_scale`, else fp32 [oc] device."""
+    (input scale read, output scale left there); scale_w None = one filter scale `filter_scale`, else fp32 [oc] device.
+    one_pass_room: hand over a tmp of bolt_gfx950_convolution_async_tmp_bytes (a dynamic u8 result may then run in one
+    pass) instead of the synchronous call's size (always two passes)."""
     arch, p, idesc, odesc, nbytes, tmp, out = _conv_call_setup(x, idf, n, ic, ih, iw, ftm, oc, fh, fw, stride, pad, odt, odf,
                                                                dilation, tmp, out)
+    if one_pass_room:
+        b = C.c_uint32(0)
+        check(lib().bolt_gfx950_convolution_async_tmp_bytes(idesc, ftm, odesc, p, C.byref(b)), "conv_async_tmp_bytes")
+        if tmp.numel() < b.value:
+            tmp = _empty_like_mode(x, b.value)
+        nbytes = b.value
     act = ActivationParamSpec()
     act.mode = ACTIVATION_RELU if relu else ACTIVATION_NULL
     e = lib().bolt_gfx950_convolution_async(idesc, ptr(x), ptr(eltwise), ftm, ptr(blob), p, tensor1d(DT_F32, oc), ptr(bias),

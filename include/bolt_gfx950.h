@@ -233,7 +233,15 @@ EE bolt_gfx950_convolution_int8_perchannel(TensorDesc inputDesc, const void *inp
  *                   (dscaleO may be NULL for DT_F32 / DT_I32). bias is required, as there.
  *   scaleW != NULL: the per-channel form above; DT_U8_Q with staticOutputScale > 0 quantises with that scale, otherwise
  *                   dynamically; *dscaleO = the scale used (untouched for DT_F32).
- * A dynamic u8 result runs the convolution twice (maximum, then store); no launch needs all its workgroups resident. */
+ * tmp: at least convolution_infer_forward_tmp_bytes_gfx950. A dynamic u8 result then runs the convolution twice
+ * (maximum, then store). With the bolt_gfx950_convolution_async_tmp_bytes it runs ONCE where the shape allows (at most
+ * 64 output channels, a reduction of at most 1024, channels a multiple of 16, every workgroup resident at once): the
+ * workgroups agree on the tensor-wide maximum with their values in registers. The extra 4 bytes per output element are
+ * only written if that agreement is abandoned (other work held the CUs; bounded wait, bolt_gfx950_set_option
+ * "quantize_fused_spin"): the workgroups then park their values there and the last one to finish quantises the
+ * tensor alone -- slow, correct, and still without the host. */
+EE bolt_gfx950_convolution_async_tmp_bytes(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
+    ConvolutionParamSpec convParamSpec, U32 *bytes);
 EE bolt_gfx950_convolution_async(TensorDesc inputDesc, const void *input, const void *eltwiseInput, TensorDesc filterDesc,
     const void *filter, ConvolutionParamSpec convParamSpec, TensorDesc biasDesc, const void *bias, U32 tmpBytes, void *tmp,
     TensorDesc outputDesc, void *output, const float *dscaleI, F32 filterScale, const F32 *scaleW, float *dscaleO,

@@ -191,8 +191,9 @@ def test_conv_perchannel_config3(torch_mod, oracle, co):
     assert np.float32(sc[1]) == np.float32(2.5) and np.array_equal(u8s, qs)
 
 
+@pytest.mark.parametrize("room", [True, False], ids=["one_pass_room", "two_passes"])
 @pytest.mark.parametrize("case", CASES)
-def test_conv_async_equals_the_synchronous_calls(torch_mod, oracle, co, case):
+def test_conv_async_equals_the_synchronous_calls(torch_mod, oracle, co, case, room):
     """bolt_gfx950_convolution_async with the input scale in device memory: bytes and the scale it leaves on the device
     equal what convolution_gfx950 (one filter scale: u8, fp32, int32) and the per-channel call (fp32, u8 dynamic, u8
     static) return; two calls in a row, the second on other data, so that the alternating maximum slots are used."""
@@ -213,7 +214,7 @@ def test_conv_async_equals_the_synchronous_calls(torch_mod, oracle, co, case):
             want = host_conv.convolution(dx, DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, db, sc, True, odt)
             dso = torch.tensor([-5.0], dtype=torch.float32, device="cuda")
             got = host_conv.convolution_async(dx, DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, db, dsi,
-                                              float(sF), None, dso, True, odt)
+                                              float(sF), None, dso, True, odt, one_pass_room=room)
             capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
             assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), (case, rep, odt)
             assert np.float32(dso.item()) == np.float32(sc[1]), (case, odt, dso.item(), sc[1])
@@ -224,7 +225,7 @@ def test_conv_async_equals_the_synchronous_calls(torch_mod, oracle, co, case):
                                                     True, odt)
             dso = torch.tensor([-5.0], dtype=torch.float32, device="cuda")
             got = host_conv.convolution_async(dx, DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, db, dsi, 0.0, dsw,
-                                              dso, True, odt, static_out=so)
+                                              dso, True, odt, static_out=so, one_pass_room=room)
             capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
             assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), (case, rep, odt, so)
             if odt == DT_U8_Q:
@@ -257,3 +258,59 @@ def test_conv_async_chain_never_touches_the_host(torch_mod, oracle, co):
     capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
     assert torch.equal(amid, mid) and torch.equal(got, want)
     assert np.float32(dmid.item()) == np.float32(s1[1]) and np.float32(dout.item()) == np.float32(s2[1])
+
+
+def test_conv_one_pass_forms_when_their_wait_gives_up(torch_mod, oracle, co):
+    """The one-pass u8 forms wait a bounded number of polls for all their workgroups. With the bound forced to one poll
+    from the host the launches of more than a few workgroups give up, and every kernel still exits normally:
+    the synchronous per-channel call gets a NaN scale and redoes the convolution in two passes (counted); the
+    asynchronous calls have no host to fall back on -- their workgroups park their values in tmp and the last one to
+    arrive quantises the tensor alone. Same bytes and scales as without the bound, and the maximum slots are left
+    clear: a two-pass call right behind still gets its own maximum."""
+    import ctypes as C
+    torch = torch_mod
+    L = capi.lib()
+    cases = [(8, 64, 56, 56, 64, 3, 3, 1, 1), (3, 16, 10, 9, 40, 3, 3, 1, 1), (5, 32, 13, 13, 64, 1, 1, 1, 0)]
+    want = {}
+    for case in cases:
+        n, ic, ih, iw, oc, fh, fw, stride, pad = case
+        xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, sum(case))
+        sw = channel_scales(oc, sum(case))
+        d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, True, DT_U8_Q, 16)
+        want[case] = (xq, sI, W, sF, bias, sw, co.conv(d, xq, W, bias, [sI, -1.0, sF]), co.conv_perchannel(oracle, d, xq, W, sw, bias, sI))
+    before = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(before)), "counter")
+
+    def run_all(tag):
+        for case in cases:
+            print("conv one-pass give-up", tag, case, flush=True)
+            n, ic, ih, iw, oc, fh, fw, stride, pad = case
+            xq, sI, W, sF, bias, sw, (w1, s1), (wc, sc_) = want[case]
+            p = capi.conv_param_spec(oc, fh, fw, stride, pad)
+            blob, ftm = host_conv.transform_filter(put(torch, W), oc, ic, fh, fw, p)
+            dx, db, dsw = put(torch, xq), put(torch, bias), put(torch, sw)
+            dsi = torch.tensor([float(sI)], dtype=torch.float32, device="cuda")
+            sc = [sI, -1.0]
+            got = host_conv.convolution_perchannel(dx, DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, dsw, db, sc, True, DT_U8_Q)
+            capi.check(L.bolt_gfx950_synchronize(), "sync")
+            assert np.float32(sc[1]) == sc_ and np.array_equal(got.cpu().numpy(), wc), (tag, case, "per-channel sync")
+            for swp, fs, (wb, wsc) in ((None, float(sF), (w1, s1[1])), (dsw, 0.0, (wc, sc_))):
+                for room in (True, False, True):
+                    dso = torch.tensor([-5.0], dtype=torch.float32, device="cuda")
+                    got = host_conv.convolution_async(dx, DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad, db, dsi, fs, swp,
+                                                      dso, True, DT_U8_Q, one_pass_room=room)
+                    capi.check(L.bolt_gfx950_synchronize(), "sync")
+                    assert np.float32(dso.item()) == np.float32(wsc), (tag, case, swp is not None, room, dso.item(), wsc)
+                    assert np.array_equal(got.cpu().numpy(), wb), (tag, case, swp is not None, room)
+    capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 1), "set_option")
+    try:
+        run_all("bound 1")
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"quantize_fused_spin", 0), "set_option")
+    after = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(after)), "counter")
+    assert after.value > before.value, "no synchronous launch gave up: the test did not exercise the fallback"
+    run_all("default bound")
+    final = C.c_ulonglong(0)
+    capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(final)), "counter")
+    assert final.value == after.value
