@@ -161,6 +161,7 @@ SIGNATURES = {
     "bolt_gfx950_free": (None, [_vp]),
     "bolt_gfx950_memcpy_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),
     "bolt_gfx950_memcpy_d2h": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "bolt_gfx950_memcpy_d2d": (C.c_int, [_vp, _vp, C.c_size_t]),
     "bolt_gfx950_timer_start": (C.c_int, []),
     "bolt_gfx950_timer_stop": (C.c_int, [_f32p]),
     "matrix_matrix_multiply_tmp_bytes_gfx950": (C.c_int, [TensorDesc, TensorDesc, _u32p, C.c_int]),

@@ -531,6 +531,16 @@ EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes)
     return SUCCESS;
 }
 
+EE bolt_gfx950_memcpy_d2d(void *dst, const void *src, size_t bytes)
+{
+    EE e = ensure_init();
+    if (e != SUCCESS) {
+        return e;
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));  // ordered on the library's stream
+    return SUCCESS;
+}
+
 EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes)
 {
     EE e = ensure_init();

@@ -80,6 +80,7 @@ void *bolt_gfx950_malloc(size_t bytes);
 void bolt_gfx950_free(void *dptr);
 EE bolt_gfx950_memcpy_h2d(void *dst, const void *src, size_t bytes);
 EE bolt_gfx950_memcpy_d2h(void *dst, const void *src, size_t bytes);
+EE bolt_gfx950_memcpy_d2d(void *dst, const void *src, size_t bytes);  /* enqueued on the library's stream, does not wait */
 /* Event pair on the library stream; stop returns the elapsed milliseconds after waiting. */
 EE bolt_gfx950_timer_start(void);
 EE bolt_gfx950_timer_stop(float *ms);
