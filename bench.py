@@ -158,6 +158,39 @@ def cpu_baseline_extras(ref, blob, tmp, xs, sI, sW0, seconds):
                         "ms": dt / n_done * 1e3, "sample": "%d calls in %.1f s" % (n_done, dt)})
         ref.lib.ref_set_threads(1)
     res["gemm_int8_matrix_matrix_multiply"] = gem
+    # the reference's int8 convolution at BASELINE configs[2] (32 x 64 x 56 x 56, 3 x 3, 64 -> 64, ReLU, u8 result with the
+    # dynamic output scale) -- convolution_int8 has no OpenMP: one thread -- and its fp32 -> u8 quantiser at 4096 x 3072
+    n, ic, ih, iw, oc = 32, 64, 56, 56, 64
+    xq = rng.integers(128, 256, size=n * ic * ih * iw, dtype=np.uint8)
+    Wc = rng.integers(-127, 128, size=(oc, ic, 3, 3), dtype=np.int8)
+    cb = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    cout = np.zeros(n * oc * ih * iw + 64, np.uint8)
+    cs = (C.c_float * 3)(40.0, -1.0, 80.0)
+    secs = C.c_double(0)
+    ref.lib.ref_conv_int8_loop.argtypes = [u32] * 4 + [C.c_int] + [u32] * 11 + [C.c_int] + [vp] * 4 + [C.c_int, C.c_int, vp, C.c_int,
+                                                                                                  C.POINTER(C.c_double)]
+    reps, total, calls = 2, 0.0, 0
+    while total < seconds / 2:
+        assert ref.lib.ref_conv_int8_loop(n, ic, ih, iw, 2, oc, 3, 3, 1, 1, 1, 1, 1, 1, ih, iw, 1, xq.ctypes.data_as(vp),
+                                          Wc.ctypes.data_as(vp), cb.ctypes.data_as(vp), C.cast(cs, vp), 1, 10, cout.ctypes.data_as(vp),
+                                          reps, C.byref(secs)) == 0
+        total += secs.value
+        calls += reps
+    ops = 2.0 * n * ih * iw * oc * ic * 9
+    res["conv_c3_u8_dynamic_scale"] = {"ms": total / calls * 1e3, "tops": ops * calls / total / 1e12, "threads": 1,
+                                       "sample": "%d calls of convolution_int8 in %.1f s (filter transformed once, outside the clock)" % (calls, total)}
+    nq = 4096 * 3072
+    xf = rng.standard_normal(nq).astype(np.float32)
+    qo = np.zeros(nq + 64, np.uint8)
+    qs = (C.c_float * 1)(-1.0)
+    n_done, t0 = 0, time.perf_counter()
+    while n_done < 2 or time.perf_counter() - t0 < seconds / 3:
+        qs[0] = -1.0
+        assert ref.lib.ref_quantize(6, xf.ctypes.data_as(vp), u32(nq), 10, qo.ctypes.data_as(vp), qs, 0) == 0
+        n_done += 1
+    dt = time.perf_counter() - t0
+    res["quantize_f32_u8_dynamic"] = {"ms": dt / n_done * 1e3, "gbps": nq * 9 * n_done / dt / 1e9, "threads": 1,
+                                      "algorithmic_bytes": nq * 9, "sample": "%d calls of quantize_x86 on 4096 x 3072 fp32 in %.1f s" % (n_done, dt)}
     return res
 
 

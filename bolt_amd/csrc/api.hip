@@ -2749,8 +2749,8 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
 // ---- int8 LSTM cell (compute/tensor/src/cpu/x86/int8/lstm.cpp:20-179) -----------------------------------
 namespace {
 struct LstmShape {
-    U32 batch, xDim, hDim, N, K;
-    size_t quantOff, dscaleOff, scaleWOff, interOff, total;
+    U32 batch, xDim, hDim, column, N, K;  // column = num_projection when there is one (lstm.cpp:60-62), else hDim
+    size_t quantOff, dscaleOff, scaleWOff, interOff, actOff, total;
 };
 
 EE lstm_shape(TensorDesc xDesc, RNNParamSpec p, LstmShape *s)
@@ -2760,18 +2760,23 @@ EE lstm_shape(TensorDesc xDesc, RNNParamSpec p, LstmShape *s)
     if (get2d(xDesc, &dt, &df, &s->batch, &s->xDim) != SUCCESS) {
         return NOT_MATCH;
     }
-    if (p.mode != RNN_LSTM || p.num_projection > 0) {
+    if (p.mode != RNN_LSTM) {
         return NOT_SUPPORTED;
     }
     s->hDim = p.num_outputs;
-    s->N = 4 * s->hDim;
+    s->column = p.num_projection > 0 ? p.num_projection : s->hDim;
+    if (p.num_projection > 0 && s->hDim % 32 != 0) {
+        return NOT_SUPPORTED;  // the projection matrix comes in blocks of 32 rows (DF_NKN32)
+    }
+    s->N = 4 * s->column;
     s->K = s->xDim + s->hDim;
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
     s->quantOff = 0;
     s->dscaleOff = up((size_t)s->batch * s->K);
     s->scaleWOff = s->dscaleOff + up((size_t)s->batch * 4);
     s->interOff = s->scaleWOff + up((size_t)s->N * 4);
-    s->total = s->interOff + up((size_t)s->batch * s->N * 4);
+    s->actOff = s->interOff + up((size_t)s->batch * s->N * 4);
+    s->total = s->actOff + (p.num_projection > 0 ? up((size_t)s->batch * s->column * 4) : 0);
     return SUCCESS;
 }
 }  // namespace
@@ -2817,9 +2822,9 @@ EE rnn_transform_filter_gfx950(TensorDesc filterDesc, const void *filter, RNNPar
     DataFormat df;
     U32 N, K;
     if (get2d(filterDesc, &dt, &df, &N, &K) != SUCCESS || dt != DT_I8 || df != DF_NORMAL) {
-        return NOT_MATCH;   // s8 [4 * num_outputs][xDim + num_outputs], row-major
+        return NOT_MATCH;   // s8 [4 * column][xDim + num_outputs], row-major (column = num_projection or num_outputs)
     }
-    if (p.mode != RNN_LSTM || p.num_projection > 0 || N != 4 * p.num_outputs) {
+    if (p.mode != RNN_LSTM || N != 4 * (p.num_projection > 0 ? p.num_projection : p.num_outputs)) {
         return NOT_SUPPORTED;
     }
     const size_t mat = packed_matrix_bytes(N, K), mvmB = mat + (size_t)N * 4;
@@ -2925,11 +2930,17 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
     Stage st;
     const size_t blobB = (size_t)packed_matrix_bytes(s.N, s.K) + (size_t)s.N * 4;   // matrix-vector part
     const size_t filterB = blobB + (fdf == DF_NKNx_NKN32 ? (size_t)packed_matrix_bytes(s.N, s.K) : 0);
-    const size_t stateB = (size_t)s.batch * 2 * s.hDim * 4;
+    const size_t stateB = (size_t)s.batch * (s.column + s.hDim) * 4;
+    const bool projected = p.num_projection > 0;
+    const size_t projB = projected ? (size_t)s.hDim * s.column * 4 : 0;
+    if (projected && (!filter[1] || filterDesc[1].dt != DT_F32)) {
+        return fail(NOT_MATCH, "a projection needs filter[1]: fp32, DF_NKN32 layout [num_outputs / 32][num_projection][32]");
+    }
     bg::LstmArgs a;
     a.batch = s.batch;
     a.xdim = s.xDim;
-    a.hdim = a.column = s.hDim;
+    a.hdim = s.hDim;
+    a.column = s.column;
     a.scale_in = scale[0];
     a.forget_bias = p.forget_bias;
     a.zoneout_cell = p.zoneout_cell;
@@ -2945,8 +2956,13 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
         dState = (float *)st.get(stateB);
         dOut = (float *)st.get((size_t)s.batch * s.hDim * 4);
         dT = (U8 *)st.get(s.total);
-        if (!dx || !db || !w || !dState || !dOut || !dT) {
+        float *dP = projected ? (float *)st.get(projB) : nullptr;
+        if (!dx || !db || !w || !dState || !dOut || !dT || (projected && !dP)) {
             return fail(ALLOC_FAILED, "device staging");
+        }
+        if (projected) {
+            HIP_TRY(hipMemcpyAsync(dP, filter[1], projB, hipMemcpyHostToDevice, c.stream));
+            a.proj = dP;
         }
         for (U32 m = 0; m < s.batch; ++m) {
             if (s.xDim) {
@@ -2974,12 +2990,14 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
         a.state = (float *)state;
         a.out = (float *)output;
         a.out_stride = batchStrideH;
+        a.proj = projected ? (const float *)filter[1] : nullptr;
     }
     a.quant = dT + s.quantOff;
     a.dscale = (float *)(dT + s.dscaleOff);
     float *scaleW = (float *)(dT + s.scaleWOff);
     float *inter = (float *)(dT + s.interOff);
     a.inter = inter;
+    a.act = projected ? (float *)(dT + s.actOff) : nullptr;
     if (fdf == DF_NKNx_NKN32 && s.batch >= (U32)g_lstm_gemm_rows) {
         // enough rows to share one pass over the weight: all rows through the matrix cores as one GEMM with exact
         // int32 results; the gates kernel dequantises them with each row's own scale, in the arithmetic of the
@@ -3011,6 +3029,9 @@ EE rnncell_gfx950(TensorDesc xDesc, const void *currentX, const TensorDesc *filt
         return e;
     }
     HIP_TRY(bg::launch_lstm_gates(a, c.stream));
+    }
+    if (projected) {
+        HIP_TRY(bg::launch_lstm_project(a, c.stream));  // lstm.cpp:170-178
     }
     if (arch == AMD_GFX950) {
         HIP_TRY(hipMemcpyAsync(state, dState, stateB, hipMemcpyDeviceToHost, c.stream));

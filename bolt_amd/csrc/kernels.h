@@ -323,8 +323,13 @@ struct LstmArgs {
     float *out = nullptr;          // row m at out + m * out_stride
     uint32_t out_stride = 0;
     float forget_bias = 0, zoneout_cell = 0, zoneout_output = 0;
+    // projection (column != hdim): the gates leave their `column` activated values per row in act, and
+    // launch_lstm_project forms out / the hidden state from proj, fp32 [hdim / 32][column][32]
+    const float *proj = nullptr;
+    float *act = nullptr;          // [batch][column]
 };
 hipError_t launch_lstm_xh_quant(const LstmArgs &a, hipStream_t st);
 hipError_t launch_lstm_gates(const LstmArgs &a, hipStream_t st);
+hipError_t launch_lstm_project(const LstmArgs &a, hipStream_t st);
 
 }  // namespace bg

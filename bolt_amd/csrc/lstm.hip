@@ -2,6 +2,7 @@
 //   lstm_xh_quant_kernel   per batch row: [x | h] gathered, its own dynamic (or the caller's static) scale,
 //                          fp32 -> u8 with the quantiser's arithmetic (lstm.cpp:89-109)
 //   lstm_gates_kernel      bias add, gates, cell / hidden state update with zoneout (lstm.cpp:113-176)
+//   lstm_project_kernel    with num_projection > 0: hidden state = fp32 projection of the gates' values (lstm.cpp:170-178)
 // The matrix-vector products in between are one launch of gemv_s8u8_kernel over all rows.
 #include "kernels.h"
 
@@ -86,11 +87,41 @@ __global__ __launch_bounds__(256) void lstm_gates_kernel(const LstmArgs a)
     } else {
         stC[h] = c1;
     }
+    if (a.proj) {
+        a.act[(size_t)m * a.column + h] = hid;  // the projection kernel takes it from here (lstm.cpp:128)
+        return;
+    }
     a.out[(size_t)m * a.out_stride + h] = hid;
     if (a.zoneout_output != 0) {
         stH[h] = hid * (1 - a.zoneout_output) + stH[h] * a.zoneout_output;
     } else {
         stH[h] = hid;
+    }
+}
+
+// mvm_nkn32_with_bias(hDim / 32, num_projection, filter[1], actOutH, projOut, nullptr) (lstm.cpp:170-173;
+// cpu/x86/fp32/mvm_nkn32.h:19-140): every output element is one chain of fused multiply-adds over k ascending from an
+// accumulator of 0 -- one thread per element here, in that order, so the sums round as the reference's do. Then the
+// hidden state follows the projected value (zoneout on the output, :175-178).
+__global__ __launch_bounds__(256) void lstm_project_kernel(const LstmArgs a)
+{
+    const uint32_t h = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t m = blockIdx.y;
+    if (h >= a.hdim) {
+        return;
+    }
+    const float *w = a.proj + (size_t)(h / 32) * a.column * 32 + (h % 32);
+    const float *v = a.act + (size_t)m * a.column;
+    float acc = 0.0f;
+    for (uint32_t k = 0; k < a.column; ++k) {
+        acc = __builtin_fmaf(v[k], w[(size_t)k * 32], acc);
+    }
+    a.out[(size_t)m * a.out_stride + h] = acc;
+    float *stH = a.state + (size_t)m * (a.column + a.hdim) + a.column;
+    if (a.zoneout_output != 0) {
+        stH[h] = acc * (1 - a.zoneout_output) + stH[h] * a.zoneout_output;
+    } else {
+        stH[h] = acc;
     }
 }
 
@@ -103,6 +134,12 @@ hipError_t launch_lstm_xh_quant(const LstmArgs &a, hipStream_t st)
 hipError_t launch_lstm_gates(const LstmArgs &a, hipStream_t st)
 {
     hipLaunchKernelGGL(lstm_gates_kernel, dim3((a.column + 255) / 256, a.batch), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_lstm_project(const LstmArgs &a, hipStream_t st)
+{
+    hipLaunchKernelGGL(lstm_project_kernel, dim3((a.hdim + 255) / 256, a.batch), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 

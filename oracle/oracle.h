@@ -125,6 +125,9 @@ void orc_concat_i8(uint32_t num, const int8_t *const *in, const uint32_t *len, c
     int8_t *out, float *oscale);
 
 /* ---- int8 LSTM cell ---------------------------------------------------------------- */
+void orc_lstmcell_int8_proj(uint32_t batch, uint32_t xdim, uint32_t hdim, uint32_t column, const float *x, uint32_t x_stride,
+    const int8_t *W, const float *Wp, const float *bias, uint32_t bias_stride, const float *scale, float *state,
+    float forget_bias, float zoneout_cell, float zoneout_output, float *out, uint32_t out_stride);
 void orc_lstmcell_int8(uint32_t batch, uint32_t xdim, uint32_t hdim, const float *x, uint32_t x_stride,
     const int8_t *W, const float *bias, uint32_t bias_stride, const float *scale, float *state, float forget_bias,
     float zoneout_cell, float zoneout_output, float *out, uint32_t out_stride);

@@ -8,6 +8,7 @@
 // Each wrapper builds the TensorDesc arguments exactly as the reference's own unit tests do
 // (compute/blas_enhance/tests/test_mmm.cpp:30-90, test_mvm.cpp:30-90) and forwards to the
 // public function; no arithmetic happens here.
+#include <omp.h>
 #include <cstdint>
 #include <cstring>
 #include "blas_enhance.h"
@@ -202,6 +203,51 @@ int ref_conv_int8(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 fw
     return e;
 }
 
+// The same convolution timed for a CPU baseline: filter transform and buffers once, then `reps` calls of
+// convolution_int8 between two clock readings (scale[1] is reset to -1 before each call: dynamic output scale).
+// *seconds receives the time of the calls alone.
+int ref_conv_int8_loop(U32 n, U32 ic, U32 ih, U32 iw, int idf, U32 oc, U32 fh, U32 fw, U32 sh, U32 sw, U32 pt, U32 pb,
+    U32 pl, U32 pr, U32 oh, U32 ow, int alg, const uint8_t *in, const int8_t *filter, const float *bias, float *scale,
+    int relu, int odt, void *out, int reps, double *seconds)
+{
+    ConvolutionParamSpec p = createConvolutionParamSpec(
+        1, 1, fh, fw, 1, sh, sw, 0, 0, pt, pb, pl, pr, 1, 1, 1, oc, CONVOLUTION_DEPTHWISE_POINTWISE);
+    ConvolutionForwardAlgorithm a = (ConvolutionForwardAlgorithm)alg;
+    TensorDesc inputDesc = tensor4df(DT_U8_Q, (DataFormat)idf, n, ic, ih, iw);
+    TensorDesc filterDesc = tensor4df(DT_I8, DF_NCHW, oc, ic, fh, fw);
+    TensorDesc biasDesc = tensor1d(DT_F32, oc);
+    TensorDesc outputDesc = tensor4df((DataType)odt, DF_NCHWC16, n, oc, oh, ow);
+    U32 fcPad = (ic + 15) / 16 * 16;
+    U32 ftmBytes = oc * fcPad * fh * fw + oc * 4 + 32;
+    INT8 *ftm = (INT8 *)calloc(ftmBytes + 64, 1);
+    TensorDesc ftmDesc;
+    EE e = convolution_transform_filter_int8(filterDesc, filter, p, a, &ftmDesc, ftm);
+    U32 tmpBytes = 0;
+    if (e == SUCCESS) {
+        e = convolution_infer_forward_tmp_bytes_int8(inputDesc, ftmDesc, outputDesc, p, a, &tmpBytes);
+    }
+    if (e != SUCCESS) {
+        free(ftm);
+        return 1000 + e;
+    }
+    void *tmp = calloc((size_t)tmpBytes + (size_t)n * oc * oh * ow * 4 + 4096, 1);
+    ActivationParamSpec act;
+    act.mode = relu ? ACTIVATION_RELU : ACTIVATION_NULL;
+    const float sI = scale[0], sF = scale[2];
+    const double t0 = omp_get_wtime();
+    for (int r = 0; r < reps && e == SUCCESS; ++r) {
+        scale[0] = sI;
+        scale[1] = -1;
+        scale[2] = sF;
+        e = convolution_int8(inputDesc, (UINT8 *)in, nullptr, ftmDesc, ftm, p, a, biasDesc, bias, tmpBytes, tmp, outputDesc, out,
+            scale, act, X86_AVX512);
+    }
+    *seconds = omp_get_wtime() - t0;
+    free(tmp);
+    free(ftm);
+    return e;
+}
+
 // u8 pooling on NCHWC16 (compute/tensor/src/cpu/x86/int8/avx512/pooling_int8.cpp:316). scale[2] = {in, out}.
 int ref_pooling_u8(U32 n, U32 c, U32 ih, U32 iw, U32 oh, U32 ow, U32 kh, U32 kw, U32 sh, U32 sw, U32 pt, U32 pl,
     int mean, int count_include_pad, const uint8_t *in, uint8_t *out, float *scale)
@@ -244,10 +290,13 @@ int ref_concat_i8(U32 num, const U32 *dims4 /* num x {n,c,h,w} */, int df, int a
 
 // int8 LSTM cell (compute/tensor/src/cpu/x86/int8/lstm.cpp:20). W: s8 [4*hdim][xdim+hdim] row-major, packed here
 // with the reference's own matrix_vector_multiply_transform_weight. state rows [C | H]; scale = {activation, weight}.
-int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_stride, const int8_t *W, const float *bias,
-    float *scale, float *state, float forget_bias, float zoneout_cell, float zoneout_output, float *out, U32 out_stride)
+// column = hdim and Wp = nullptr: no projection; else column = num_projection, W is [4 * column][K] and Wp the fp32
+// projection matrix in the DF_NKN32 layout the cell reads it in, [hdim / 32][column][32] (lstm.cpp:170-173)
+int ref_lstmcell_int8_proj(U32 batch, U32 xdim, U32 hdim, U32 column, const float *x, U32 x_stride, const int8_t *W,
+    const float *Wp, const float *bias, float *scale, float *state, float forget_bias, float zoneout_cell,
+    float zoneout_output, float *out, U32 out_stride)
 {
-    const U32 N = 4 * hdim, K = xdim + hdim;
+    const U32 N = 4 * column, K = xdim + hdim;
     TensorDesc wDesc = tensor2df(DT_I8, DF_NORMAL, N, K);
     U32 bytes = 0;
     EE e = matrix_vector_multiply_transform_weight_bytes(wDesc, &bytes, X86_AVX512);
@@ -266,7 +315,7 @@ int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_strid
     p.mode = RNN_LSTM;
     p.num_outputs = hdim;
     p.steps = -1;
-    p.num_projection = 0;
+    p.num_projection = Wp ? column : 0;
     p.zoneout_cell = zoneout_cell;
     p.zoneout_output = zoneout_output;
     p.bi_direction = false;
@@ -276,7 +325,7 @@ int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_strid
     TensorDesc hDesc = tensor2df(DT_F32, DF_NORMAL, batch, hdim);
     TensorDesc fDesc = tensor2df(DT_I8, DF_NKN32, N, K);
     TensorDesc bDesc = tensor1d(DT_F32, N);
-    const void *filters[2] = {blob, nullptr};
+    const void *filters[2] = {blob, Wp};
     const void *biases[2] = {bias, nullptr};
     U32 tmpBytes = (K + N) * 4 + K + 256;
     void *tmp = calloc(tmpBytes, 1);
@@ -286,6 +335,13 @@ int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_strid
     free(tmp);
     free(blob);
     return e;
+}
+
+int ref_lstmcell_int8(U32 batch, U32 xdim, U32 hdim, const float *x, U32 x_stride, const int8_t *W, const float *bias,
+    float *scale, float *state, float forget_bias, float zoneout_cell, float zoneout_output, float *out, U32 out_stride)
+{
+    return ref_lstmcell_int8_proj(batch, xdim, hdim, hdim, x, x_stride, W, nullptr, bias, scale, state, forget_bias,
+        zoneout_cell, zoneout_output, out, out_stride);
 }
 
 }  // extern "C"

@@ -8,8 +8,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 from bolt_amd import capi, host_lstm  # noqa: E402
-from checkers_lstm import lstm_case, orc_lstmcell  # noqa: E402
-from test_oracle_lstm import CASES, W_SCALE  # noqa: E402
+from checkers_lstm import lstm_case, lstm_proj_case, nkn32, orc_lstmcell, orc_lstmcell_proj  # noqa: E402
+from test_oracle_lstm import CASES, PROJ_CASES, W_SCALE  # noqa: E402
 
 TOL = 2e-6
 
@@ -168,3 +168,32 @@ def test_lstmcell_gemm_route_decode_shape(torch_mod):
         capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
         outs.append((out, st))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+@pytest.mark.parametrize("both_packings", [False, True])
+@pytest.mark.parametrize("case", PROJ_CASES + [(6, 64, 128, 256, 1.0, 0.0, 0.1)])
+def test_lstmcell_projection_vs_oracle(torch_mod, oracle, case, device_mode, both_packings):
+    """num_projection > 0 (lstm.cpp:60-62, 128, 165-178): the cell's `column` activated values per row go through the
+    fp32 projection matrix (DF_NKN32) to give the output and the hidden state. The projection is one chain of fused
+    multiply-adds per element in the reference's order, so it adds nothing to the gates' tolerance. Both weight routes
+    (batched GEMV, and the GEMM packing from 4 rows on)."""
+    print("lstm projection", case, device_mode, both_packings, flush=True)
+    torch = torch_mod
+    batch, xdim, hdim, column, fb, zc, zo = case
+    x, W, Wp, bias, state = lstm_proj_case(batch, xdim, hdim, column, 31)
+    want, wst = orc_lstmcell_proj(oracle, x, W, Wp, bias, [-1.0, W_SCALE], state, hdim, column, fb, zc, zo)
+    put = (lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()) if device_mode else np.ascontiguousarray
+    st = put(np.array(state, copy=True))
+    out = put(np.zeros((batch, hdim), np.float32))
+    p = host_lstm.lstm_param_spec(hdim, fb, zc, zo, num_projection=column)
+    if both_packings:
+        blob = host_lstm.rnn_transform_filter(put(W), 4 * column, xdim + hdim, p)
+    else:
+        blob = host_lstm.transform_weight(put(W), 4 * column, xdim + hdim)
+    host_lstm.lstmcell(put(x), blob, put(bias), [-1.0, W_SCALE], st, p, batch, xdim, out, both_packings=both_packings, proj=put(nkn32(Wp)))
+    if device_mode:
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        out, st = out.cpu().numpy(), st.cpu().numpy()
+    assert np.abs(out - want).max() <= TOL and np.abs(st - wst).max() <= TOL
+    assert np.abs(want).max() > 0.05

@@ -112,3 +112,31 @@ def test_ws_converter_rejects(torch_mod):
     assert L.ws_datatype_converter_int4_gfx950(w.ctypes.data, q.ctypes.data, 9, s, capi.AMD_GFX950) == capi.NOT_SUPPORTED
     assert L.ws_datatype_converter_bnn_gfx950(w.ctypes.data, q.ctypes.data, 9, s, capi.AMD_GFX950) == capi.NOT_MATCH
     assert L.ws_datatype_converter_int8_gfx950(None, q.ctypes.data, 9, s, capi.AMD_GFX950) == capi.NULL_POINTER
+
+
+@pytest.mark.parametrize("device_mode", [False, True])
+def test_stored_weights_next_to_the_model_loader(torch_mod, device_mode):
+    """A weight as a quantised .bolt model stores it (int8 bytes, or two int4 values per byte, with its one scale), expanded
+    by the reference's compiled model loader (TransWeightFromI8ToF32 / I4ToF32 / I4ToI8 / I4ToU8,
+    common/model_spec/src/model_deserialize.cpp:270-331) and by this library's load-time expanders, side by side: the same
+    bytes. Needs oracle/_ref on the box (built where the reference checkout is present)."""
+    from checkers import Ref
+    if not Ref.available():
+        pytest.skip("oracle/_ref not built or host lacks avx512_vnni")
+    ref = Ref(threads=1)
+    L = ref.lib.ref_loader_expand_weight
+    L.argtypes, L.restype = [C.c_int, vp, C.c_uint, vp, vp], C.c_uint
+    n = 3072 * 768
+    rng = np.random.default_rng(9)
+    q8 = rng.integers(-127, 128, size=n, dtype=np.int8)
+    nib = rng.integers(0, 15, size=n, dtype=np.uint8)
+    q4 = (nib[0::2] | (nib[1::2] << 4)).astype(np.uint8).view(np.int8)
+    for kind, stored, out_dt, name, scaled in ((0, q8, F, "dequantize_int8_weight_gfx950", True),
+                                               (1, q4, F, "dequantize_int4_weight_gfx950", True),
+                                               (2, q4, np.int8, "dequantize_int4_int8_gfx950", False),
+                                               (3, q4, np.uint8, "dequantize_int4_u8_q_gfx950", False)):
+        sc = np.array([51.75], F)
+        want = np.zeros(n, out_dt)
+        assert L(kind, _p(stored), stored.nbytes, _p(sc), _p(want)) == want.nbytes
+        got = expand(torch_mod, device_mode, name, n, stored, out_dt, F(51.75) if scaled else None)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name

@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 
 from checkers import DT_U8_Q
-from checkers_lstm import lstm_case, orc_lstmcell, ref_lstmcell
+from checkers_lstm import (lstm_case, lstm_proj_case, orc_lstmcell, orc_lstmcell_proj, ref_lstmcell, ref_lstmcell_proj)
 
 W_SCALE = np.float32(1.0) / np.float32(0.004)
 
@@ -67,3 +67,45 @@ def test_lstmcell_oracle_vs_float64_numpy(oracle):
         assert np.abs(got[m] - hid).max() <= 3e-6
         assert np.abs(gst[m, :hdim] - (c1 * 0.85 + c0 * 0.15)).max() <= 3e-6
         assert np.abs(gst[m, hdim:] - (hid * 0.65 + state[m, hdim:] * 0.35)).max() <= 3e-6
+
+
+PROJ_CASES = [  # batch, xdim, hdim (num_outputs), column (num_projection), forget_bias, zoneout_cell, zoneout_output
+    (2, 24, 32, 64, 1.0, 0.0, 0.0),
+    (3, 40, 64, 32, 0.0, 0.0, 0.0),
+    (2, 16, 32, 96, 1.0, 0.2, 0.0),
+    (2, 16, 64, 48, 0.5, 0.1, 0.3),
+]
+
+
+@pytest.mark.parametrize("case", PROJ_CASES)
+def test_lstmcell_projection_oracle_vs_reference(oracle, ref, case):
+    """num_projection > 0 (lstm.cpp:60-62, 128, 165-173): the gates give `column` values per row, the hidden state and
+    the output are the fp32 projection of those, and the zoneout of the output acts on the projected values. Against the
+    reference's compiled cell to 6e-4 (the gates' own tolerance; the projection adds sums of at most 96 products of
+    values below 1): a wrong layout of the projection matrix, state offset or order of projection and zoneout shows as
+    an error of 1e-1."""
+    batch, xdim, hdim, column, fb, zc, zo = case
+    x, W, Wp, bias, state = lstm_proj_case(batch, xdim, hdim, column, 23)
+    want, wst = ref_lstmcell_proj(ref, x, W, Wp, bias, [-1.0, W_SCALE], state, hdim, column, fb, zc, zo)
+    got, gst = orc_lstmcell_proj(oracle, x, W, Wp, bias, [-1.0, W_SCALE], state, hdim, column, fb, zc, zo)
+    assert np.abs(got - want).max() <= 6e-4 and np.abs(gst - wst).max() <= 6e-4
+    assert np.abs(want).max() > 0.05
+
+
+def test_lstmcell_projection_oracle_vs_float64_numpy(oracle):
+    batch, xdim, hdim, column = 2, 20, 32, 40
+    x, W, Wp, bias, state = lstm_proj_case(batch, xdim, hdim, column, 3)
+    got, gst = orc_lstmcell_proj(oracle, x, W, Wp, bias, [-1.0, W_SCALE], state, hdim, column, 1.0, 0.15, 0.35)
+    for m in range(batch):
+        xh = np.concatenate([x[m], state[m, column:]])
+        q, s = oracle.quantize_f32(xh, DT_U8_Q)
+        acc = W.astype(np.int64) @ (q.astype(np.int64) - 128)
+        g = acc / (np.float64(s) * np.float64(W_SCALE)) + bias[m]
+        i, gg, f, o = (g[k * column:(k + 1) * column] for k in range(4))
+        sig = lambda v: 1 / (1 + np.exp(-v))  # noqa: E731
+        c0 = state[m, :column].astype(np.float64)
+        c1 = c0 * sig(f + 1.0) + sig(i) * np.tanh(gg)
+        hid = Wp.astype(np.float64) @ (sig(o) * np.tanh(c1))
+        assert np.abs(got[m] - hid).max() <= 5e-6
+        assert np.abs(gst[m, :column] - (c1 * 0.85 + c0 * 0.15)).max() <= 3e-6
+        assert np.abs(gst[m, column:] - (hid * 0.65 + state[m, column:] * 0.35)).max() <= 5e-6

@@ -108,6 +108,37 @@ def test_load_time_expansion(oracle, ref, n):
     assert np.array_equal(d4.view(np.int32), viaref.view(np.int32))
 
 
+@pytest.mark.parametrize("n", [16, 1000, 65536])
+def test_model_loader_expansion(oracle, ref, n):
+    """The model loader itself (common/model_spec/src/model_deserialize.cpp:270-331: TransWeightFromI8ToF32,
+    TransWeightFromI4ToF32 / ToI8 / ToU8, applied to a WeightSpec as the .bolt file stores it) against the oracle's four
+    expanders: the expanded bytes, the new bytes_of_weight (x 4, x 8, x 2, x 2) and what happens to the stored scale (an
+    fp32 result zeroes it). This also pins the int4 -> fp32 expansion, which the compiled reference instantiates only here."""
+    o = bind(oracle.lib, "orc_")
+    oracle.lib.orc_dequantize_int4_weight.argtypes = [C.c_int, C.c_float, vp, vp]
+    L = ref.lib.ref_loader_expand_weight
+    L.argtypes, L.restype = [C.c_int, vp, C.c_uint, vp, vp], C.c_uint
+    rng = np.random.default_rng(n + 1)
+    q8 = rng.integers(-127, 128, size=n, dtype=np.int8)
+    nib = rng.integers(0, 15, size=n, dtype=np.uint8)
+    q4 = (nib[0::2] | (nib[1::2] << 4)).astype(np.uint8).view(np.int8)
+    for kind, stored, out_dt, grow, zeroes in ((0, q8, F, 4, True), (1, q4, F, 8, True), (2, q4, np.int8, 2, False),
+                                               (3, q4, np.uint8, 2, False)):
+        sc = np.array([37.3], F)
+        got = np.zeros(n, out_dt)
+        nbytes = L(kind, _p(stored), stored.nbytes, _p(sc), _p(got))
+        assert nbytes == stored.nbytes * grow == got.nbytes
+        assert sc[0] == (0 if zeroes else F(37.3))
+        want = np.zeros(n, out_dt)
+        if kind == 0:
+            o["dequantize_int8_weight"](n, F(37.3), _p(stored), _p(want))
+        elif kind == 1:
+            oracle.lib.orc_dequantize_int4_weight(n, F(37.3), _p(stored), _p(want))
+        else:
+            o["dequantize_int4_int8" if kind == 2 else "dequantize_int4_u8q"](n, _p(stored), _p(want))
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), kind
+
+
 def test_operator_scales_rule():
     """bolt_gfx950_operator_scales (pure host logic) against the three rules of the engine's operator classes, each
     written out here from the header it comes from and evaluated case by case:
