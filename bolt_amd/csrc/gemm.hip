@@ -180,9 +180,18 @@ __device__ __forceinline__ void store_c16(V *p, V v)
     }
 }
 
-template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN>
+// per-column offsets a kernel formed ahead of its K loop (16 columns per lane: a wave tile of 64 columns), handed to the
+// epilogue BY VALUE: a pointer to a local array is kept in scratch memory by the compiler
+struct PreBase {
+    bool have = false;
+    uint32_t v[4][4];
+};
+
+// SYNC: the kernel's launches may carry a grid-wide agreement (GemmArgs::sync; the filter-panel convolution only) -- the
+// code for it, the parking of values when it is abandoned included, is left out of every other kernel
+template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN, bool SYNC = false>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, const uint32_t (*pre_base)[4] = nullptr)
+    uint32_t wave, uint32_t m0, uint32_t n0, const PreBase pre_base = PreBase())
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -194,11 +203,11 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     if (CONV && MODE == EPI_U8) {
         // tensor-wide dynamic requantisation (avx512/quantize.cpp:364-416 after the abs-max of :70-119)
         int mx = 0;
-        if (!a.sync.slots) {
+        if (!(SYNC && a.sync.slots)) {
             mx = ws_read_max(a.conv.absmax);
         }
         factor = (mx == 0) ? 1.0f : 127.0f / (float)mx;
-        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out && !a.sync.slots) {
+        if (blockIdx.x == 0 && threadIdx.x == 0 && a.conv.dscale_out && !(SYNC && a.sync.slots)) {
             *a.conv.dscale_out = conv_acc_scale(a.conv) * factor;
         }
     } else if (MODE == EPI_F32 || MODE == EPI_U8) {
@@ -231,7 +240,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 bi[y * 4 + c] = bip[nn[y * 4 + c]];
             }
         }
-        if (!pre_base) {
+        if (!pre_base.have) {
             column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, fold_scale, nn, flat);
         }
 #pragma unroll
@@ -240,7 +249,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const bool ok = FULL || (n + c < a.N);
-                base[y][c] = pre_base ? pre_base[y][c] : (ok ? flat[y * 4 + c] : 0u);
+                base[y][c] = pre_base.have ? pre_base.v[y % 4][c] : (ok ? flat[y * 4 + c] : 0u);
                 qs[y][c] = 1.0f;
                 bs[y][c] = 0.0f;
                 if ((MODE == EPI_F32_CH || MODE == EPI_U8_CH) && ok) {
@@ -266,7 +275,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
         }
     }
 
-    if (CONV && MODE == EPI_U8 && a.sync.slots) {
+    if (SYNC && CONV && MODE == EPI_U8 && a.sync.slots) {
         // one pass: the maximum is agreed on by all workgroups of the launch while the accumulators are still in
         // registers (smem: 18 ints of LDS that no wave of the workgroup is still reading tiles from)
         int lm = 0;
@@ -795,7 +804,7 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
 // and then, by conv.ch_out: stored as fp32; or quantised like a fp32 tensor (q_u8, avx512/quantize.cpp:150-155) with
 // the static scale epi.factor or the dynamic one 127 / max|f| from the scratch slots; or only max|f| folded into those
 // slots. With every sW[oc] equal, no bias and an fp32 result this is the reference's epilogue bit for bit.
-template <int WM, int WN, int TM, int TN>
+template <int WM, int WN, int TM, int TN, bool SYNC>
 __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
     uint32_t wave, uint32_t m0, uint32_t n0)
 {
@@ -835,7 +844,7 @@ __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[T
             cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
         }
     }
-    if (out == CONV_CH_U8 && a.sync.slots) {
+    if (SYNC && out == CONV_CH_U8 && a.sync.slots) {
         // ONE pass (filter-panel kernel, every workgroup resident): the fp32 values replace the accumulators in their
         // registers, the workgroups agree on max|f| (smem: 18 ints of LDS nobody reads tiles from), and each quantises
         // its own values. Should that agreement be abandoned: with no spill buffer (synchronous form) nothing is
@@ -989,9 +998,9 @@ __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[T
     }
 }
 
-template <int MODE, bool CONV, int WM, int WN, int TM, int TN>
+template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool SYNC = false>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, const uint32_t (*pre_base)[4] = nullptr)
+    uint32_t wave, uint32_t m0, uint32_t n0, const PreBase pre_base = PreBase())
 {
     const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
     const bool cin = !CONV && a.add_cin && MODE != EPI_U8 && MODE != EPI_U8_CH;
@@ -1019,30 +1028,30 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
         }
     }
     if (full && !cin) {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0>(a, acc, smem, lane, wave, m0, n0, pre_base);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 0, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
     } else if (full && MODE != EPI_U8 && MODE != EPI_U8_CH && !CONV) {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1>(a, acc, smem, lane, wave, m0, n0, pre_base);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, true, 1, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
     } else {
-        epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2>(a, acc, smem, lane, wave, m0, n0, pre_base);
+        epilogue_rows<MODE, CONV, WM, WN, TM, TN, false, 2, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
     }
 }
 
-template <int WM, int WN, int TM, int TN, bool CONV = false>
+template <int WM, int WN, int TM, int TN, bool CONV = false, bool SYNC = false>
 __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes, const uint32_t (*pre_base)[4] = nullptr)
+    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes, const PreBase pre_base = PreBase())
 {
     (void)lds_bytes;
     if (CONV) {
         if (a.epi.mode == EPI_I32) {
-            epilogue_mode<EPI_I32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
+            epilogue_mode<EPI_I32, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_U8) {
-            epilogue_mode<EPI_U8, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
+            epilogue_mode<EPI_U8, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_F32_CH) {
-            epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
+            epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_CONV_CH) {
-            epilogue_conv_ch<WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_conv_ch<WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0);
         } else {
-            epilogue_mode<EPI_F32, true, WM, WN, TM, TN>(a, acc, smem, lane, wave, m0, n0, pre_base);
+            epilogue_mode<EPI_F32, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         }
         return;
     }
@@ -2185,7 +2194,8 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
     // Formed ahead of the K loop, while the first loads are on their way, instead of on the critical path behind it.
     // All loads first, none behind a branch (columns past N read column N - 1 and are dropped; the vector that the
     // mode does not use is read from the other one's address), so that they are in flight together.
-    uint32_t pre_base[4][4];
+    PreBase pre_base;
+    pre_base.have = true;
     int32_t pb_c[4][4], pb_o[4][4];
     float pb_f[4][4];
     const bool fold = a.fold_bias != nullptr;
@@ -2212,7 +2222,7 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
                 const uint32_t n = y * 16 + 4 * g + c;
                 const float p_ = pb_f[y][c] * fold_scale_;  // as column_base() forms it
                 const int32_t o_ = fold ? (int32_t)(round((double)p_) + (double)pb_c[y][c]) : pb_o[y][c];
-                pre_base[y][c] = (n < a.N) ? (uint32_t)o_ - (uint32_t)pb_c[y][c] : 0u;
+                pre_base.v[y][c] = (n < a.N) ? (uint32_t)o_ - (uint32_t)pb_c[y][c] : 0u;
             }
         }
     };
@@ -2332,7 +2342,7 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
     } else {
         k_loop(std::false_type{});
     }
-    epilogue_panel<4, 1, TM, 4, true>(a, acc, (uint8_t *)sync_lds, lane, wave, m0, 0u, 0, pre_base);
+    epilogue_panel<4, 1, TM, 4, true, true>(a, acc, (uint8_t *)sync_lds, lane, wave, m0, 0u, 0, pre_base);
 }
 
 // Skinny kernel for few rows (FullyConnected at small batch: M <= 64 per block, any N, K % 64 == 0).
