@@ -180,18 +180,22 @@ __device__ __forceinline__ void store_c16(V *p, V v)
     }
 }
 
-// per-column offsets a kernel formed ahead of its K loop (16 columns per lane: a wave tile of 64 columns), handed to the
-// epilogue BY VALUE: a pointer to a local array is kept in scratch memory by the compiler
-struct PreBase {
-    bool have = false;
-    uint32_t v[4][4];
+// Per-column terms a kernel formed ahead of its K loop and parked in its LDS, one entry per column of the block tile
+// (the filter-panel convolution: 64 columns): the epilogue reads its 16 entries from there instead of loading the
+// vectors from memory and repeating the arithmetic in every lane. Handed over BY VALUE (a pointer to a struct is kept in
+// scratch memory by the compiler). base: offset - compensation with the bias folded in (column_base); qs / bs: the
+// per-channel form's reciprocal scale 1.0f / (sI * sW[n]) and bias (0 without one). Null: nothing was formed.
+struct ColTerms {
+    const uint32_t *base = nullptr;
+    const float *qs = nullptr;
+    const float *bs = nullptr;
 };
 
 // SYNC: the kernel's launches may carry a grid-wide agreement (GemmArgs::sync; the filter-panel convolution only) -- the
 // code for it, the parking of values when it is abandoned included, is left out of every other kernel
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool FULL, int CIN, bool SYNC = false>
 __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, const PreBase pre_base = PreBase())
+    uint32_t wave, uint32_t m0, uint32_t n0, const ColTerms pre_base = ColTerms())
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -240,7 +244,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
                 bi[y * 4 + c] = bip[nn[y * 4 + c]];
             }
         }
-        if (!pre_base.have) {
+        if (!pre_base.base) {
             column_bases<TN * 4>(a.ob, a.comp, a.fold_bias, fold_scale, nn, flat);
         }
 #pragma unroll
@@ -249,7 +253,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const bool ok = FULL || (n + c < a.N);
-                base[y][c] = pre_base.have ? pre_base.v[y % 4][c] : (ok ? flat[y * 4 + c] : 0u);
+                base[y][c] = pre_base.base ? pre_base.base[(wn * TN + y) * 16 + 4 * g + c] : (ok ? flat[y * 4 + c] : 0u);
                 qs[y][c] = 1.0f;
                 bs[y][c] = 0.0f;
                 if ((MODE == EPI_F32_CH || MODE == EPI_U8_CH) && ok) {
@@ -806,7 +810,7 @@ __device__ __forceinline__ void epilogue_gelu_sync(const GemmArgs &a, v4i (&acc)
 // slots. With every sW[oc] equal, no bias and an fp32 result this is the reference's epilogue bit for bit.
 template <int WM, int WN, int TM, int TN, bool SYNC>
 __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0)
+    uint32_t wave, uint32_t m0, uint32_t n0, const ColTerms ct = ColTerms())
 {
     const uint32_t i = lane & 15, g = lane >> 4;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -814,7 +818,25 @@ __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[T
     const int out = a.conv.ch_out;
     uint32_t base[TN][4], cblk_off[TN], cblk_w[TN];
     float qs[TN][4], bs[TN][4];
-    {
+    if (ct.qs) {
+        // formed once per workgroup ahead of the K loop (see ColTerms)
+#pragma unroll
+        for (int y = 0; y < TN; ++y) {
+            const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
+            const uint32_t at = (wn * TN + y) * 16 + 4 * g;
+            const v4i b4 = *(const v4i *)(ct.base + at);
+            const v4f q4 = *(const v4f *)(ct.qs + at), s4 = *(const v4f *)(ct.bs + at);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                base[y][c] = (uint32_t)b4[c];
+                qs[y][c] = q4[c];
+                bs[y][c] = s4[c];
+            }
+            const uint32_t xc = a.conv.out_c, blk = n / xc;
+            cblk_w[y] = (a.N - blk * xc < xc) ? a.N - blk * xc : xc;
+            cblk_off[y] = blk * xc * a.conv.OHW + (n % xc);
+        }
+    } else {
         // every per-column term in one batch of loads, none behind a branch; columns past N read column N - 1
         uint32_t nn[TN * 4], flat[TN * 4];
         float sw[TN * 4], bi[TN * 4];
@@ -1000,7 +1022,7 @@ __device__ __forceinline__ void epilogue_conv_ch(const GemmArgs &a, v4i (&acc)[T
 
 template <int MODE, bool CONV, int WM, int WN, int TM, int TN, bool SYNC = false>
 __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, const PreBase pre_base = PreBase())
+    uint32_t wave, uint32_t m0, uint32_t n0, const ColTerms pre_base = ColTerms())
 {
     const bool full = (m0 + WM * TM * 16 <= a.M) && (n0 + WN * TN * 16 <= a.N) && (CONV || (a.N & 3) == 0);
     const bool cin = !CONV && a.add_cin && MODE != EPI_U8 && MODE != EPI_U8_CH;
@@ -1038,7 +1060,7 @@ __device__ __forceinline__ void epilogue_mode(const GemmArgs &a, v4i (&acc)[TM][
 
 template <int WM, int WN, int TM, int TN, bool CONV = false, bool SYNC = false>
 __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM][TN], uint8_t *smem, uint32_t lane,
-    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes, const PreBase pre_base = PreBase())
+    uint32_t wave, uint32_t m0, uint32_t n0, int lds_bytes, const ColTerms pre_base = ColTerms())
 {
     (void)lds_bytes;
     if (CONV) {
@@ -1049,7 +1071,7 @@ __device__ __forceinline__ void epilogue_panel(const GemmArgs &a, v4i (&acc)[TM]
         } else if (a.epi.mode == EPI_F32_CH) {
             epilogue_mode<EPI_F32_CH, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else if (a.epi.mode == EPI_CONV_CH) {
-            epilogue_conv_ch<WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0);
+            epilogue_conv_ch<WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         } else {
             epilogue_mode<EPI_F32, true, WM, WN, TM, TN, SYNC>(a, acc, smem, lane, wave, m0, n0, pre_base);
         }
@@ -2190,42 +2212,36 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
         }
     };
 
-    // ---- per-column terms of the epilogue (offsetC - compensation, with the bias folded in) -------------------
-    // Formed ahead of the K loop, while the first loads are on their way, instead of on the critical path behind it.
-    // All loads first, none behind a branch (columns past N read column N - 1 and are dropped; the vector that the
-    // mode does not use is read from the other one's address), so that they are in flight together.
-    PreBase pre_base;
-    pre_base.have = true;
-    int32_t pb_c[4][4], pb_o[4][4];
-    float pb_f[4][4];
-    const bool fold = a.fold_bias != nullptr;
-    auto pre_base_request = [&]() {
-        const int32_t *obp = fold ? a.comp : a.ob;
-        const float *fbp = fold ? a.fold_bias : (const float *)a.comp;
-#pragma unroll
-        for (int y = 0; y < 4; ++y) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t n = y * 16 + 4 * g + c, nc = n < a.N ? n : a.N - 1;
-                pb_c[y][c] = a.comp[nc];
-                pb_o[y][c] = obp[nc];
-                pb_f[y][c] = fbp[nc];
+    // ---- per-column terms of the epilogue ------------------------------------------------------------------------
+    // offsetC - compensation with the bias folded in (column_base's arithmetic) and, for per-channel filter scales, the
+    // reciprocal scale and the bias of each of the (at most 64) output channels: formed ONCE per workgroup by its first
+    // 64 threads, while the filter panel and the first tiles are on their way, and parked in LDS; the barrier in front
+    // of the K loop publishes them. The epilogue then reads its 16 entries per lane from there -- no loads from memory
+    // and no double-precision rounding or division on the critical path behind the K loop, and no registers held
+    // across it.
+    __shared__ __attribute__((aligned(16))) uint32_t col_base[64];
+    __shared__ __attribute__((aligned(16))) float col_qs[64], col_bs[64];
+    auto column_terms = [&]() {
+        if (threadIdx.x < 64) {
+            const uint32_t n = threadIdx.x, nc = n < a.N ? n : a.N - 1;
+            const float fold_scale_ = a.conv.dscaleI ? conv_acc_scale(a.conv) : a.fold_scale;
+            col_base[n] = (n < a.N) ? column_base(a.ob, a.comp, a.fold_bias, fold_scale_, nc) : 0u;
+            float q_ = 1.0f, b_ = 0.0f;
+            if (a.epi.mode == EPI_CONV_CH) {
+                const float sI_ = a.conv.dscaleI ? *a.conv.dscaleI : a.conv.scaleI;
+                q_ = 1.0f / (sI_ * a.epi.scaleW[nc]);
+                b_ = a.epi.bias ? a.epi.bias[nc] : 0.0f;
             }
+            col_qs[n] = q_;
+            col_bs[n] = b_;
         }
     };
-    auto pre_base_form = [&]() {
-        const float fold_scale_ = a.conv.dscaleI ? conv_acc_scale(a.conv) : a.fold_scale;
-#pragma unroll
-        for (int y = 0; y < 4; ++y) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t n = y * 16 + 4 * g + c;
-                const float p_ = pb_f[y][c] * fold_scale_;  // as column_base() forms it
-                const int32_t o_ = fold ? (int32_t)(round((double)p_) + (double)pb_c[y][c]) : pb_o[y][c];
-                pre_base.v[y][c] = (n < a.N) ? (uint32_t)o_ - (uint32_t)pb_c[y][c] : 0u;
-            }
-        }
-    };
+    ColTerms pre_base;
+    pre_base.base = col_base;
+    if (a.epi.mode == EPI_CONV_CH) {
+        pre_base.qs = col_qs;
+        pre_base.bs = col_bs;
+    }
 
     // this lane's K-group g covers 16-channel chunk 4 * tile + g; its (kh, kw, c16) is stepped in registers
     uint32_t c16 = g % cpc, kw = (g / cpc) % a.conv.fw, kh = (g / cpc) / a.conv.fw, at = 0;  // at: tile the walk points to
@@ -2288,9 +2304,8 @@ __global__ __launch_bounds__(256, 2) void conv_u8s8_panel_kernel(GemmArgs a)
         // all of it is on its way
         pixel_terms();
         first_tiles();
-        pre_base_request();
-        pre_base_form();
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the panel (and the first A tiles) have landed
+        column_terms();
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) lgkmcnt(0): the panel (and the first A tiles) have landed, the column terms are written
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
