@@ -237,8 +237,10 @@ def other_kernels(L, capi, host, torch, dev, only=None):
     if want("gemm"):
         from bolt_amd.capi import AMD_GFX950_DEVICE, DT_I8, tensor1d
         gemm = []
-        for (M, K, N, reps) in ((2048, 2048, 2048, 50), (4096, 4096, 4096, 30), (8192, 8192, 8192, 10), (4096, 768, 768, 50),
-                                (4096, 768, 3072, 50), (4096, 3072, 768, 50)):
+        # 8192^3: 30 untimed calls first and 20 timed ones -- the clock the device holds under this load takes ~10 ms to
+        # settle, and a figure taken from a cold start reads up to 20 % off in either direction
+        for (M, K, N, reps, warm) in ((2048, 2048, 2048, 50, 3), (4096, 4096, 4096, 30, 10), (8192, 8192, 8192, 20, 30),
+                                      (4096, 768, 768, 50, 3), (4096, 768, 3072, 50, 3), (4096, 3072, 768, 50, 3)):
             A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g)
             W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
             blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
@@ -256,7 +258,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                 Cb = torch.zeros((M, N), dtype=tdt, device=dev)
                 cd = tensor2df(cdt, DF_NORMAL, M, N)
                 add("matrix_matrix_multiply", nm,
-                    timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps))
+                    timed(lambda: capi.check(host.matrix_matrix_multiply(A, ad, blob, bd, off, Cb, cd, sc), "mmm"), reps, warm))
                 del Cb
             for odt, tdt, so0, nm in ((DT_F32, torch.float32, -1.0, "f32"), (DT_U8_Q, torch.uint8, 0.05, "u8_static_scale")):
                 nbytes = host.fully_connected_tmp_bytes(M, K, N, DF_NKNxKx, odt, AMD_GFX950_DEVICE)
@@ -268,7 +270,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                     timed(lambda: capi.check(L.fully_connected_gfx950(ad, host.ptr(A), 30.0, fdesc, host.ptr(blob), 100.0,
                                                                       tensor1d(DT_F32, N), host.ptr(bias), nbytes, host.ptr(tmp),
                                                                       od, host.ptr(out), C.byref(so), AMD_GFX950_DEVICE),
-                                             "fully_connected"), reps))
+                                             "fully_connected"), reps, warm))
                 del tmp, out
             del A, W, blob
         res["gemm_int8"] = gemm
@@ -345,6 +347,29 @@ def other_kernels(L, capi, host, torch, dev, only=None):
         rate["note"] = ("v_mfma_i32_16x16x64_i8 back to back from registers, 8 waves per CU, no memory traffic: the device "
                         "lowers its clock when the operand bits are random")
         res["gemm_int8_8192_by_operand_data"] = by_data
+        # the vendor library's int8 product on the same box and operand bits, as a yardstick only (int32 result, no
+        # epilogue; torch routes _int_mm to the ROCm BLAS libraries): not a kernel of this library
+        try:
+            M = K = N = 8192
+            va = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+            vb = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
+            for _ in range(30):
+                torch._int_mm(va, vb.t())
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                torch._int_mm(va, vb.t())
+            e1.record()
+            torch.cuda.synchronize()
+            tv = e0.elapsed_time(e1) / 20
+            res["vendor_int8_gemm_8192"] = {"ms": tv, "tops": 2.0 * M * N * K / tv / 1e9,
+                                            "frac_mfma_peak": 2.0 * M * N * K / tv / 1e9 / MFMA_PEAK_TOPS,
+                                            "note": "torch._int_mm(A, B.t()) s8 x s8 -> int32, uniform random bytes, 30 untimed "
+                                                    "calls first: the ROCm BLAS library's kernel, for comparison only"}
+            del va, vb
+        except Exception as ex:                                   # a build of torch without the int8 product
+            res["vendor_int8_gemm_8192"] = {"error": repr(ex)[:200]}
         res["mfma_int8_sustained"] = rate
     # -- C1: FullyConnected M=64 K=1024 N=1024, fp32 out
     if want("fc"):

@@ -282,21 +282,23 @@ __device__ __forceinline__ void epilogue_rows(const GemmArgs &a, v4i (&acc)[TM][
     if (SYNC && CONV && MODE == EPI_U8 && a.sync.slots) {
         // one pass: the maximum is agreed on by all workgroups of the launch while the accumulators are still in
         // registers (smem: 18 ints of LDS that no wave of the workgroup is still reading tiles from)
+        // The column terms and the ReLU go into the accumulators in place, and the terms are zeroed for the code
+        // behind: held beside the accumulators across the exchange, the sums cost 64 more registers than there are.
         int lm = 0;
 #pragma unroll
         for (int y = 0; y < TN; ++y) {
             const uint32_t n = n0 + (wn * TN + y) * 16 + 4 * g;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                if (n + c < a.N) {
 #pragma unroll
-                    for (int x = 0; x < TM; ++x) {
-                        int t = (int)((uint32_t)acc[x][y][c] + base[y][c]);
-                        t = (a.conv.relu && t < 0) ? 0 : t;
-                        const int av = (t == (int)0x80000000) ? t : (t < 0 ? -t : t);
-                        lm = av > lm ? av : lm;
-                    }
+                for (int x = 0; x < TM; ++x) {
+                    int t = (int)((uint32_t)acc[x][y][c] + base[y][c]);
+                    t = (a.conv.relu && t < 0) ? 0 : t;
+                    acc[x][y][c] = t;
+                    const int av = (t == (int)0x80000000) ? t : (t < 0 ? -t : t);
+                    lm = (n + c < a.N && m0 + (wm * TM + x) * 16 + i < a.M && av > lm) ? av : lm;
                 }
+                base[y][c] = 0u;
             }
         }
         const uint32_t outcome = grid_max_sync(a.sync, lm, (int *)smem);

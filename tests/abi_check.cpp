@@ -68,6 +68,31 @@ SAME(deconvolution_cpu, deconvolution_gfx950);
 SAME_PLUS_ARCH(depthwise_convolution_transform_filter_int8, depthwise_convolution_transform_filter_int8_gfx950);
 SAME_PLUS_ARCH(depthwise_pointwise_convolution_int8, depthwise_pointwise_convolution_int8_gfx950);
 
+SAME_PLUS_ARCH(pooling_x86, pooling_gfx950);                          // cpu/x86/tensor_computing_x86.h:191-197
+SAME(rnncell_x86, rnncell_gfx950);                                   // cpu/x86/tensor_computing_x86.h:166-181
+SAME(rnncell_infer_forward_tmp_bytes_cpu, rnncell_infer_forward_tmp_bytes_gfx950);
+
+// Twins that std::is_same cannot hold against a reference prototype, and why:
+//  * fully_connected_gfx950, fully_connected_infer_forward_tmp_bytes_gfx950, matmul_gfx950,
+//    matmul_infer_forward_tmp_bytes_gfx950: the reference has only the Tensor-class forms of these
+//    (tensor_computing.h); the x86 int8 branch inside them is not a function of its own. The C forms take the
+//    unwrapped descs, pointers and scales; include/bolt_gfx950_tensor.hpp puts the reference's Tensor argument
+//    lists back on top, and tests/glue_test.cpp compiles those against tensor_computing.h.
+//  * convolution_gfx950: convolution_x86 carries a scaleDesc and an untyped scale pointer between algorithm and
+//    biasDesc; the C form takes F32 *scale after output, const input pointers, and no scaleDesc.
+//  * convolution_infer_output_size_gfx950, convolution_infer_forward_algorithm_gfx950,
+//    deconvolution_infer_output_size_gfx950: the reference's forms take Tensor * / ArchInfo_t.
+//  * concat_gfx950, concat_infer_forward_tmp_bytes_gfx950: concat_cpu takes std::vector by value, which has no C form;
+//    the twin takes a count and two arrays.
+//  * rnn_transform_filter_gfx950, rnn_transform_filter_bytes_gfx950: the reference's forms take arrays of descs and
+//    pointers (the int8 weight and the fp32 projection together); the twin transforms the int8 weight alone.
+//  * convolution_*_bnn_gfx950: the reference's 1-bit convolution is declared in the ARM header
+//    (cpu/arm/tensor_computing_arm.h), which does not compile for x86.
+//  * ws_datatype_converter_*_gfx950, dequantize_int8_weight_gfx950, dequantize_int4_*_gfx950: the reference declares
+//    these in no header (model_data_type_converter.cpp, model_deserialize.cpp); oracle/ref_shim_ptq.cpp repeats their
+//    declarations and links them, so a changed argument list fails that link.
+//  * depthwise_convolution_transform_filter_bytes_int8_gfx950 and every bolt_gfx950_* entry point: no counterpart.
+
 // ---- plain-data types ---------------------------------------------------------------------------------------------
 #define SIZE(T) static_assert(sizeof(ours::T) == sizeof(::T), "sizeof " #T)
 #define FIELD(T, f) static_assert(offsetof(ours::T, f) == offsetof(::T, f), "offset of " #T "." #f)

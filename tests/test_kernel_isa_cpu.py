@@ -73,6 +73,14 @@ def test_no_scratch_in_any_loop_with_hand_counted_memory_operations(gemm_asm):
         assert rs[n]["NumVgprs"] + rs[n]["NumAgprs"] <= 256, n    # two waves per SIMD
         assert not [ins for ins in ks[n] if ins.startswith("scratch_")], n
     assert {3, 4} <= pipes, "the whole-line loops (PIPE 3 and 4) are missing: %s" % sorted(pipes)
+    # the convolution's filter-panel kernels keep 64 (TM = 4) accumulators in registers across a grid-wide exchange in
+    # their epilogue: spilled there, every launch writes and re-reads a tensor's worth of scratch (25 MB at 32 x 64 x 56
+    # x 56 -> 64 channels, seen as five times the result's bytes on the write counter)
+    panels = [n for n in rs if "conv_u8s8_panel_kernel" in n]
+    assert len(panels) == 4, sorted(panels)
+    for n in panels:
+        assert rs[n]["ScratchSize"] == 0, "%s: %d bytes of scratch per lane" % (n, rs[n]["ScratchSize"])
+        assert not [ins for ins in ks[n] if ins.startswith("scratch_")], n
 
 
 def test_no_spill_stores_inside_the_register_b_loop(gemm_asm):
