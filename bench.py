@@ -438,7 +438,7 @@ def other_kernels(L, capi, host, torch, dev, only=None):
                                                                  host.ptr(cb), ctmp.numel(), host.ptr(ctmp), odesc, host.ptr(cout), sc2, act,
                                                                  AMD_GFX950_DEVICE), "conv perchannel")
         entry("conv_c3_u8_perchannel", timed(perchannel_dynamic, 50), alg_bytes_u8 + 512,
-              "per-output-channel filter scales, dynamic output scale returned to the host (two passes of the convolution)")
+              "per-output-channel filter scales, dynamic output scale returned to the host (one pass; two when the grid-wide agreement is abandoned)")
         sc3 = (C.c_float * 2)(40.0, 2.5)
         t = timed(lambda: capi.check(L.bolt_gfx950_convolution_int8_perchannel(
             idesc, host.ptr(xq), None, ftm, host.ptr(cblob), p, host.ptr(sw), bdesc, host.ptr(cb), ctmp.numel(), host.ptr(ctmp), odesc,

@@ -429,8 +429,13 @@ EE concat_gfx950(U32 num, const TensorDesc *inputDesc, void *const *input, const
  *   tmp          rnncell_infer_forward_tmp_bytes_gfx950 bytes
  * Integer accumulators are exact; the gates use expf / tanhf where the reference's vector loop uses its
  * polynomial exp and its scalar tail uses double-precision libm: results agree to about 1e-6.
- * num_projection > 0 (an fp32 projection matrix), modes other than RNN_LSTM and activation types other
- * than ACTIVATION_TANH return NOT_SUPPORTED. */
+ * With num_projection > 0 (lstm.cpp:60-62, 128, 165-178) the gates produce num_projection values per row:
+ * filterDesc[0] is [4 * num_projection, xDim + num_outputs], the bias row 4 * num_projection floats, the state row
+ * [num_projection (C) | num_outputs (H)], and filter[1] is the fp32 projection matrix in the DF_NKN32 layout the
+ * reference reads, [num_outputs / 32][num_projection][32] (num_outputs % 32 == 0); the hidden state and the output are
+ * that matrix times the gates' values, every element one chain of fused multiply-adds over k ascending from 0
+ * (mvm_nkn32_with_bias, cpu/x86/fp32/mvm_nkn32.h:19-140).
+ * Modes other than RNN_LSTM and activation types other than ACTIVATION_TANH return NOT_SUPPORTED. */
 EE rnncell_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
     RNNParamSpec rnnParamSpec, U32 *bytes, Arch arch);
 /* rnn_transform_filter_bytes / rnn_transform_filter (compute/tensor/src/rnn.cpp:33-141) for the int8 LSTM weight:

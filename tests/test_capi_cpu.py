@@ -194,8 +194,16 @@ def test_pool_concat_lstm_argument_checks_and_size_queries():
                                                     AMD_GFX950) == capi.SUCCESS and nb.value >= 3 * (K + 4 + 4 * N)
     proj = lstm_param_spec(64)
     proj.num_projection = 32
-    assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, N, K), hd, proj, C.byref(nb),
-                                                    AMD_GFX950) == capi.NOT_SUPPORTED
+    plain = nb.value
+    # with a projection the gates give num_projection values per row: the weight is [4 * 32][32 + 64], and tmp also
+    # holds those values ahead of the fp32 projection
+    assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, 128, K), hd, proj, C.byref(nb),
+                                                    AMD_GFX950) == capi.SUCCESS and nb.value >= 3 * (K + 4 + 4 * 128 + 4 * 32)
+    assert nb.value != plain
+    odd = lstm_param_spec(48)                 # the projection matrix comes in blocks of 32 rows (DF_NKN32)
+    odd.num_projection = 32
+    assert L.rnncell_infer_forward_tmp_bytes_gfx950(xd, tensor2df(DT_I8, DF_NORMAL, 128, 80), tensor2df(DT_F32, DF_NORMAL, 3, 48),
+                                                    odd, C.byref(nb), AMD_GFX950) == capi.NOT_SUPPORTED
     assert C.sizeof(RNNParamSpec) == 36
 
 
