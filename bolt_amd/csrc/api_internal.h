@@ -59,7 +59,7 @@ EE fail(EE code, const char *what, hipError_t he = hipSuccess);  // records the 
 
 EE ensure_init();  // allocates the context's device state on first use; call before any launch
 
-// A scale that a kernel computes and the interface returns through a host pointer (see api.hip)
+// A scale that a kernel computes and the interface returns through a host pointer (api.hip)
 void arm_scale(Ctx &c);
 EE take_scale(Ctx &c, float *dst, bool *gave_up = nullptr);
 
@@ -95,9 +95,24 @@ struct Stage {
     }
 };
 
-EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w);
+// options behind bolt_gfx950_set_option (process-wide; api.hip explains each where it is defined)
+extern int g_bnn_mfma, g_conv_direct, g_conv_onepass, g_lstm_gemm_rows, g_quantize_fused, g_encoder_fused;
 
-// ---- int8 convolution core (api.hip), also the 1x1 product inside the deconvolution ---------------------------
+// descriptor helpers and the device-pointer cores of the two matrix products (api.hip)
+EE get2d(TensorDesc d, DataType *dt, DataFormat *df, U32 *rows, U32 *cols);
+EE get1d(TensorDesc d, DataType *dt, U32 *len);
+EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w);
+uint32_t f32_bits(float f);
+bool aligned4(const void *p);
+bg::Epilogue epi_from_scale(const F32 *scale);
+void pack_host(bool mmm, const INT8 *src, size_t sk, size_t sn, U32 K, U32 N, INT8 *dst, I32 *comp);
+U32 packed_matrix_bytes(U32 N, U32 K);  // bytes of the packed matrix part for an N x K weight
+EE mmm_device(U32 M, U32 N, U32 K, DataFormat adf, const void *A, DataFormat bdf, const void *B, void *tmp, DataType cdt, void *C,
+    const F32 *scale);
+EE mvm_device(U32 N, U32 K, DataType mdt, DataFormat mdf, const void *W, const void *x, void *tmp, void *y, const F32 *scale);
+U32 out_elem_bytes(const F32 *scale);
+
+// ---- int8 convolution core (api_conv.hip), also the 1x1 product inside the deconvolution ---------------------------
 struct ConvShape {
     U32 n, ic, ih, iw, oc, fh, fw, oh, ow;
     U32 sh, sw, pt, pb, pl, pr, dh, dw;

@@ -1,5 +1,5 @@
 // Launchers of the gfx950 kernels. Every pointer is a device pointer; launches are asynchronous on
-// the given stream. The C-ABI layer (api.hip) validates shapes before calling any of these.
+// the given stream. The C-ABI layer (api*.hip) validates shapes before calling any of these.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -10,7 +10,7 @@ namespace bg {
 // Every field of the argument structs below has a default (null / 0): a caller that leaves one out hands the
 // kernel a harmless value, never an indeterminate pointer.
 
-// ---- shared with the C-ABI layer (api.hip) ---------------------------------------------------------
+// ---- shared with the C-ABI layer (api*.hip) ---------------------------------------------------------
 hipStream_t api_stream();                              // the stream every call is enqueued on (null until set)
 void api_set_error(const char *what, hipError_t he);   // text behind bolt_gfx950_last_error()
 int noalloc_init_current_device();                     // noalloc.hip: looks up the static scratch array's device address
