@@ -314,3 +314,75 @@ def test_conv_one_pass_forms_when_their_wait_gives_up(torch_mod, oracle, co):
     final = C.c_ulonglong(0)
     capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(final)), "counter")
     assert final.value == after.value
+
+
+def test_conv_random_shapes_every_form(torch_mod, oracle, co):
+    """Twenty seeded random shapes (channels 8-144, filters 1-5, strides, paddings, ragged images) under random kernel
+    options, each through every form: the reference's three result types in both output layouts, the per-channel forms
+    (fp32, static u8, dynamic u8) and the asynchronous twins with and without room for the one-pass form -- all against
+    the CPU checker, bit for bit, scales included."""
+    torch = torch_mod
+    L = capi.lib()
+    rng = np.random.default_rng(20240607)
+    try:
+        for it in range(20):
+            n = int(rng.integers(1, 5))
+            ic = int(rng.choice([8, 16, 24, 32, 48, 64]))
+            oc = int(rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 96, 144]))
+            fh = fw = int(rng.choice([1, 2, 3, 5]))
+            stride = int(rng.choice([1, 1, 2]))
+            pad = int(rng.integers(0, (fh + 1) // 2 + 1))
+            ih = int(rng.integers(max(fh - 2 * pad, 1) + 1, 24))
+            iw = int(rng.integers(max(fw - 2 * pad, 1) + 1, 24))
+            case = (n, ic, ih, iw, oc, fh, fw, stride, pad)
+            relu = bool(rng.random() < 0.6)
+            panel, direct, onepass = int(rng.choice([0, 2, 4])), int(rng.choice([0, 1, 2])), int(rng.choice([0, 1]))
+            print("conv random", it, case, relu, panel, direct, onepass, flush=True)
+            capi.check(L.bolt_gfx950_set_option(b"conv_panel", panel), "set_option")
+            capi.check(L.bolt_gfx950_set_option(b"conv_direct", direct), "set_option")
+            capi.check(L.bolt_gfx950_set_option(b"conv_onepass", onepass), "set_option")
+            xq, sI, W, sF, bias = make_conv_case(oracle, n, ic, ih, iw, oc, fh, fw, 977 * it + 5)
+            sw = channel_scales(oc, it)
+            p = capi.conv_param_spec(oc, fh, fw, stride, pad)
+            blob, ftm = host_conv.transform_filter(put(torch, W), oc, ic, fh, fw, p)
+            for odf, out_c in ((DF_NCHWC16, 16), (DF_NCHWC8, 8)):
+                for odt in (DT_U8_Q, DT_F32, DT_I32):
+                    d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, relu, odt, out_c)
+                    want, ws = co.conv(d, xq, W, bias, [sI, -1.0, sF])
+                    sc = [sI, -1.0, sF]
+                    got = host_conv.convolution(put(torch, xq), DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad,
+                                                put(torch, bias), sc, relu, odt, odf)
+                    capi.check(L.bolt_gfx950_synchronize(), "sync")
+                    assert np.array_equal(np.array(sc, np.float32), ws), (case, odt, sc, ws)
+                    assert np.array_equal(got.cpu().numpy().view(np.uint8), want.view(np.uint8)), (case, odt, out_c)
+                d = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, relu, DT_F32, out_c)
+                want, _ = co.conv_perchannel(oracle, d, xq, W, sw, bias, sI)
+                got = run_perchannel(torch, True, xq, DF_NCHWC8, W, sw, bias, [sI, -1.0], case, relu, DT_F32, odf)
+                assert np.array_equal(got.view(np.int32), want.view(np.int32)), (case, out_c)
+                du = co.desc(n, ic, ih, iw, oc, fh, fw, stride, pad, relu, DT_U8_Q, out_c)
+                for so in (-1.0, 2.5):
+                    wq, ws = co.conv_perchannel(oracle, du, xq, W, sw, bias, sI, out_scale=so)
+                    sc = [sI, so]
+                    gq = run_perchannel(torch, True, xq, DF_NCHWC8, W, sw, bias, sc, case, relu, DT_U8_Q, odf)
+                    assert np.float32(sc[1]) == ws and np.array_equal(gq, wq), (case, so, out_c)
+                    for room in (True, False):
+                        dsi = torch.tensor([sI], dtype=torch.float32, device="cuda")
+                        dso = torch.zeros(1, dtype=torch.float32, device="cuda")
+                        ga = host_conv.convolution_async(put(torch, xq), DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride,
+                                                         pad, put(torch, bias), dsi, 0.0, put(torch, sw), dso, relu, DT_U8_Q, odf,
+                                                         static_out=(so if so > 0 else 0.0), one_pass_room=room)
+                        capi.check(L.bolt_gfx950_synchronize(), "sync")
+                        assert np.array_equal(ga.cpu().numpy(), wq) and np.float32(dso.item()) == ws, (case, so, out_c, room)
+                want, ws = co.conv(du, xq, W, bias, [sI, -1.0, sF])
+                for room in (True, False):
+                    dsi = torch.tensor([sI], dtype=torch.float32, device="cuda")
+                    dso = torch.zeros(1, dtype=torch.float32, device="cuda")
+                    ga = host_conv.convolution_async(put(torch, xq), DF_NCHWC8, n, ic, ih, iw, blob, ftm, oc, fh, fw, stride, pad,
+                                                     put(torch, bias), dsi, sF, None, dso, relu, DT_U8_Q, odf, one_pass_room=room)
+                    capi.check(L.bolt_gfx950_synchronize(), "sync")
+                    assert np.array_equal(ga.cpu().numpy().view(np.uint8), want.view(np.uint8)), (case, out_c, room)
+                    assert np.float32(dso.item()) == ws[1], (case, out_c, room)
+    finally:
+        capi.check(L.bolt_gfx950_set_option(b"conv_panel", 4), "set_option")
+        capi.check(L.bolt_gfx950_set_option(b"conv_direct", 1), "set_option")
+        capi.check(L.bolt_gfx950_set_option(b"conv_onepass", 1), "set_option")

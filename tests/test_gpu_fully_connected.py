@@ -80,3 +80,43 @@ def test_fully_connected_rejects_unquantised_input(torch_mod):
                                  capi.tensor1d(DT_F32, 4), None, 4096, host.ptr(tmp),
                                  capi.tensor2df(DT_F32, DF_NORMAL, 2, 4), host.ptr(out), C.byref(so), capi.AMD_GFX950)
     assert e == capi.NOT_MATCH   # x86 requires DT_U8_Q activations (fully_connected.cpp:395)
+
+
+def test_fully_connected_random_shapes(torch_mod, oracle):
+    """Forty seeded random shapes (one row = the matrix-vector route, a few rows, a few hundred; K and N ragged, multiples
+    of 8 and of 64) through every result type with and without a bias, against the CPU checker bit for bit."""
+    torch = torch_mod
+    rng = np.random.default_rng(20240608)
+
+    def put(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def get(t):
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        return t.cpu().numpy()
+    for it in range(40):
+        M = int(rng.choice([1, 1, rng.integers(2, 20), rng.integers(20, 300), rng.choice([64, 128, 256, 320, 512])]))
+        K = int(rng.choice([rng.integers(1, 100), 8 * rng.integers(1, 200), 64 * rng.integers(1, 40), rng.choice([768, 1024, 2048])]))
+        N = int(rng.choice([rng.integers(1, 100), 8 * rng.integers(1, 150), rng.choice([256, 512, 768, 1024])]))
+        print("fc random", it, M, K, N, flush=True)
+        xq, sI, W, sW, bias = make_case(oracle, M, K, N, 7919 * it + 3)
+        if M == 1:
+            blob, _ = host.mvm_transform_weight(W, DF_NORMAL, N, K)
+            fdf = DF_NKN32K4
+        else:
+            blob, _, _ = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+            fdf = DF_NKNxKx
+        dx, dblob, dbias = put(xq), put(blob), put(bias)
+        for b, db in ((bias, dbias), (None, None)):
+            out, so = host.fully_connected(dx, sI, dblob, fdf, sW, db, M, K, N, DT_F32)
+            want, wso = oracle.fully_connected(xq, sI, W, sW, b, DT_F32)
+            assert so == wso and np.array_equal(get(out).view(np.int32), want.view(np.int32)), (M, K, N, "f32")
+            out, so = host.fully_connected(dx, sI, dblob, fdf, sW, db, M, K, N, DT_I32)
+            want, _ = oracle.fully_connected(xq, sI, W, sW, b, DT_I32)
+            assert np.array_equal(get(out), want), (M, K, N, "i32")
+            out, so = host.fully_connected(dx, sI, dblob, fdf, sW, db, M, K, N, DT_U8_Q, -1.0)
+            want, wso = oracle.fully_connected(xq, sI, W, sW, b, DT_U8_Q, -1.0)
+            assert so == wso and np.array_equal(get(out), want), (M, K, N, "u8 dynamic")
+            out, _ = host.fully_connected(dx, sI, dblob, fdf, sW, db, M, K, N, DT_U8_Q, float(wso))
+            want, _ = oracle.fully_connected(xq, sI, W, sW, b, DT_U8_Q, float(wso))
+            assert np.array_equal(get(out), want), (M, K, N, "u8 static")
