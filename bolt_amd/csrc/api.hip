@@ -1304,11 +1304,30 @@ EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDe
 }
 
 // ---- int8 FullyConnected (x86 branch of compute/tensor/src/fully_connected.cpp:372-495) ------------
-static void fc_dims(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, U32 *M, U32 *K, U32 *N)
+// element count of a desc in 64 bits (the reference's tensorNumElements multiplies in 32 bits and wraps)
+static uint64_t elements64(TensorDesc d)
 {
-    *N = outputDesc.dims[0];                                     // fw, fully_connected.cpp:370
-    *K = (*N) ? tensorNumElements(filterDesc) / (*N) : 0;        // fh
-    *M = (*K) ? tensorNumElements(inputDesc) / (*K) : 0;
+    if (d.nDims == 0) {
+        return 0;
+    }
+    uint64_t r = 1;
+    for (U32 i = 0; i < d.nDims && i < DIM_LEN; i++) {
+        r *= d.dims[i];
+    }
+    return r;
+}
+
+// false: a tensor of 2^32 elements or more, which the interface's 32-bit sizes cannot describe
+static bool fc_dims(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, U32 *M, U32 *K, U32 *N)
+{
+    const uint64_t in = elements64(inputDesc), fl = elements64(filterDesc), out = elements64(outputDesc);
+    if (in > 0xffffffffull || fl > 0xffffffffull || out > 0xffffffffull) {
+        return false;
+    }
+    *N = outputDesc.dims[0];                       // fw, fully_connected.cpp:370
+    *K = (*N) ? (U32)(fl / (*N)) : 0;              // fh
+    *M = (*K) ? (U32)(in / (*K)) : 0;
+    return true;
 }
 
 EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc,
@@ -1324,7 +1343,9 @@ EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDe
         return NOT_MATCH;
     }
     U32 M, K, N;
-    fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N);
+    if (!fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N)) {
+        return NOT_SUPPORTED;
+    }
     EE e;
     if (M != 1) {
         e = matrix_matrix_multiply_tmp_bytes_gfx950(tensor2df(inputDesc.dt, DF_NORMAL, M, K), filterDesc, bytes, arch);
@@ -1335,11 +1356,18 @@ EE fully_connected_infer_forward_tmp_bytes_gfx950(TensorDesc inputDesc, TensorDe
         return e;
     }
     if (filterDesc.dt == DT_I8) {  // fully_connected.cpp:149-156
+        // the reference sums these in 32 bits and wraps; a tmp that size would be overrun, so a shape whose tmp does
+        // not fit the interface's 32-bit byte count is refused
+        uint64_t total = *bytes;
         if (inputDesc.dt != DT_I8) {
-            *bytes += tensorNumBytes(inputDesc);
+            total += (uint64_t)M * K * bytesOf(inputDesc.dt);
         }
-        *bytes += N * 4;
-        *bytes += tensorNumElements(outputDesc) * 4;
+        total += (uint64_t)N * 4;
+        total += (uint64_t)M * N * 4;
+        if (total > 0xffffffffull) {
+            return NOT_SUPPORTED;
+        }
+        *bytes = (U32)total;
     }
     return SUCCESS;
 }
@@ -1459,7 +1487,9 @@ EE fully_connected_gfx950(TensorDesc inputDesc, const void *input, F32 inputScal
         return NOT_SUPPORTED;
     }
     U32 M, K, N;
-    fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N);
+    if (!fc_dims(inputDesc, filterDesc, outputDesc, &M, &K, &N)) {
+        return NOT_SUPPORTED;
+    }
     if (M == 0 || N == 0 || K == 0) {
         return NOT_MATCH;
     }

@@ -30,6 +30,12 @@ EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w)
     *h = d.dims[1];
     *c = d.dims[2];
     *n = d.dims[3];
+    // every 4-D operator sizes its buffers and addresses its elements in 32 bits, as the reference's interface does
+    // (tensorNumElements, U32 byte counts): a tensor of 2^32 elements or more is refused rather than wrapped
+    if ((uint64_t)d.dims[0] * d.dims[1] >= (1ull << 32) || (uint64_t)d.dims[0] * d.dims[1] * d.dims[2] >= (1ull << 32) ||
+        (uint64_t)d.dims[0] * d.dims[1] * d.dims[2] * d.dims[3] >= (1ull << 32)) {
+        return NOT_SUPPORTED;
+    }
     return SUCCESS;
 }
 
@@ -37,8 +43,12 @@ EE conv_shape(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc
     ConvShape *s)
 {
     U32 on, fc;
-    if (get4d(inputDesc, &s->n, &s->ic, &s->ih, &s->iw) != SUCCESS || get4d(filterDesc, &s->oc, &fc, &s->fh, &s->fw) != SUCCESS ||
-        get4d(outputDesc, &on, &s->oc, &s->oh, &s->ow) != SUCCESS) {
+    const EE ei = get4d(inputDesc, &s->n, &s->ic, &s->ih, &s->iw), ef = get4d(filterDesc, &s->oc, &fc, &s->fh, &s->fw);
+    const EE eo = get4d(outputDesc, &on, &s->oc, &s->oh, &s->ow);
+    if (ei == NOT_SUPPORTED || ef == NOT_SUPPORTED || eo == NOT_SUPPORTED) {
+        return NOT_SUPPORTED;  // a tensor too large for 32-bit sizes
+    }
+    if (ei != SUCCESS || ef != SUCCESS || eo != SUCCESS) {
         return NOT_MATCH;
     }
     if (p.group != 1) {
@@ -67,6 +77,11 @@ EE conv_shape(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc
     const U32 eh = (s->fh - 1) * s->dh + 1, ew = (s->fw - 1) * s->dw + 1;
     if (s->Hp < eh || s->Wp < ew || (s->Hp - eh) / s->sh + 1 < s->oh || (s->Wp - ew) / s->sw + 1 < s->ow) {
         return NOT_MATCH;  // the output must fit the padded input (every gather stays inside it)
+    }
+    // the kernels address the image (the caller's, and the padded copy in tmp) with 32-bit byte offsets; the reference's
+    // own tmp-bytes interface is 32-bit as well
+    if ((uint64_t)s->n * s->ic * s->ih * s->iw >= (1ull << 32) || (uint64_t)s->n * s->Hp * s->Wp * s->ICp >= (1ull << 32)) {
+        return NOT_SUPPORTED;
     }
     return SUCCESS;
 }

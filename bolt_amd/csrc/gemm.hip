@@ -77,8 +77,8 @@ __global__ __launch_bounds__(256, 2) void gemm_u8s8_general_kernel(GemmArgs a)
 {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t i = lane & 15, g = lane >> 4;
-    const uint32_t m0 = blockIdx.y * 64 + wave * 16;
-    const uint32_t n0 = blockIdx.x * 64;
+    const uint32_t m0 = blockIdx.x * 64 + wave * 16;  // rows along x: a grid's x extent has room for any row count
+    const uint32_t n0 = blockIdx.y * 64;
     if (m0 >= a.M) {
         return;
     }
@@ -2632,8 +2632,11 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     if (a.M == 0 || a.N == 0) {
         return hipSuccess;
     }
+    // the tiled kernels address both operands with 32-bit byte offsets from a 64-bit base: operands of 4 GiB and more go
+    // to the general kernel, which indexes with 64 bits
+    const bool fits32 = (uint64_t)a.M * a.lda < (1ull << 32) && (uint64_t)align_up(a.N, 16) * align_up(a.K, 8) < (1ull << 32);
     const bool tiled_ok = !a.transA && (a.K % 16 == 0) && (a.lda % 16 == 0) && (((uintptr_t)a.A & 15) == 0) &&
-        (((uintptr_t)a.Bp & 15) == 0) && a.K >= 64;
+        (((uintptr_t)a.Bp & 15) == 0) && a.K >= 64 && fits32;
     int tile = 0;
     if (tiled_ok) {
         const uint64_t b256 = (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
@@ -2678,6 +2681,9 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
     const bool dma_ok = tiled_ok && (a.K % 64 == 0);
     if (tile >= 3 && !dma_ok) {
         tile = tiled_ok ? 2 : 0;
+    }
+    if (tile == 2 && (a.M + 127) / 128 > 65535u) {
+        tile = 0;  // the register-staged kernel counts its row tiles along the grid's y extent
     }
     if (tile == 13 && a.K % 128 != 0) {
         tile = 11;
@@ -2750,7 +2756,10 @@ hipError_t launch_gemm_u8s8(const GemmArgs &a, hipStream_t st)
         hipLaunchKernelGGL(gemm_u8s8_skinny_kernel, dim3((a.N + 15) / 16, (a.M + 63) / 64), dim3(512), 0, st, a);
         return hipGetLastError();
     }
-    dim3 grid((a.N + 63) / 64, (a.M + 63) / 64);
+    if ((a.N + 63) / 64 > 65535u) {
+        return hipErrorInvalidValue;  // more than 4 M columns: beyond a grid's y extent
+    }
+    dim3 grid((a.M + 63) / 64, (a.N + 63) / 64);
     hipLaunchKernelGGL(gemm_u8s8_general_kernel, grid, dim3(256), 0, st, a);
     return hipGetLastError();
 }

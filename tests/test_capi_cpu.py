@@ -150,6 +150,30 @@ def test_error_codes_follow_the_reference():
                              AMD_GFX950) == capi.NOT_SUPPORTED
 
 
+def test_sizes_beyond_32_bits_are_refused_not_wrapped():
+    """The reference's tmp sizes are 32-bit byte counts and its sums wrap silently; a tmp of a wrapped size would be
+    overrun. Shapes whose tmp (FullyConnected: input copy + bias + an int32 result) or whose image (convolution: the
+    kernels address it with 32-bit byte offsets) does not fit 32 bits are refused before anything is launched."""
+    from bolt_amd.capi import DF_NCHWC8, DF_NCHWC16, DT_I8, tensor4df
+    L = capi.lib()
+    nb = C.c_uint32(0)
+    M, K, N = (1 << 26) + 64, 64, 16                      # an int32 result of 4 GiB and a bit
+    idesc, fdesc = tensor2df(DT_U8_Q, DF_NORMAL, M, K), tensor2df(DT_I8, DF_NKNxKx, K, N)
+    assert L.fully_connected_infer_forward_tmp_bytes_gfx950(idesc, fdesc, tensor2df(DT_U8_Q, DF_NORMAL, M, N), C.byref(nb),
+                                                            AMD_GFX950) == capi.NOT_SUPPORTED
+    M = 1 << 20                                           # the same query at a size that fits
+    idesc = tensor2df(DT_U8_Q, DF_NORMAL, M, K)
+    assert L.fully_connected_infer_forward_tmp_bytes_gfx950(idesc, fdesc, tensor2df(DT_U8_Q, DF_NORMAL, M, N), C.byref(nb),
+                                                            AMD_GFX950) == capi.SUCCESS
+    assert nb.value >= M * K + 4 * N + 4 * M * N
+    p = capi.conv_param_spec(64, 3, 3, 1, 1)
+    big = tensor4df(DT_U8_Q, DF_NCHWC8, 64, 64, 1024, 1024)          # 4 GiB of input
+    assert L.convolution_infer_forward_tmp_bytes_gfx950(big, tensor4df(DT_I8, capi.DF_NCHWC2NxC4, 64, 64, 3, 3),
+                                                        tensor4df(DT_U8_Q, DF_NCHWC16, 64, 64, 1024, 1024), p,
+                                                        capi.CONVOLUTION_ALGORITHM_DIRECT, C.byref(nb), AMD_GFX950) \
+        == capi.NOT_SUPPORTED
+
+
 def test_pool_concat_lstm_argument_checks_and_size_queries():
     """Shape validation and size queries of the pooling / concatenation / LSTM-cell entry points answer before
     anything touches a GPU."""

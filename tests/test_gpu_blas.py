@@ -541,3 +541,38 @@ def test_mvm_strided_batch_arguments(torch_mod):
     assert L.bolt_gfx950_mvm_int8_strided_batch(2, 16, 16, p, 16, 2, p, q, q, q, None) == capi.NOT_MATCH   # stride < blob
     assert L.bolt_gfx950_mvm_int8_strided_batch(2, 16, 16, p, 322, 2, p, q, q, q, None) == capi.NOT_MATCH  # stride % 4
     assert L.bolt_gfx950_mvm_int8_strided_batch(0, 16, 16, p, 0, 1, p, q, q, q, None) == capi.SUCCESS
+
+
+def test_mmm_operand_of_four_gib_and_more(torch_mod):
+    """A left-hand side of 4 GiB + 4 KiB (2^26 + 64 rows of 64 bytes): beyond what the tiled kernels address with their
+    32-bit byte offsets, so the launcher must send it to the kernel that indexes with 64 bits -- through
+    matrix_matrix_multiply with int32 and fp32 results, every row checked against an fp32 product of
+    the same small integers (exact: every sum is below 2^24) taken in chunks."""
+    torch = torch_mod
+    M, K, N = (1 << 26) + 64, 64, 16
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77)
+    A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+    W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+    off = blob[rhs:rhs + 4 * N].clone()
+    Ci = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    print("mmm 4 GiB operand", M, K, N, flush=True)
+    capi.check(host.matrix_matrix_multiply(A, tensor2df(DT_U8_Q, DF_NORMAL, M, K), blob, bd, off, Ci,
+                                           tensor2df(DT_I32, DF_NORMAL, M, N), None), "mmm i32")
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    Wf = W.to(torch.float32).t().contiguous()
+    step = 1 << 22
+    for lo in range(0, M, step):
+        hi = min(M, lo + step)
+        want = (A[lo:hi].to(torch.float32) - 128.0) @ Wf
+        assert torch.equal(Ci[lo:hi], want.to(torch.int32)), (lo, hi)
+    # an fp32 result of the same product (C += A.B on zeros, cvt(acc) * (1 / scale)) at the far end of the operand
+    tail = slice(M - 4096, M)
+    Cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    capi.check(host.matrix_matrix_multiply(A, tensor2df(DT_U8_Q, DF_NORMAL, M, K), blob, bd, off, Cf,
+                                           tensor2df(DT_F32, DF_NORMAL, M, N), [8.0]), "mmm f32")
+    capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+    assert torch.equal(Cf[tail], Ci[tail].to(torch.float32) * (torch.tensor(1.0, device="cuda") / 8.0))
+    del A, Ci, Cf
+    torch.cuda.empty_cache()
