@@ -250,6 +250,31 @@ EE get1d(TensorDesc d, DataType *dt, U32 *len)
     return SUCCESS;
 }
 
+// element count of a desc in 64 bits (the reference's tensorNumElements multiplies in 32 bits and wraps)
+uint64_t elements64(TensorDesc d)
+{
+    if (d.nDims == 0) {
+        return 0;
+    }
+    uint64_t r = 1;
+    for (U32 i = 0; i < d.nDims && i < DIM_LEN; i++) {
+        r *= d.dims[i];
+    }
+    return r;
+}
+
+// Element count for the element-wise operators, whose kernels walk a tensor with 32-bit indices in grid strides: false
+// for more than kMaxElementwise elements (a stride added to an index that close to 2^32 would wrap).
+bool elementwise_count(TensorDesc d, U32 *n)
+{
+    const uint64_t e = elements64(d);
+    if (e > kMaxElementwise) {
+        return false;
+    }
+    *n = (U32)e;
+    return true;
+}
+
 uint32_t f32_bits(float f)
 {
     uint32_t u;
@@ -1056,7 +1081,10 @@ EE quantize_gfx950(TensorDesc dDesc, const void *data, TensorDesc *qDesc, void *
     if (needs_scale && scale == nullptr) {
         return NOT_MATCH;  // avx512/quantize.cpp:123-125
     }
-    const U32 n = tensorNumElements(dDesc);
+    U32 n;
+    if (!elementwise_count(dDesc, &n)) {
+        return NOT_SUPPORTED;
+    }
     if (n != 0 && (!data || !qData)) {
         return NULL_POINTER;
     }
@@ -1157,7 +1185,10 @@ EE dequantize_gfx950(TensorDesc qDesc, void *qData, const F32 *scale, TensorDesc
     if (!scale) {
         return NULL_POINTER;
     }
-    const U32 n = tensorNumElements(dDesc);
+    U32 n;
+    if (!elementwise_count(dDesc, &n)) {
+        return NOT_SUPPORTED;
+    }
     if (n == 0) {
         return SUCCESS;
     }
@@ -1267,7 +1298,10 @@ EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDe
     if (!IS_GFX950(arch)) {
         return NOT_SUPPORTED;
     }
-    const U32 n = tensorNumElements(outputDesc);
+    U32 n;
+    if (!elementwise_count(outputDesc, &n)) {
+        return NOT_SUPPORTED;
+    }
     if (n == 0) {
         return SUCCESS;
     }
@@ -1304,19 +1338,6 @@ EE requantize_gfx950(TensorDesc inputDesc, INT8 *input, F32 inputScale, TensorDe
 }
 
 // ---- int8 FullyConnected (x86 branch of compute/tensor/src/fully_connected.cpp:372-495) ------------
-// element count of a desc in 64 bits (the reference's tensorNumElements multiplies in 32 bits and wraps)
-static uint64_t elements64(TensorDesc d)
-{
-    if (d.nDims == 0) {
-        return 0;
-    }
-    uint64_t r = 1;
-    for (U32 i = 0; i < d.nDims && i < DIM_LEN; i++) {
-        r *= d.dims[i];
-    }
-    return r;
-}
-
 // false: a tensor of 2^32 elements or more, which the interface's 32-bit sizes cannot describe
 static bool fc_dims(TensorDesc inputDesc, TensorDesc filterDesc, TensorDesc outputDesc, U32 *M, U32 *K, U32 *N)
 {
@@ -1549,6 +1570,9 @@ EE bolt_gfx950_quantize_f32_async(const float *data, U32 n, DataType qdt, void *
     }
     if (!data || !q || !dscale) {
         return NULL_POINTER;
+    }
+    if (n > kMaxElementwise) {
+        return NOT_SUPPORTED;
     }
     EE e = ensure_init();
     if (e != SUCCESS) {

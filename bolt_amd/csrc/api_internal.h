@@ -102,6 +102,9 @@ extern int g_bnn_mfma, g_conv_direct, g_conv_onepass, g_lstm_gemm_rows, g_quanti
 EE get2d(TensorDesc d, DataType *dt, DataFormat *df, U32 *rows, U32 *cols);
 EE get1d(TensorDesc d, DataType *dt, U32 *len);
 EE get4d(TensorDesc d, U32 *n, U32 *c, U32 *h, U32 *w);
+uint64_t elements64(TensorDesc d);  // element count in 64 bits (tensorNumElements multiplies in 32 bits and wraps)
+constexpr uint64_t kMaxElementwise = 0xf0000000ull;  // element-wise kernels index in 32 bits with grid strides
+bool elementwise_count(TensorDesc d, U32 *n);        // false beyond kMaxElementwise
 uint32_t f32_bits(float f);
 bool aligned4(const void *p);
 bg::Epilogue epi_from_scale(const F32 *scale);

@@ -166,6 +166,15 @@ def test_sizes_beyond_32_bits_are_refused_not_wrapped():
     assert L.fully_connected_infer_forward_tmp_bytes_gfx950(idesc, fdesc, tensor2df(DT_U8_Q, DF_NORMAL, M, N), C.byref(nb),
                                                             AMD_GFX950) == capi.SUCCESS
     assert nb.value >= M * K + 4 * N + 4 * M * N
+    # element-wise operators walk a tensor with 32-bit indices in grid strides: counts near 2^32 (and descs whose 32-bit
+    # product wraps to something small) are refused before any pointer is looked at
+    f = np.zeros(8, np.float32)
+    x = np.zeros(8, np.uint8)
+    qd = tensor1d(DT_U8_Q, 8)
+    s1 = (C.c_float * 2)(-1, 0)
+    for huge in (tensor1d(capi.DT_F32, 0xfffffff0), tensor4df(capi.DT_F32, capi.DF_NCHW, 65536, 65536, 1, 2)):
+        assert L.quantize_gfx950(huge, host.ptr(f), C.byref(qd), host.ptr(x), C.cast(s1, C.c_void_p), 0, AMD_GFX950) == \
+            capi.NOT_SUPPORTED
     p = capi.conv_param_spec(64, 3, 3, 1, 1)
     big = tensor4df(DT_U8_Q, DF_NCHWC8, 64, 64, 1024, 1024)          # 4 GiB of input
     assert L.convolution_infer_forward_tmp_bytes_gfx950(big, tensor4df(DT_I8, capi.DF_NCHWC2NxC4, 64, 64, 3, 3),

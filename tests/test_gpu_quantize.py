@@ -305,3 +305,41 @@ def test_one_launch_quantiser_falls_back_when_its_wait_gives_up(torch_mod, oracl
     final = C.c_ulonglong(0)
     capi.check(L.bolt_gfx950_get_counter(b"quantize_fused_fallbacks", C.byref(final)), "counter")
     assert final.value == after.value
+
+
+def test_quantize_beyond_two_to_the_31_elements(torch_mod):
+    """2^31 + 12 345 fp32 values (8.6 GB): element indices above 2^31 and byte offsets above 2^33. The tensor-wide dynamic
+    scale must be 127 / max|x| with the maximum placed near the far end, and the bytes must equal those of chunk-wise
+    calls with that scale given (static mode), which run at sizes the other tests hold against the CPU checker; the
+    dequantised tensor is within half a step everywhere."""
+    torch = torch_mod
+    n = (1 << 31) + 12345
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.empty(n, dtype=torch.float32, device="cuda")
+    step = 1 << 28
+    for lo in range(0, n, step):
+        x[lo:lo + step].normal_(generator=g)
+    x[n - 7] = 9.5                       # the maximum sits where only 64-bit addressing reaches
+    print("quantize", n, "elements", flush=True)
+    for qdt in (DT_U8_Q, DT_I8):
+        s = [-1.0]
+        q = host.quantize(x, DT_F32, qdt, s)
+        capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+        assert s[0] == np.float32(127.0) / np.float32(9.5), s
+        for lo in (0, (1 << 31) - (1 << 20), n - (1 << 24) - 5):          # head, across 2^31, the ragged tail
+            hi = min(n, lo + (1 << 24) + 5)
+            sc = [float(s[0])]
+            part = host.quantize(x[lo:hi].clone(), DT_F32, qdt, sc, 1)
+            capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+            assert sc[0] == s[0] and torch.equal(part, q[lo:hi]), (qdt, lo)
+        if qdt == DT_U8_Q:
+            back = host.dequantize(q, DT_U8_Q, s[0])
+            capi.check(capi.lib().bolt_gfx950_synchronize(), "sync")
+            worst = 0.0
+            for lo in range(0, n, step):
+                worst = max(worst, float((back[lo:lo + step] - x[lo:lo + step]).abs().max().item()))
+            assert worst <= 0.5 / float(s[0]) * 1.0001, worst
+            del back
+        del q
+    del x
+    torch.cuda.empty_cache()
