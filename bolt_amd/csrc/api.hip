@@ -683,8 +683,13 @@ EE matrix_matrix_multiply_transform_rhs_bytes_gfx950(TensorDesc desc, U32 *bytes
     }
     U32 matrix = 0, total = 0;
     if (df != DF_NKNxKx) {
-        matrix = packed_matrix_bytes(N, K);
-        total = N * 4 + matrix + 64;
+        // a weight whose blob does not fit the interface's 32-bit byte count is refused, not wrapped
+        const uint64_t m64 = (uint64_t)align_up(N, 16) * align_up(K, 8), t64 = (uint64_t)N * 4 + m64 + 64;
+        if (t64 > 0xffffffffull) {
+            return NOT_SUPPORTED;
+        }
+        matrix = (U32)m64;
+        total = (U32)t64;
     }
     if (rhsBytes) {
         *rhsBytes = matrix;
@@ -897,17 +902,21 @@ static EE mvm_bytes(TensorDesc matrixDesc, U32 *bytes)
         return NOT_SUPPORTED;
     }
     // x86/mvm.cpp:23-42
-    *bytes = 0;
+    uint64_t b = 0;
     if (dt == DT_I8) {
-        *bytes += row * 4;
+        b += (uint64_t)row * 4;
     }
     if (dt == DT_U8_Q && col % 32 != 0) {
-        *bytes += 32 * (row + 1);
+        b += 32ull * ((uint64_t)row + 1);
     }
     if (df != matrix_vector_multiply_weight_format_gfx950(dt)) {
-        *bytes += align_up(row, 16) * align_up(col, 8);
-        *bytes += 32;
+        b += (uint64_t)align_up(row, 16) * align_up(col, 8);
+        b += 32;
     }
+    if (b > 0xffffffffull) {
+        return NOT_SUPPORTED;  // does not fit the interface's 32-bit byte count
+    }
+    *bytes = (U32)b;
     return SUCCESS;
 }
 

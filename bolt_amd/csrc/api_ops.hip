@@ -562,7 +562,7 @@ EE rnn_transform_filter_bytes_gfx950(TensorDesc filterDesc, RNNParamSpec p, U32 
         *bytes = 0;   // already transformed
         return SUCCESS;
     }
-    const size_t b = 2 * (size_t)packed_matrix_bytes(N, K) + (size_t)N * 4;
+    const size_t b = 2 * ((size_t)align_up(N, 16) * align_up(K, 8)) + (size_t)N * 4;  // 64-bit: a 32-bit product would wrap
     if (b > 0xffffffffull) {
         return NOT_SUPPORTED;
     }

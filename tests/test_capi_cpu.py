@@ -166,6 +166,11 @@ def test_sizes_beyond_32_bits_are_refused_not_wrapped():
     assert L.fully_connected_infer_forward_tmp_bytes_gfx950(idesc, fdesc, tensor2df(DT_U8_Q, DF_NORMAL, M, N), C.byref(nb),
                                                             AMD_GFX950) == capi.SUCCESS
     assert nb.value >= M * K + 4 * N + 4 * M * N
+    # weight blobs of 4 GiB and more do not fit the 32-bit byte counts of the transform queries
+    rb = C.c_uint32(0)
+    wide = tensor2df(DT_I8, DF_NORMAL, 65536, 65536)
+    assert L.matrix_matrix_multiply_transform_rhs_bytes_gfx950(wide, C.byref(nb), C.byref(rb), AMD_GFX950) == capi.NOT_SUPPORTED
+    assert L.matrix_vector_multiply_transform_weight_bytes_gfx950(wide, C.byref(nb), AMD_GFX950) == capi.NOT_SUPPORTED
     # element-wise operators walk a tensor with 32-bit indices in grid strides: counts near 2^32 (and descs whose 32-bit
     # product wraps to something small) are refused before any pointer is looked at
     f = np.zeros(8, np.float32)
