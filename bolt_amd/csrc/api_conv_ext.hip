@@ -9,9 +9,11 @@
 //    every layer; here the input scale is read from, and the output scale left in, device memory.
 //
 // Both run the kernels of convolution_gfx950 (gemm.hip: conv_u8s8_panel_kernel, gemm_u8s8_dma_kernel<..., CONV>); what
-// differs is the epilogue (EPI_CONV_CH) and where the scales live. A dynamic u8 result takes two passes of the
-// convolution -- the first only folds the tensor-wide maximum into scratch slots, the second stores -- so that no
-// launch depends on all of its workgroups being resident at once and nothing ever waits for the host.
+// differs is the epilogue (EPI_CONV_CH) and where the scales live. A dynamic u8 result runs in ONE pass of the filter-
+// panel kernel where all its workgroups are resident at once (they agree on the tensor-wide maximum with their values
+// in registers; if that agreement is abandoned the synchronous forms redo the call in two passes from the host, and the
+// asynchronous form -- given a tmp with spill room -- finishes on the device), and otherwise in two passes: the first
+// only folds the maximum into scratch slots, the second stores. Nothing in the asynchronous form waits for the host.
 #include "api_internal.h"
 
 using namespace bg;
