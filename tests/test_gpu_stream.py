@@ -55,3 +55,58 @@ def test_calls_follow_the_callers_stream(oracle):
                                            tensor2df(DT_I32, DF_NORMAL, M, N), None), "mmm")
     capi.check(L.bolt_gfx950_synchronize(), "sync")
     assert torch.equal(Cd, Cd2)
+
+
+def test_grid_wide_agreements_while_another_stream_holds_the_cus():
+    """The one-pass u8 convolution and the one-launch quantiser keep values in registers while all workgroups of a
+    launch agree on a maximum, which needs the whole grid resident. Here another stream keeps every CU busy with large
+    bf16 products the whole time (a serving process sharing the device): the calls must return the bytes and scales
+    they return on an idle device, whether their agreement completes once the other stream's workgroups drain or is
+    abandoned after its bounded wait and redone in two passes."""
+    import time
+
+    import torch
+    from bolt_amd import host_conv
+    from bolt_amd.capi import DF_NCHWC8, DF_NCHWC16
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_init(), "init")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    n, ic, ih, iw, oc = 32, 64, 56, 56, 64
+    xq = torch.randint(128, 256, (n * ic * ih * iw,), dtype=torch.uint8, device="cuda", generator=g)
+    Wc = torch.randint(-127, 128, (oc, ic, 3, 3), dtype=torch.int8, device="cuda", generator=g)
+    p = capi.conv_param_spec(oc, 3, 3, 1, 1)
+    cblob, ftm = host_conv.transform_filter(Wc, oc, ic, 3, 3, p)
+    cb = torch.randn(oc, device="cuda", generator=g) * 0.1
+    xf = torch.randn(1 << 18, device="cuda", generator=g)
+
+    def conv():
+        sc = [30.0, -1.0, 80.0]
+        out = host_conv.convolution(xq, DF_NCHWC8, n, ic, ih, iw, cblob, ftm, oc, 3, 3, 1, 1, cb, sc, True, DT_U8_Q, DF_NCHWC16)
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+        return out.clone(), sc[1]
+
+    def quant():
+        s = [-1.0]
+        q = host.quantize(xf, DT_F32, DT_U8_Q, s)
+        capi.check(L.bolt_gfx950_synchronize(), "sync")
+        return q.clone(), s[0]
+    ref_c, ref_cs = conv()
+    ref_q, ref_qs = quant()
+    side = torch.cuda.Stream()          # default priority
+    A = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    B = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    worst = 0.0
+    for it in range(40):
+        with torch.cuda.stream(side):
+            for _ in range(6):
+                A @ B                   # half a millisecond each on every CU
+        t1 = time.time()
+        got_c, got_cs = conv()
+        got_q, got_qs = quant()
+        worst = max(worst, time.time() - t1)
+        assert torch.equal(got_c, ref_c) and got_cs == ref_cs, it
+        assert torch.equal(got_q, ref_q) and got_qs == ref_qs, it
+    side.synchronize()
+    print("worst pair of calls under contention: %.1f ms" % (worst * 1e3), flush=True)
+    assert worst < 5.0                  # seconds: the bounded waits end (2^19 polls each) and nothing hangs
