@@ -110,3 +110,57 @@ def test_grid_wide_agreements_while_another_stream_holds_the_cus():
     side.synchronize()
     print("worst pair of calls under contention: %.1f ms" % (worst * 1e3), flush=True)
     assert worst < 5.0                  # seconds: the bounded waits end (2^19 polls each) and nothing hangs
+
+
+def test_async_entry_points_replay_from_a_captured_graph():
+    """The device-scale forms depend on their arguments only, so a chain of them can be captured in a HIP graph: the
+    dynamic quantiser that leaves its scale on the device (two passes, its slots cleared by a fill kernel, no memset
+    node) feeding the per-channel product that reads that scale from the device. The graph is replayed four times with
+    new activations, eager work and synchronisations in between; every replay must equal the eager chain."""
+    import torch
+    L = capi.lib()
+    capi.check(L.bolt_gfx950_init(), "init")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4)
+    M, K, N = 256, 1024, 768
+    x = torch.randn(M * K, device="cuda", generator=g)
+    W = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    blob, bd, rhs = host.mmm_transform_rhs(W, DF_TRANSPOSE, K, N)
+    off = blob[rhs:rhs + 4 * N].view(torch.int32).clone()
+    sw = torch.rand(N, device="cuda", generator=g) * 150 + 50
+    bias = torch.randn(N, device="cuda", generator=g) * 0.1
+    q = torch.empty(M * K, dtype=torch.uint8, device="cuda")
+    ds = torch.full((1,), -1.0, device="cuda")
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    L.bolt_gfx950_mmm_int8_perchannel.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32] + [C.c_void_p] * 7
+
+    def chain():
+        ds.fill_(-1.0)               # a fill kernel on the current stream (the library's stream below): dynamic scale asked for
+        capi.check(L.bolt_gfx950_quantize_f32_async(x.data_ptr(), M * K, DT_U8_Q, q.data_ptr(), ds.data_ptr(), 0), "quantize")
+        capi.check(L.bolt_gfx950_mmm_int8_perchannel(M, N, K, q.data_ptr(), blob.data_ptr(), off.data_ptr(), out.data_ptr(),
+                                                     ds.data_ptr(), sw.data_ptr(), bias.data_ptr()), "mmm_int8_perchannel")
+    side = torch.cuda.Stream()       # default priority
+    torch.cuda.synchronize()
+    try:
+        capi.check(L.bolt_gfx950_set_stream(C.c_void_p(side.cuda_stream)), "set_stream")
+        with torch.cuda.stream(side):
+            chain()
+            chain()                  # nothing left to initialise inside the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            chain()
+        side.synchronize()
+        for rep in range(4):
+            x.copy_(torch.randn(M * K, device="cuda", generator=g) * (rep + 1))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got, got_scale = out.clone(), ds.clone()
+            with torch.cuda.stream(side):
+                chain()
+            side.synchronize()
+            print("graph replay", rep, float(got_scale.item()), flush=True)
+            assert torch.equal(got_scale, ds) and torch.equal(got, out), rep
+    finally:
+        capi.check(L.bolt_gfx950_set_stream(None), "set_stream")
